@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Benchmark of the routed-expert layer (pack -> grouped SwiGLU FFN -> combine).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c1|c2]
+
+One "step" is one ek_layer_forward over one synthetic batch whose inputs and
+weights are already resident in HBM.  Prints ONE JSON line: whole-job
+token-expert pairs/s, the roofline of the dominant kernel (per-phase HIP events
+recorded on the launch stream inside the timed region) and, beside it, the
+reference-equivalent CPU backend timed on this box's host cores on a bounded
+sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "expert-kit_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK = 8.0e12        # B/s, MI355X HBM3E
+MFMA_PEAK_16 = 2.5e15    # FLOP/s, bf16/fp16 dense
+
+
+def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
+    """Reference-equivalent CPU backend (libtorch ops of ffn/expert_torch.rs:81-84,
+    grouped per expert, weighted sum of qwen3_moe.py:102-104) on the pairs routed to
+    a sample of experts; weights pre-cast to the compute dtype as load_module does."""
+    import torch
+    from oracle import oracle
+    E = w.n_experts
+    wu, wg, wd = [None] * E, [None] * E, [None] * E
+    for e, ew in ws_sample.items():
+        if w.w8:
+            wu[e] = oracle.torch_dequant_channel(ew.up_w, ew.up_scale)
+            wg[e] = oracle.torch_dequant_channel(ew.gate_w, ew.gate_scale)
+            wd[e] = oracle.torch_dequant_channel(ew.down_w, ew.down_scale)
+        else:
+            wu[e], wg[e], wd[e] = ew.up_w.cpu(), ew.gate_w.cpu(), ew.down_w.cpu()
+    sample = set(ws_sample)
+    times, pairs = [], 0
+    t_all = time.time()
+    while len(times) < 5 and (time.time() - t_all < target_s or not times):
+        t0 = time.time()
+        _, pairs = oracle.torch_layer_forward(x, ids, gw, wu, wg, wd, experts=sample)
+        times.append(time.time() - t0)
+    med = sorted(times)[len(times) // 2]
+    return pairs / med, pairs, len(times)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import ek_hip
+    from ek_hip import workloads as wl
+
+    ek_hip.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    w = wl.resolve(wl.CONFIGS[args.workload])
+    layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype,
+                            w_dtype=torch.int8 if w.w8 else w.act_dtype, max_tokens=w.tokens)
+    ids, gw = wl.make_routing(w)
+    counts = torch.bincount(ids.reshape(-1).long(), minlength=w.n_experts)
+    order = torch.argsort(counts, descending=True, stable=True).tolist()
+    sample_ids = sorted(order[:: max(1, w.n_experts // max(args.cpu_experts, 1))][: args.cpu_experts]) if args.cpu_experts else []
+    ws_sample = {}
+    for e in range(w.n_experts):
+        ew = wl.make_expert(w, e, device="cuda")
+        layer.set_expert(e, ew)
+        if e in sample_ids:
+            ws_sample[e] = ek_hip.ExpertWeight(*[None if t is None else t.cpu() for t in
+                                                 (ew.up_w, ew.gate_w, ew.down_w, ew.up_scale, ew.gate_scale, ew.down_scale)])
+        del ew
+    x = wl.make_x(w)
+    xd, idd, gwd = x.to(dev), ids.to(dev), gw.to(dev)
+    y = torch.empty_like(xd)
+    stream = torch.cuda.current_stream()
+
+    # parity gate on this very input: routing tables vs a CPU stable sort
+    _, rt = layer.forward(xd, idd, gwd, return_route=True)
+    ref_perm = torch.argsort(ids.reshape(-1).long(), stable=True).to(torch.int32)
+    assert torch.equal(rt.perm.cpu(), ref_perm), "routing permutation mismatch"
+
+    for _ in range(args.warmup):
+        layer.forward(xd, idd, gwd, stream=stream, out=y)
+    torch.cuda.synchronize()
+    layer.profile(True)
+    t0 = time.perf_counter()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record(stream)
+    for _ in range(args.steps):
+        layer.forward(xd, idd, gwd, stream=stream, out=y)
+    ev1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_s = ev0.elapsed_time(ev1) * 1e-3
+    st = layer.stats()
+    layer.profile(False)
+    step_s = max(wall, dev_s) / args.steps
+    value = w.pairs / step_s
+
+    n_prof = max(st["profiled_calls"], 1)
+    k_us = [v / n_prof for v in st["kernel_us"]]
+    active = int((counts > 0).sum())
+    wsz = 1 if w.w8 else 2
+    a = 2
+    # algorithmic bytes of each phase (weights of active experts once, activations in/out once)
+    b_ffn1 = active * (2 * w.hidden * w.inter * wsz + (2 * w.inter * 2 if w.w8 else 0)) + w.tokens * w.hidden * a + w.pairs * w.inter * a
+    b_ffn2 = active * (w.hidden * w.inter * wsz + (w.hidden * 2 if w.w8 else 0)) + w.pairs * w.inter * a + w.pairs * w.hidden * a
+    b_layer = wl.algorithmic_bytes(w, counts)
+    f_layer = w.pairs * w.flops_per_pair()
+    hbm_frac = b_layer / step_s / HBM_PEAK
+    mfma_frac = f_layer / step_s / MFMA_PEAK_16
+    dom = 1 if k_us[1] >= k_us[2] else 2
+    dom_name = "ffn_stream_kernel(stage 1: up/gate + SwiGLU)" if dom == 1 else "ffn_stream_kernel(stage 2: down)"
+    dom_bytes = b_ffn1 if dom == 1 else b_ffn2
+    dom_flops = w.pairs * (4 if dom == 1 else 2) * w.hidden * w.inter
+    dom_s = k_us[dom] * 1e-6
+    if hbm_frac >= mfma_frac:
+        roof = {"bound": "hbm", "achieved": dom_bytes / dom_s / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                "frac": dom_bytes / dom_s / HBM_PEAK, "traffic": None}
+    else:
+        roof = {"bound": "mfma", "achieved": dom_flops / dom_s / 1e12, "peak": MFMA_PEAK_16 / 1e12, "unit": "TFLOP/s",
+                "frac": dom_flops / dom_s / MFMA_PEAK_16, "traffic": None}
+    roof.update({"kernel": dom_name, "kernel_us": k_us[dom], "algorithmic_bytes": dom_bytes,
+                 "algorithmic_flops": dom_flops})
+
+    out = {
+        "metric": "token-expert pairs/s on 1 MI355X (DSv3 W8A16 layer); % HBM / MFMA roofline",
+        "value": value, "unit": "pairs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": step_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": ("i8 weights x " if w.w8 else "") + str(w.act_dtype).replace("torch.", "") + ", fp32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": w.name, "hidden": w.hidden, "moe_intermediate": w.inter, "experts": w.n_experts,
+                   "top_k": w.top_k, "tokens": w.tokens, "pairs": w.pairs, "active_experts": active,
+                   "zipf_s": w.zipf_s},
+        "roofline": roof,
+        "layer": {"algorithmic_bytes": b_layer, "algorithmic_flops": f_layer, "hbm_frac": hbm_frac,
+                  "mfma_frac": mfma_frac,
+                  "phase_us": {"pack": k_us[0], "ffn_up_gate": k_us[1], "ffn_down": k_us[2], "combine": k_us[3]},
+                  "device_ms_per_step": dev_s / args.steps * 1e3},
+    }
+    if args.cpu_experts:
+        cores = os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"])
+        torch.set_num_threads(cores)
+        v, pairs, iters = cpu_baseline(w, ws_sample, x, ids, gw)
+        out["cpu_baseline"] = {"value": v, "unit": "pairs/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"pairs routed to {len(ws_sample)} of {w.n_experts} experts ({pairs} pairs), "
+                                         f"median of {iters} runs, libtorch CPU ops, weights pre-cast to "
+                                         f"{str(w.act_dtype).replace('torch.', '')}"}
+    layer.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

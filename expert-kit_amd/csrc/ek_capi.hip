@@ -1,0 +1,808 @@
+// C-ABI host layer of libek_hip.so (see include/ek_hip.h for the contract).
+#include "../../include/ek_hip.h"
+#include "ek_internal.h"
+
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_last_error;
+
+ek_status fail(ek_status st, const char *fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return st;
+}
+
+ek_status hip_fail(hipError_t e, const char *what)
+{
+    (void)hipGetLastError();   // clear the sticky error
+    return fail(e == hipErrorOutOfMemory ? EK_OOM : EK_HIP_ERROR, "%s: %s", what,
+                hipGetErrorString(e));
+}
+
+#define EK_HIP(call)                                                  \
+    do {                                                              \
+        hipError_t _e = (call);                                       \
+        if (_e != hipSuccess) return hip_fail(_e, #call);             \
+    } while (0)
+
+#define EK_TRY(call)                                                  \
+    do {                                                              \
+        ek_status _s = (call);                                        \
+        if (_s != EK_OK) return _s;                                   \
+    } while (0)
+
+// Makes `dev` current for the scope and restores the caller's device.
+struct DeviceGuard {
+    int prev = -1;
+    bool ok = false;
+    explicit DeviceGuard(int dev)
+    {
+        if (hipGetDevice(&prev) != hipSuccess) { (void)hipGetLastError(); prev = -1; }
+        ok = hipSetDevice(dev) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+    }
+    ~DeviceGuard()
+    {
+        if (prev >= 0 && ok) (void)hipSetDevice(prev);
+    }
+};
+
+int64_t elem_size(int dt)
+{
+    switch (dt) {
+    case EK_BF16: case EK_F16: return 2;
+    case EK_F32: return 4;
+    case EK_I8: return 1;
+    default: return 0;
+    }
+}
+
+}  // namespace
+
+struct ek_layer {
+    ek_cfg cfg{};
+    int act = 0;        // 0 bf16, 1 f16
+    bool w8 = false;
+    int64_t Pmax = 0;
+    hipStream_t stream = nullptr;
+    std::mutex mu;       // serialises users of the workspace and the slab table
+    std::mutex load_mu;  // serialises weight ingestion
+
+    std::vector<void *> expert_mem;          // one allocation per loaded expert
+    std::vector<ek::ExpertSlab> h_slabs;
+    ek::ExpertSlab *d_slabs = nullptr;
+
+    // workspace
+    int32_t *counts = nullptr, *offsets = nullptr, *perm = nullptr, *inv_perm = nullptr;
+    int32_t *row_token = nullptr, *block_hist = nullptr, *err = nullptr;
+    void *h = nullptr, *yp = nullptr;
+    int32_t *h_err = nullptr;                // pinned
+
+    // staging for host-memory callers (allocated on first use)
+    void *st_x = nullptr, *st_w = nullptr, *st_y = nullptr, *st_xp = nullptr;
+    int32_t *st_ids = nullptr;
+    void *st_raw = nullptr;                  // raw weight bytes during ingestion
+    size_t st_raw_bytes = 0;
+    hipStream_t load_stream = nullptr;
+
+    ek_stats stats{};
+    std::mutex stats_mu;
+
+    // per-phase event timing (ek_layer_profile)
+    bool profiling = false;
+    std::vector<hipEvent_t> events;          // 5 per recorded call
+    size_t events_used = 0;
+};
+
+struct ek_expert {
+    ek_layer *layer = nullptr;
+};
+
+namespace {
+
+ek_status dev_alloc(void **p, size_t bytes, const char *what)
+{
+    hipError_t e = hipMalloc(p, bytes ? bytes : 16);
+    if (e != hipSuccess) {
+        *p = nullptr;
+        (void)hipGetLastError();
+        return fail(e == hipErrorOutOfMemory ? EK_OOM : EK_HIP_ERROR, "hipMalloc(%s, %zu bytes): %s",
+                    what, bytes, hipGetErrorString(e));
+    }
+    return EK_OK;
+}
+
+void free_layer(ek_layer *L)
+{
+    if (!L) return;
+    (void)hipDeviceSynchronize();
+    for (void *p : L->expert_mem) if (p) (void)hipFree(p);
+    void *bufs[] = {L->d_slabs, L->counts, L->offsets, L->perm, L->inv_perm, L->row_token,
+                    L->block_hist, L->err, L->h, L->yp, L->st_x, L->st_w, L->st_y, L->st_xp,
+                    L->st_ids, L->st_raw};
+    for (void *p : bufs) if (p) (void)hipFree(p);
+    for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
+    if (L->h_err) (void)hipHostFree(L->h_err);
+    if (L->stream) (void)hipStreamDestroy(L->stream);
+    if (L->load_stream) (void)hipStreamDestroy(L->load_stream);
+    delete L;
+}
+
+ek_status validate_cfg(const ek_cfg *c)
+{
+    if (!c) return fail(EK_INVALID_INPUT, "cfg is NULL");
+    if (c->act_dtype != EK_BF16 && c->act_dtype != EK_F16)
+        return fail(EK_INVALID_INPUT, "act_dtype must be EK_BF16 or EK_F16 (got %d)", c->act_dtype);
+    if (c->w_dtype != c->act_dtype && c->w_dtype != EK_I8)
+        return fail(EK_INVALID_INPUT, "w_dtype must equal act_dtype or be EK_I8 (got %d)", c->w_dtype);
+    const int64_t ke = c->w_dtype == EK_I8 ? 64 : 32;
+    if (c->hidden <= 0 || c->inter <= 0 || c->hidden % ke || c->inter % ke)
+        return fail(EK_INVALID_INPUT, "hidden (%lld) and inter (%lld) must be positive multiples of %lld",
+                    (long long)c->hidden, (long long)c->inter, (long long)ke);
+    if (c->n_experts < 1 || c->n_experts > ek::kMaxExperts)
+        return fail(EK_INVALID_INPUT, "n_experts must be in [1, %d] (got %d)", ek::kMaxExperts,
+                    c->n_experts);
+    if (c->top_k < 1 || c->top_k > c->n_experts)
+        return fail(EK_INVALID_INPUT, "top_k must be in [1, n_experts] (got %d)", c->top_k);
+    if (c->max_tokens < 1 || c->max_tokens * (int64_t)c->top_k >= (1ll << 31))
+        return fail(EK_INVALID_INPUT, "max_tokens * top_k must be in [1, 2^31) (max_tokens %lld)",
+                    (long long)c->max_tokens);
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess) { (void)hipGetLastError(); ndev = 0; }
+    if (c->device_id < 0 || c->device_id >= ndev)
+        return fail(EK_HIP_ERROR, "device_id %d not available (%d HIP devices visible)", c->device_id,
+                    ndev);
+    return EK_OK;
+}
+
+ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
+{
+    ek_layer *L = new (std::nothrow) ek_layer();
+    if (!L) return fail(EK_OOM, "host allocation failed");
+    L->cfg = *cfg;
+    L->act = cfg->act_dtype == EK_BF16 ? 0 : 1;
+    L->w8 = cfg->w_dtype == EK_I8;
+    L->Pmax = pmax;
+    const int E = cfg->n_experts;
+    L->expert_mem.assign(E, nullptr);
+    L->h_slabs.assign(E, ek::ExpertSlab{nullptr, nullptr, nullptr, nullptr, nullptr});
+    const int64_t nblocks = (pmax + ek::kPackChunk - 1) / ek::kPackChunk;
+    ek_status st = EK_OK;
+    auto A = [&](void **p, size_t bytes, const char *what) {
+        if (st == EK_OK) st = dev_alloc(p, bytes, what);
+    };
+    A((void **)&L->d_slabs, sizeof(ek::ExpertSlab) * E, "slab table");
+    A((void **)&L->counts, sizeof(int32_t) * E, "counts");
+    A((void **)&L->offsets, sizeof(int32_t) * (E + 1), "offsets");
+    A((void **)&L->perm, sizeof(int32_t) * pmax, "perm");
+    A((void **)&L->inv_perm, sizeof(int32_t) * pmax, "inv_perm");
+    A((void **)&L->row_token, sizeof(int32_t) * pmax, "row_token");
+    A((void **)&L->block_hist, sizeof(int32_t) * nblocks * E, "block_hist");
+    A((void **)&L->err, sizeof(int32_t) * 4, "err");
+    A(&L->h, (size_t)pmax * cfg->inter * 2, "h");
+    A(&L->yp, (size_t)pmax * cfg->hidden * 2, "yp");
+    if (st == EK_OK) {
+        hipError_t e = hipMemset(L->d_slabs, 0, sizeof(ek::ExpertSlab) * E);
+        if (e == hipSuccess) e = hipMemset(L->err, 0, sizeof(int32_t) * 4);
+        if (e == hipSuccess) e = hipHostMalloc((void **)&L->h_err, sizeof(int32_t) * 4, hipHostMallocDefault);
+        if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
+        if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->load_stream, hipStreamNonBlocking);
+        if (e != hipSuccess) st = hip_fail(e, "layer setup");
+    }
+    if (st != EK_OK) {
+        std::string keep = g_last_error;
+        free_layer(L);
+        g_last_error = keep;
+        return st;
+    }
+    *out = L;
+    return EK_OK;
+}
+
+ek_status check_desc(const ek_weight_desc *d, const char *name, int64_t rows, int64_t cols, bool w8)
+{
+    if (!d || !d->ptr) return fail(EK_WEIGHT_NOT_FOUND, "%s weight is missing", name);
+    if (d->rows != rows || d->cols != cols)
+        return fail(EK_INVALID_INPUT, "%s weight is [%lld,%lld], expected [%lld,%lld]", name,
+                    (long long)d->rows, (long long)d->cols, (long long)rows, (long long)cols);
+    if (d->mem != EK_HOST && d->mem != EK_DEVICE)
+        return fail(EK_INVALID_INPUT, "%s weight: bad mem %d", name, d->mem);
+    if (w8) {
+        if (d->dtype != EK_I8)
+            return fail(EK_INVALID_INPUT, "%s weight must be EK_I8 for an int8 layer (got %d)", name,
+                        d->dtype);
+        if (d->scale_kind != EK_SCALE_PER_CHANNEL)
+            return fail(EK_INVALID_INPUT, "%s weight: int8 needs EK_SCALE_PER_CHANNEL", name);
+        if (!d->scale) return fail(EK_WEIGHT_NOT_FOUND, "%s scale is missing", name);
+        if (d->scale_dtype != EK_BF16 && d->scale_dtype != EK_F32 && d->scale_dtype != EK_F16)
+            return fail(EK_INVALID_INPUT, "%s scale: bad dtype %d", name, d->scale_dtype);
+    } else {
+        if (d->dtype != EK_BF16 && d->dtype != EK_F16 && d->dtype != EK_F32)
+            return fail(EK_INVALID_INPUT, "%s weight: dtype %d cannot be cast to the layer's 16-bit type",
+                        name, d->dtype);
+        if (d->scale_kind != EK_SCALE_NONE)
+            return fail(EK_INVALID_INPUT, "%s weight: scales are only valid with EK_I8", name);
+    }
+    return EK_OK;
+}
+
+// Brings `bytes` of (host or device) source to a device address usable by the
+// tiling kernels.  Host sources go through the layer's raw staging buffer.
+ek_status stage_raw(ek_layer *L, const void *src, int mem, size_t bytes, size_t stage_off,
+                    const void **dev)
+{
+    if (mem == EK_DEVICE) { *dev = src; return EK_OK; }
+    EK_HIP(hipMemcpyAsync((char *)L->st_raw + stage_off, src, bytes, hipMemcpyHostToDevice,
+                          L->load_stream));
+    *dev = (char *)L->st_raw + stage_off;
+    return EK_OK;
+}
+
+ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
+                            const ek_weight_desc *gate, const ek_weight_desc *down)
+{
+    const int64_t H = L->cfg.hidden, I = L->cfg.inter;
+    EK_TRY(check_desc(up, "up", I, H, L->w8));
+    EK_TRY(check_desc(gate, "gate", I, H, L->w8));
+    EK_TRY(check_desc(down, "down", H, I, L->w8));
+    const size_t wsz = L->w8 ? 1 : 2;
+    const size_t mat_bytes = (size_t)H * I * wsz;
+    const size_t scale_floats = L->w8 ? (size_t)(2 * I + H) : 0;
+    const size_t total = 3 * mat_bytes + scale_floats * sizeof(float);
+
+    // staging for host sources: three raw matrices (+ scales) back to back
+    const ek_weight_desc *ds[3] = {up, gate, down};
+    size_t need = 0;
+    for (auto d : ds) {
+        if (d->mem == EK_HOST) {
+            need += (size_t)d->rows * d->cols * elem_size(d->dtype);
+            need = (need + 255) & ~(size_t)255;
+            if (L->w8) need += ((size_t)d->rows * elem_size(d->scale_dtype) + 255) & ~(size_t)255;
+        }
+    }
+    if (need > L->st_raw_bytes) {
+        EK_HIP(hipStreamSynchronize(L->load_stream));
+        if (L->st_raw) (void)hipFree(L->st_raw);
+        L->st_raw = nullptr; L->st_raw_bytes = 0;
+        EK_TRY(dev_alloc(&L->st_raw, need, "weight staging"));
+        L->st_raw_bytes = need;
+    }
+
+    void *mem = nullptr;
+    EK_TRY(dev_alloc(&mem, total, "expert weights"));
+    uint8_t *base = (uint8_t *)mem;
+    ek::ExpertSlab slab;
+    slab.upgate = base;
+    slab.down = base + 2 * mat_bytes;
+    float *sc = (float *)(base + 3 * mat_bytes);
+    slab.s_up = L->w8 ? sc : nullptr;
+    slab.s_gate = L->w8 ? sc + I : nullptr;
+    slab.s_down = L->w8 ? sc + 2 * I : nullptr;
+
+    ek_status st = EK_OK;
+    size_t off = 0;
+    const int dst_dt = L->w8 ? EK_I8 : L->cfg.act_dtype;
+    float *sdst[3] = {sc, sc + I, sc + 2 * I};
+    uint8_t *wdst[3] = {base, base, base + 2 * mat_bytes};
+    const int mi[3] = {0, 1, 0}, nmat[3] = {2, 2, 1};
+    for (int i = 0; i < 3 && st == EK_OK; ++i) {
+        const ek_weight_desc *d = ds[i];
+        const void *src = nullptr;
+        const size_t bytes = (size_t)d->rows * d->cols * elem_size(d->dtype);
+        st = stage_raw(L, d->ptr, d->mem, bytes, off, &src);
+        if (d->mem == EK_HOST) off = (off + bytes + 255) & ~(size_t)255;
+        if (st != EK_OK) break;
+        ek::launch_tile_weights(src, d->dtype, d->rows, d->cols, wdst[i], dst_dt, mi[i], nmat[i],
+                                L->load_stream);
+        if (L->w8) {
+            const void *ssrc = nullptr;
+            const size_t sbytes = (size_t)d->rows * elem_size(d->scale_dtype);
+            st = stage_raw(L, d->scale, d->mem, sbytes, off, &ssrc);
+            if (d->mem == EK_HOST) off = (off + sbytes + 255) & ~(size_t)255;
+            if (st != EK_OK) break;
+            ek::launch_scales_to_f32(ssrc, d->scale_dtype, d->rows, sdst[i], L->load_stream);
+        }
+    }
+    if (st == EK_OK) {
+        hipError_t e = hipGetLastError();
+        if (e == hipSuccess) e = hipStreamSynchronize(L->load_stream);
+        if (e != hipSuccess) st = hip_fail(e, "weight tiling");
+    }
+    if (st != EK_OK) { (void)hipFree(mem); return st; }
+
+    // publish: swap the slab entry under the forward lock; free any old copy
+    void *old = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(L->mu);
+        old = L->expert_mem[e];
+        if (old) (void)hipDeviceSynchronize();   // drain work that may read the old copy
+        L->expert_mem[e] = mem;
+        L->h_slabs[e] = slab;
+        hipError_t er = hipMemcpy(L->d_slabs + e, &slab, sizeof slab, hipMemcpyHostToDevice);
+        if (er != hipSuccess) return hip_fail(er, "slab table update");
+    }
+    if (old) (void)hipFree(old);
+    return EK_OK;
+}
+
+struct Timer {
+    std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
+    double us() const
+    {
+        return std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+    }
+};
+
+ek_status ensure_io_staging(ek_layer *L)
+{
+    if (L->st_x) return EK_OK;
+    const int64_t T = L->cfg.max_tokens, K = L->cfg.top_k, H = L->cfg.hidden;
+    // st_x / st_y also serve ek_layer_expert_forward, whose n may reach Pmax
+    const int64_t rows = L->Pmax > T ? L->Pmax : T;
+    EK_TRY(dev_alloc(&L->st_x, (size_t)rows * H * 2, "x staging"));
+    EK_TRY(dev_alloc(&L->st_y, (size_t)rows * H * 2, "y staging"));
+    EK_TRY(dev_alloc(&L->st_w, (size_t)T * K * 4, "gate-weight staging"));
+    EK_TRY(dev_alloc((void **)&L->st_ids, (size_t)T * K * 4, "ids staging"));
+    return EK_OK;
+}
+
+ek_status err_to_status(int32_t err)
+{
+    if (err & 1) return fail(EK_INVALID_INPUT, "expert id outside [0, n_experts)");
+    if (err & 2) return fail(EK_EXPERT_NOT_FOUND, "a pair was routed to an expert that is not loaded");
+    return EK_OK;
+}
+
+ek_status copy_route_out(ek_layer *L, const ek_route_out *r, int64_t P, int mem, hipStream_t s)
+{
+    if (!r) return EK_OK;
+    const hipMemcpyKind kind = mem == EK_DEVICE ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost;
+    const int E = L->cfg.n_experts;
+    if (r->counts) EK_HIP(hipMemcpyAsync(r->counts, L->counts, sizeof(int32_t) * E, kind, s));
+    if (r->offsets) EK_HIP(hipMemcpyAsync(r->offsets, L->offsets, sizeof(int32_t) * (E + 1), kind, s));
+    if (P > 0 && r->perm) EK_HIP(hipMemcpyAsync(r->perm, L->perm, sizeof(int32_t) * P, kind, s));
+    if (P > 0 && r->inv_perm) EK_HIP(hipMemcpyAsync(r->inv_perm, L->inv_perm, sizeof(int32_t) * P, kind, s));
+    return EK_OK;
+}
+
+ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_loaded)
+{
+    ek::PackArgs a;
+    a.ids = ids;
+    a.P = P;
+    a.E = L->cfg.n_experts;
+    a.K = L->cfg.top_k;
+    a.nblocks = (int32_t)((P + ek::kPackChunk - 1) / ek::kPackChunk);
+    a.slabs = check_loaded ? L->d_slabs : nullptr;
+    a.block_hist = L->block_hist;
+    a.counts = L->counts;
+    a.offsets = L->offsets;
+    a.perm = L->perm;
+    a.inv_perm = L->inv_perm;
+    a.row_token = L->row_token;
+    a.err = L->err;
+    return a;
+}
+
+// pack -> stage 1 -> stage 2 -> combine on stream s; all pointers are device.
+ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const void *w, int w_f32,
+                          int64_t T, void *y, hipStream_t s)
+{
+    const int64_t H = L->cfg.hidden, I = L->cfg.inter;
+    const int E = L->cfg.n_experts, K = L->cfg.top_k;
+    const int64_t P = T * K;
+    hipEvent_t *ev = nullptr;
+    if (L->profiling && L->events_used + 5 <= L->events.size()) {
+        ev = L->events.data() + L->events_used;
+        L->events_used += 5;
+    }
+    if (ev) EK_HIP(hipEventRecord(ev[0], s));
+    ek::launch_clear_err(L->err, s);
+    ek::launch_pack(pack_args(L, ids, P, true), s);
+    if (ev) EK_HIP(hipEventRecord(ev[1], s));
+    if (P > 0) {
+        ek::StreamArgs a1;
+        a1.x = x; a1.x_stride = H; a1.rows = L->row_token; a1.offsets = L->offsets;
+        a1.slabs = L->d_slabs; a1.out = L->h; a1.out_stride = I; a1.N = (int32_t)I;
+        a1.Kdim = (int32_t)H; a1.E = E; a1.e0 = 0; a1.single_n = -1; a1.min_rows = 1;
+        a1.max_rows = INT32_MAX;
+        EK_HIP(ek::launch_ffn_stream(a1, 1, L->act, L->w8, E, s));
+        if (ev) EK_HIP(hipEventRecord(ev[2], s));
+        ek::StreamArgs a2 = a1;
+        a2.x = L->h; a2.x_stride = I; a2.rows = nullptr; a2.out = L->yp; a2.out_stride = H;
+        a2.N = (int32_t)H; a2.Kdim = (int32_t)I;
+        EK_HIP(ek::launch_ffn_stream(a2, 2, L->act, L->w8, E, s));
+        if (ev) EK_HIP(hipEventRecord(ev[3], s));
+        ek::CombineArgs c;
+        c.yp = L->yp; c.inv_perm = L->inv_perm; c.w = w; c.y = y; c.T = T; c.K = K; c.H = H;
+        c.act = L->act; c.w_f32 = w_f32;
+        ek::launch_combine(c, s);
+    } else if (ev) {
+        EK_HIP(hipEventRecord(ev[2], s));
+        EK_HIP(hipEventRecord(ev[3], s));
+    }
+    if (ev) EK_HIP(hipEventRecord(ev[4], s));
+    EK_HIP(hipGetLastError());
+    return EK_OK;
+}
+
+ek_status finish_blocking(ek_layer *L, hipStream_t s)
+{
+    EK_HIP(hipMemcpyAsync(L->h_err, L->err, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    EK_HIP(hipStreamSynchronize(s));
+    return err_to_status(L->h_err[0]);
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ C ABI
+
+#define EK_GUARDED(...)                                               \
+    try {                                                             \
+        __VA_ARGS__                                                   \
+    } catch (const std::bad_alloc &) {                                \
+        return fail(EK_OOM, "host allocation failed");                \
+    } catch (const std::exception &ex) {                              \
+        return fail(EK_INTERNAL, "exception: %s", ex.what());         \
+    } catch (...) {                                                   \
+        return fail(EK_INTERNAL, "unknown exception");                \
+    }
+
+extern "C" {
+
+const char *ek_backend_name(void) { return "hip"; }
+
+const char *ek_last_error(void) { return g_last_error.c_str(); }
+
+int32_t ek_device_count(void)
+{
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    return n;
+}
+
+ek_status ek_layer_create(const ek_cfg *cfg, ek_layer **out)
+{
+    EK_GUARDED(
+        if (!out) return fail(EK_INVALID_INPUT, "out is NULL");
+        *out = nullptr;
+        EK_TRY(validate_cfg(cfg));
+        DeviceGuard dg(cfg->device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", cfg->device_id);
+        return create_layer(cfg, cfg->max_tokens * (int64_t)cfg->top_k, out);
+    )
+}
+
+ek_status ek_layer_destroy(ek_layer *layer)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        DeviceGuard dg(layer->cfg.device_id);
+        {
+            // wait for users of the workspace
+            std::lock_guard<std::mutex> l1(layer->load_mu);
+            std::lock_guard<std::mutex> l2(layer->mu);
+        }
+        free_layer(layer);
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_set_expert(ek_layer *layer, int32_t expert, const ek_weight_desc *up,
+                              const ek_weight_desc *gate, const ek_weight_desc *down)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        if (expert < 0 || expert >= layer->cfg.n_experts)
+            return fail(EK_INVALID_INPUT, "expert %d outside [0, %d)", expert, layer->cfg.n_experts);
+        DeviceGuard dg(layer->cfg.device_id);
+        std::lock_guard<std::mutex> lk(layer->load_mu);
+        return set_expert_locked(layer, expert, up, gate, down);
+    )
+}
+
+ek_status ek_layer_remove_expert(ek_layer *layer, int32_t expert)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        if (expert < 0 || expert >= layer->cfg.n_experts)
+            return fail(EK_INVALID_INPUT, "expert %d outside [0, %d)", expert, layer->cfg.n_experts);
+        DeviceGuard dg(layer->cfg.device_id);
+        std::lock_guard<std::mutex> lk0(layer->load_mu);
+        void *old = nullptr;
+        {
+            std::lock_guard<std::mutex> lk(layer->mu);
+            old = layer->expert_mem[expert];
+            if (!old) return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", expert);
+            EK_HIP(hipDeviceSynchronize());
+            layer->expert_mem[expert] = nullptr;
+            layer->h_slabs[expert] = ek::ExpertSlab{nullptr, nullptr, nullptr, nullptr, nullptr};
+            EK_HIP(hipMemcpy(layer->d_slabs + expert, &layer->h_slabs[expert], sizeof(ek::ExpertSlab),
+                             hipMemcpyHostToDevice));
+        }
+        (void)hipFree(old);
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_has_expert(ek_layer *layer, int32_t expert, int32_t *loaded)
+{
+    EK_GUARDED(
+        if (!layer || !loaded) return fail(EK_INVALID_INPUT, "NULL argument");
+        if (expert < 0 || expert >= layer->cfg.n_experts)
+            return fail(EK_INVALID_INPUT, "expert %d outside [0, %d)", expert, layer->cfg.n_experts);
+        std::lock_guard<std::mutex> lk(layer->mu);
+        *loaded = layer->expert_mem[expert] != nullptr;
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, const void *w,
+                           int32_t w_dtype, int64_t T, void *y, const ek_route_out *route,
+                           int32_t mem, void *stream)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        if (T < 0 || T > layer->cfg.max_tokens)
+            return fail(EK_INVALID_INPUT, "T = %lld outside [0, max_tokens = %lld]", (long long)T,
+                        (long long)layer->cfg.max_tokens);
+        if (mem != EK_HOST && mem != EK_DEVICE) return fail(EK_INVALID_INPUT, "bad mem %d", mem);
+        if (w_dtype != layer->cfg.act_dtype && w_dtype != EK_F32)
+            return fail(EK_INVALID_INPUT, "w_dtype must be the activation dtype or EK_F32 (got %d)",
+                        w_dtype);
+        if (T > 0 && (!x || !ids || !w || !y)) return fail(EK_INVALID_INPUT, "NULL tensor pointer");
+        if (mem == EK_HOST && stream)
+            return fail(EK_INVALID_INPUT, "host-memory calls are blocking: stream must be NULL");
+        DeviceGuard dg(layer->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
+        Timer tm;
+        const int64_t H = layer->cfg.hidden, K = layer->cfg.top_k, P = T * K;
+        const int w_f32 = w_dtype == EK_F32;
+        std::lock_guard<std::mutex> lk(layer->mu);
+        hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+        ek_status st = EK_OK;
+        if (mem == EK_DEVICE) {
+            EK_TRY(enqueue_forward(layer, x, ids, w, w_f32, T, y, s));
+            EK_TRY(copy_route_out(layer, route, P, mem, s));
+            if (!stream) st = finish_blocking(layer, s);
+        } else {
+            EK_TRY(ensure_io_staging(layer));
+            if (T > 0) {
+                EK_HIP(hipMemcpyAsync(layer->st_x, x, (size_t)T * H * 2, hipMemcpyHostToDevice, s));
+                EK_HIP(hipMemcpyAsync(layer->st_ids, ids, (size_t)P * 4, hipMemcpyHostToDevice, s));
+                EK_HIP(hipMemcpyAsync(layer->st_w, w, (size_t)P * (w_f32 ? 4 : 2), hipMemcpyHostToDevice, s));
+            }
+            EK_TRY(enqueue_forward(layer, layer->st_x, layer->st_ids, layer->st_w, w_f32, T,
+                                   layer->st_y, s));
+            if (T > 0) EK_HIP(hipMemcpyAsync(y, layer->st_y, (size_t)T * H * 2, hipMemcpyDeviceToHost, s));
+            EK_TRY(copy_route_out(layer, route, P, mem, s));
+            st = finish_blocking(layer, s);
+        }
+        {
+            std::lock_guard<std::mutex> sl(layer->stats_mu);
+            layer->stats.forward_calls += 1;
+            layer->stats.tokens += T;
+            layer->stats.pairs += P;
+            if (!stream) layer->stats.last_forward_us = tm.us();
+        }
+        return st;
+    )
+}
+
+ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek_route_out *route,
+                        const void *x, void *xp, int32_t mem, void *stream)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        if (T < 0 || T > layer->cfg.max_tokens)
+            return fail(EK_INVALID_INPUT, "T = %lld outside [0, max_tokens = %lld]", (long long)T,
+                        (long long)layer->cfg.max_tokens);
+        if (mem != EK_HOST && mem != EK_DEVICE) return fail(EK_INVALID_INPUT, "bad mem %d", mem);
+        if (T > 0 && !ids) return fail(EK_INVALID_INPUT, "ids is NULL");
+        if (xp && !x) return fail(EK_INVALID_INPUT, "xp requested but x is NULL");
+        if (mem == EK_HOST && stream)
+            return fail(EK_INVALID_INPUT, "host-memory calls are blocking: stream must be NULL");
+        DeviceGuard dg(layer->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
+        const int64_t H = layer->cfg.hidden, K = layer->cfg.top_k, P = T * K;
+        std::lock_guard<std::mutex> lk(layer->mu);
+        hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+        const int32_t *d_ids = ids;
+        const void *d_x = x;
+        void *d_xp = xp;
+        if (mem == EK_HOST) {
+            EK_TRY(ensure_io_staging(layer));
+            if (P > 0) EK_HIP(hipMemcpyAsync(layer->st_ids, ids, (size_t)P * 4, hipMemcpyHostToDevice, s));
+            d_ids = layer->st_ids;
+            if (xp && T > 0) {
+                EK_HIP(hipMemcpyAsync(layer->st_x, x, (size_t)T * H * 2, hipMemcpyHostToDevice, s));
+                d_x = layer->st_x;
+                d_xp = layer->yp;   // [Pmax, H] scratch of the right size
+            }
+        }
+        ek::launch_clear_err(layer->err, s);
+        ek::launch_pack(pack_args(layer, d_ids, P, false), s);
+        if (xp) ek::launch_gather(d_x, layer->row_token, P, H * 2, d_xp, s);
+        EK_HIP(hipGetLastError());
+        if (mem == EK_HOST && xp && P > 0)
+            EK_HIP(hipMemcpyAsync(xp, d_xp, (size_t)P * H * 2, hipMemcpyDeviceToHost, s));
+        EK_TRY(copy_route_out(layer, route, P, mem, s));
+        if (!stream) return finish_blocking(layer, s);
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x, int64_t n,
+                                  void *out, int32_t mem, void *stream)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        if (expert < 0 || expert >= layer->cfg.n_experts)
+            return fail(EK_INVALID_INPUT, "expert %d outside [0, %d)", expert, layer->cfg.n_experts);
+        if (n < 0 || n > layer->Pmax)
+            return fail(EK_INVALID_INPUT, "n = %lld outside [0, %lld]", (long long)n,
+                        (long long)layer->Pmax);
+        if (mem != EK_HOST && mem != EK_DEVICE) return fail(EK_INVALID_INPUT, "bad mem %d", mem);
+        if (n > 0 && (!x || !out)) return fail(EK_INVALID_INPUT, "NULL tensor pointer");
+        if (mem == EK_HOST && stream)
+            return fail(EK_INVALID_INPUT, "host-memory calls are blocking: stream must be NULL");
+        DeviceGuard dg(layer->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
+        const int64_t H = layer->cfg.hidden, I = layer->cfg.inter;
+        std::lock_guard<std::mutex> lk(layer->mu);
+        if (!layer->expert_mem[expert])
+            return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", expert);
+        hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+        if (n > 0) {
+            const void *d_x = x;
+            void *d_out = out;
+            if (mem == EK_HOST) {
+                EK_TRY(ensure_io_staging(layer));
+                EK_HIP(hipMemcpyAsync(layer->st_x, x, (size_t)n * H * 2, hipMemcpyHostToDevice, s));
+                d_x = layer->st_x;
+                d_out = layer->st_y;
+            }
+            ek::StreamArgs a1;
+            a1.x = d_x; a1.x_stride = H; a1.rows = nullptr; a1.offsets = nullptr;
+            a1.slabs = layer->d_slabs; a1.out = layer->h; a1.out_stride = I; a1.N = (int32_t)I;
+            a1.Kdim = (int32_t)H; a1.E = layer->cfg.n_experts; a1.e0 = expert;
+            a1.single_n = (int32_t)n; a1.min_rows = 1; a1.max_rows = INT32_MAX;
+            EK_HIP(ek::launch_ffn_stream(a1, 1, layer->act, layer->w8, 1, s));
+            ek::StreamArgs a2 = a1;
+            a2.x = layer->h; a2.x_stride = I; a2.out = d_out; a2.out_stride = H; a2.N = (int32_t)H;
+            a2.Kdim = (int32_t)I;
+            EK_HIP(ek::launch_ffn_stream(a2, 2, layer->act, layer->w8, 1, s));
+            if (mem == EK_HOST)
+                EK_HIP(hipMemcpyAsync(out, layer->st_y, (size_t)n * H * 2, hipMemcpyDeviceToHost, s));
+        }
+        if (!stream) EK_HIP(hipStreamSynchronize(s));
+        {
+            std::lock_guard<std::mutex> sl(layer->stats_mu);
+            layer->stats.expert_forward_calls += 1;
+        }
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_profile(ek_layer *layer, int32_t enable)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        DeviceGuard dg(layer->cfg.device_id);
+        std::lock_guard<std::mutex> lk(layer->mu);
+        if (enable && layer->events.empty()) {
+            layer->events.reserve(5 * 1024);
+            for (int i = 0; i < 5 * 1024; ++i) {
+                hipEvent_t ev;
+                EK_HIP(hipEventCreate(&ev));
+                layer->events.push_back(ev);
+            }
+        }
+        if (layer->events_used) EK_HIP(hipEventSynchronize(layer->events[layer->events_used - 1]));
+        layer->events_used = 0;
+        layer->profiling = enable != 0;
+        std::lock_guard<std::mutex> sl(layer->stats_mu);
+        for (double &v : layer->stats.kernel_us) v = 0.0;
+        layer->stats.profiled_calls = 0;
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_get_stats(ek_layer *layer, ek_stats *out)
+{
+    EK_GUARDED(
+        if (!layer || !out) return fail(EK_INVALID_INPUT, "NULL argument");
+        DeviceGuard dg(layer->cfg.device_id);
+        std::lock_guard<std::mutex> lk(layer->mu);
+        std::lock_guard<std::mutex> sl(layer->stats_mu);
+        for (size_t i = 0; i + 5 <= layer->events_used; i += 5) {
+            hipEvent_t *ev = layer->events.data() + i;
+            EK_HIP(hipEventSynchronize(ev[4]));
+            for (int k = 0; k < 4; ++k) {
+                float ms = 0.f;
+                EK_HIP(hipEventElapsedTime(&ms, ev[k], ev[k + 1]));
+                layer->stats.kernel_us[k] += 1e3 * ms;
+            }
+            layer->stats.profiled_calls += 1;
+        }
+        layer->events_used = 0;
+        *out = layer->stats;
+        return EK_OK;
+    )
+}
+
+ek_status ek_expert_create(const ek_cfg *cfg, int64_t max_rows, const ek_weight_desc *up,
+                           const ek_weight_desc *gate, const ek_weight_desc *down, ek_expert **out)
+{
+    EK_GUARDED(
+        if (!out) return fail(EK_INVALID_INPUT, "out is NULL");
+        *out = nullptr;
+        if (!cfg) return fail(EK_INVALID_INPUT, "cfg is NULL");
+        ek_cfg c = *cfg;
+        c.n_experts = 1;
+        c.top_k = 1;
+        c.max_tokens = max_rows;
+        EK_TRY(validate_cfg(&c));
+        DeviceGuard dg(c.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", c.device_id);
+        ek_layer *L = nullptr;
+        EK_TRY(create_layer(&c, max_rows, &L));
+        ek_status st;
+        {
+            std::lock_guard<std::mutex> lk(L->load_mu);
+            st = set_expert_locked(L, 0, up, gate, down);
+        }
+        if (st != EK_OK) {
+            std::string keep = g_last_error;
+            free_layer(L);
+            g_last_error = keep;
+            return st;
+        }
+        ek_expert *x = new (std::nothrow) ek_expert();
+        if (!x) { free_layer(L); return fail(EK_OOM, "host allocation failed"); }
+        x->layer = L;
+        *out = x;
+        return EK_OK;
+    )
+}
+
+ek_status ek_expert_forward(ek_expert *expert, const void *x, int64_t n, void *out, int32_t mem,
+                            void *stream)
+{
+    if (!expert || !expert->layer) return fail(EK_INVALID_INPUT, "expert is NULL");
+    return ek_layer_expert_forward(expert->layer, 0, x, n, out, mem, stream);
+}
+
+ek_status ek_expert_shape(ek_expert *expert, int64_t *hidden, int64_t *inter)
+{
+    if (!expert || !expert->layer || !hidden || !inter) return fail(EK_INVALID_INPUT, "NULL argument");
+    *hidden = expert->layer->cfg.hidden;
+    *inter = expert->layer->cfg.inter;
+    return EK_OK;
+}
+
+ek_status ek_expert_destroy(ek_expert *expert)
+{
+    EK_GUARDED(
+        if (!expert) return fail(EK_INVALID_INPUT, "expert is NULL");
+        ek_status st = expert->layer ? ek_layer_destroy(expert->layer) : EK_OK;
+        delete expert;
+        return st;
+    )
+}
+
+}  // extern "C"

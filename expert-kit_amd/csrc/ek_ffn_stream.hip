@@ -1,0 +1,241 @@
+// Ragged grouped SwiGLU FFN, weight-streaming kernel (short segments).
+//
+// Computes, per expert segment, the four ops of TorchFFN's closure
+// (ek-computation/src/ffn/expert_torch.rs:81-84):
+//   stage 1:  h   = (x . W_up^T) * silu(x . W_gate^T)
+//   stage 2:  out = h . W_down^T
+// with the reference's storage roundings (up, gate, silu(gate), h and out are
+// each rounded to the activation dtype) and fp32 accumulation on MFMA.
+//
+// Regime: a handful of rows per expert, so the kernel is bound by streaming
+// every active expert's weights from HBM exactly once.  One wavefront owns NG
+// groups of 16 output channels and walks the whole contraction:
+//   - weights are the MFMA "A" operand (16 channels x 32 k), fetched with one
+//     16-byte load per lane straight from the chunked HBM layout (no LDS);
+//   - the <= 16 activation rows of the segment are the "B" operand (32 k x 16
+//     rows), re-read from L2 by every wave;
+//   - D loads deep software prefetch keeps >= D KiB per wave in flight.
+// int8 weights are stored offset-binary (q + 128): v_cvt_f32_ubyteN +
+// v_cvt_pk_bf16_f32 turn 4 bytes into 4 exact bf16 integers, one extra MFMA
+// against an all-ones A operand accumulates sum_k x[k], and the epilogue
+// forms (acc - 128 * sum_x) * scale[channel].
+#include "ek_internal.h"
+
+namespace ek {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Act;
+template <> struct Act<__bf16> {
+    using V8 = bf16x8;
+    static __device__ __forceinline__ f32x4 mfma(V8 a, V8 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Act<_Float16> {
+    using V8 = f16x8;
+    static __device__ __forceinline__ f32x4 mfma(V8 a, V8 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <typename T> __device__ __forceinline__ float rnd(float v) { return (float)(T)v; }
+
+// 8 offset-binary bytes (two dwords) -> 8 exact integers in T
+template <typename T>
+__device__ __forceinline__ typename Act<T>::V8 cvt_u8x8(uint32_t lo, uint32_t hi)
+{
+    typename Act<T>::V8 r;
+    r[0] = (T)(float)(lo & 0xffu);
+    r[1] = (T)(float)((lo >> 8) & 0xffu);
+    r[2] = (T)(float)((lo >> 16) & 0xffu);
+    r[3] = (T)(float)(lo >> 24);
+    r[4] = (T)(float)(hi & 0xffu);
+    r[5] = (T)(float)((hi >> 8) & 0xffu);
+    r[6] = (T)(float)((hi >> 16) & 0xffu);
+    r[7] = (T)(float)(hi >> 24);
+    return r;
+}
+
+template <typename T, bool W8, int NMAT, int NG, int D>
+__global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
+{
+    using V8 = typename Act<T>::V8;
+    constexpr int KE = W8 ? 64 : 32;   // contraction elements per chunk
+    constexpr int XV = W8 ? 2 : 1;     // 16-byte activation loads per chunk per lane
+    constexpr int NW = NMAT * NG;      // weight chunks per k step per wave
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int e, seg0, n;
+    if (a.single_n >= 0) {
+        e = a.e0; seg0 = 0; n = a.single_n;
+    } else {
+        e = blockIdx.y;
+        seg0 = a.offsets[e];
+        n = a.offsets[e + 1] - seg0;
+    }
+    if (n < a.min_rows || n > a.max_rows) return;
+    const int NT = a.N >> 4;
+    const int nt0 = (blockIdx.x * 4 + wave) * NG;
+    if (nt0 >= NT) return;
+    const ExpertSlab slab = a.slabs[e];
+    const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
+    if (wmat == nullptr) return;   // expert not loaded: pack has flagged the call
+    const int KT = a.Kdim / KE;
+    const int j = lane & 15, g = lane >> 4;
+
+    const uint8_t *wp[NG];
+#pragma unroll
+    for (int gi = 0; gi < NG; ++gi)
+        wp[gi] = wmat + (int64_t)(nt0 + gi) * KT * (NMAT * kChunkBytes) + lane * 16;
+
+    V8 ones;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ones[i] = (T)1.0f;
+
+    for (int r0 = 0; r0 < n; r0 += 16) {
+        const int jr = min(r0 + j, n - 1);   // lanes past the segment re-read its last row
+        const int64_t row = a.rows ? (int64_t)a.rows[seg0 + jr] : (int64_t)(seg0 + jr);
+        const T *xp = (const T *)a.x + row * a.x_stride + g * (KE / 4);
+
+        f32x4 acc[NMAT][NG];
+        f32x4 accs = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi) acc[m][gi] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+        uint4 wq[D][NW];
+        uint4 xq[D][XV];
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+                    wq[d][gi * NMAT + m] =
+                        *(const uint4 *)(wp[gi] + (int64_t)(d * NMAT + m) * kChunkBytes);
+#pragma unroll
+            for (int v = 0; v < XV; ++v) xq[d][v] = *(const uint4 *)(xp + d * KE + v * 8);
+        }
+
+        for (int kt0 = 0; kt0 < KT; kt0 += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                const int kt = kt0 + d;
+                // consume slot d
+                if constexpr (W8) {
+                    const V8 x0 = __builtin_bit_cast(V8, xq[d][0]);
+                    const V8 x1 = __builtin_bit_cast(V8, xq[d][1]);
+                    accs = Act<T>::mfma(ones, x0, accs);
+                    accs = Act<T>::mfma(ones, x1, accs);
+#pragma unroll
+                    for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+                        for (int m = 0; m < NMAT; ++m) {
+                            const uint4 q = wq[d][gi * NMAT + m];
+                            acc[m][gi] = Act<T>::mfma(cvt_u8x8<T>(q.x, q.y), x0, acc[m][gi]);
+                            acc[m][gi] = Act<T>::mfma(cvt_u8x8<T>(q.z, q.w), x1, acc[m][gi]);
+                        }
+                } else {
+                    const V8 x0 = __builtin_bit_cast(V8, xq[d][0]);
+#pragma unroll
+                    for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+                        for (int m = 0; m < NMAT; ++m)
+                            acc[m][gi] = Act<T>::mfma(__builtin_bit_cast(V8, wq[d][gi * NMAT + m]),
+                                                      x0, acc[m][gi]);
+                }
+                // refill slot d with chunk kt + D
+                if (kt + D < KT) {
+#pragma unroll
+                    for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+                        for (int m = 0; m < NMAT; ++m)
+                            wq[d][gi * NMAT + m] = *(const uint4 *)(
+                                wp[gi] + (int64_t)((kt + D) * NMAT + m) * kChunkBytes);
+#pragma unroll
+                    for (int v = 0; v < XV; ++v)
+                        xq[d][v] = *(const uint4 *)(xp + (int64_t)(kt + D) * KE + v * 8);
+                }
+            }
+        }
+
+        // epilogue: lane (g, j) holds channels nt*16 + 4g + r (r = 0..3) of row r0 + j
+        if (r0 + j < n) {
+            T *orow = (T *)a.out + (int64_t)(seg0 + r0 + j) * a.out_stride;
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi) {
+                const int ch = (nt0 + gi) * 16 + 4 * g;
+                typedef T T4 __attribute__((ext_vector_type(4)));
+                T4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if constexpr (NMAT == 2) {
+                        float up = acc[0][gi][r], gate = acc[1][gi][r];
+                        if constexpr (W8) {
+                            up = (up - 128.f * accs[r]) * slab.s_up[ch + r];
+                            gate = (gate - 128.f * accs[r]) * slab.s_gate[ch + r];
+                        }
+                        up = rnd<T>(up);
+                        gate = rnd<T>(gate);
+                        const float sg = rnd<T>(gate / (1.0f + expf(-gate)));
+                        o[r] = (T)(up * sg);
+                    } else {
+                        float v = acc[0][gi][r];
+                        if constexpr (W8) v = (v - 128.f * accs[r]) * slab.s_down[ch + r];
+                        o[r] = (T)v;
+                    }
+                }
+                *(uint2 *)(orow + ch) = __builtin_bit_cast(uint2, o);
+            }
+        }
+    }
+}
+
+template <typename T, bool W8, int NMAT, int NG>
+static hipError_t launch_d(const StreamArgs &a, int32_t nseg, hipStream_t s)
+{
+    constexpr int KE = W8 ? 64 : 32;
+    const int KT = a.Kdim / KE;
+    const int NT = a.N / 16;
+    dim3 grid((NT + 4 * NG - 1) / (4 * NG), nseg);
+    if (KT % 4 == 0)
+        hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, 4>), grid, dim3(256), 0, s, a);
+    else if (KT % 2 == 0)
+        hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, 2>), grid, dim3(256), 0, s, a);
+    else
+        hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, 1>), grid, dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+template <typename T, bool W8, int NMAT>
+static hipError_t launch_g(const StreamArgs &a, int32_t nseg, hipStream_t s)
+{
+    const int NT = a.N / 16;
+    if (NMAT == 1 && NT % 4 == 0) return launch_d<T, W8, NMAT, 4>(a, nseg, s);
+    if (NT % 2 == 0) return launch_d<T, W8, NMAT, 2>(a, nseg, s);
+    return launch_d<T, W8, NMAT, 1>(a, nseg, s);
+}
+
+hipError_t launch_ffn_stream(const StreamArgs &a, int stage, int act, bool w8, int32_t n_segments,
+                             hipStream_t s)
+{
+    if (n_segments <= 0) return hipSuccess;
+    if (act == 0) {
+        if (w8) return stage == 1 ? launch_g<__bf16, true, 2>(a, n_segments, s)
+                                  : launch_g<__bf16, true, 1>(a, n_segments, s);
+        return stage == 1 ? launch_g<__bf16, false, 2>(a, n_segments, s)
+                          : launch_g<__bf16, false, 1>(a, n_segments, s);
+    }
+    if (w8) return stage == 1 ? launch_g<_Float16, true, 2>(a, n_segments, s)
+                              : launch_g<_Float16, true, 1>(a, n_segments, s);
+    return stage == 1 ? launch_g<_Float16, false, 2>(a, n_segments, s)
+                      : launch_g<_Float16, false, 1>(a, n_segments, s);
+}
+
+}  // namespace ek

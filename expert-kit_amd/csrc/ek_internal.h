@@ -1,0 +1,98 @@
+// Internal declarations shared by the HIP kernels and the C-ABI host code.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ek {
+
+// ---- HBM weight layout ------------------------------------------------------
+// A weight matrix [N, K] (row-major, out_features x in_features) is stored as
+// 1 KiB chunks.  One chunk is what one wavefront fetches with a single 16-byte
+// load per lane and feeds to MFMA without any shuffle:
+//   chunk (nt, kt) covers rows nt*16 .. nt*16+15 and KE consecutive k
+//   (KE = 64 for int8, 32 for 16-bit types); lane l = g*16 + i holds the
+//   16 bytes W[nt*16 + i][kt*KE + g*KE/4 .. + KE/4).
+// A "matrix group" interleaves NMAT matrices of equal shape chunk by chunk
+// (up and gate are one group, so one wave streams one contiguous range):
+//   byte offset of chunk (nt, kt, m) = ((nt*KT + kt)*NMAT + m) * 1024.
+// int8 values are stored offset-binary (q + 128, i.e. q ^ 0x80) so that
+// v_cvt_f32_ubyte* converts them; the kernels subtract 128 * sum_k x[k].
+constexpr int kChunkBytes = 1024;
+
+struct ExpertSlab {           // device addresses of one expert's tensors
+    const uint8_t *upgate;    // matrix group {up, gate}: N = I, K = H
+    const uint8_t *down;      // matrix group {down}:     N = H, K = I
+    const float *s_up;        // [I] fp32 scales (int8 only, else nullptr)
+    const float *s_gate;      // [I]
+    const float *s_down;      // [H]
+};
+
+// ---- routing (pack) ---------------------------------------------------------
+struct PackArgs {
+    const int32_t *ids;       // [P]
+    int64_t P;
+    int32_t E;
+    int32_t K;
+    int32_t nblocks;          // ceil(P / kPackChunk)
+    const ExpertSlab *slabs;  // [E]; upgate == nullptr means "not loaded"
+    int32_t *block_hist;      // [nblocks][E]
+    int32_t *counts;          // [E]
+    int32_t *offsets;         // [E+1]
+    int32_t *perm;            // [P]
+    int32_t *inv_perm;        // [P]
+    int32_t *row_token;       // [P]  perm[j] / K
+    int32_t *err;             // bit 0: id out of range, bit 1: expert not loaded
+};
+constexpr int kPackChunk = 4096;   // pairs per workgroup
+constexpr int kPackThreads = 256;
+constexpr int kMaxExperts = 1024;
+
+void launch_clear_err(int32_t *err, hipStream_t s);   // fill kernel (graph-capture safe)
+void launch_pack(const PackArgs &a, hipStream_t s);
+void launch_gather(const void *x, const int32_t *row_token, int64_t P, int64_t row_bytes, void *xp,
+                   hipStream_t s);
+
+// ---- grouped FFN, weight-streaming kernel -------------------------------------
+struct StreamArgs {
+    const void *x;            // activations, row stride x_stride elements
+    int64_t x_stride;
+    const int32_t *rows;      // packed position -> row of x, or nullptr (identity)
+    const int32_t *offsets;   // [E+1] segment starts (ignored when single_n >= 0)
+    const ExpertSlab *slabs;  // [E]
+    void *out;                // stage 1: h [P, N]; stage 2: yp [P, N]
+    int64_t out_stride;
+    int32_t N;                // output channels of this stage
+    int32_t Kdim;             // contraction length of this stage
+    int32_t E;
+    int32_t e0;               // expert id when single_n >= 0
+    int32_t single_n;         // >= 0: one segment [0, single_n) of expert e0
+    int32_t min_rows;         // segments with fewer rows are skipped
+    int32_t max_rows;         // segments with more rows are skipped
+};
+// stage = 1: up/gate + SwiGLU epilogue;  stage = 2: down projection
+// act: 0 bf16, 1 f16;  w8: int8 weights with per-channel scales
+hipError_t launch_ffn_stream(const StreamArgs &a, int stage, int act, bool w8, int32_t n_segments,
+                             hipStream_t s);
+
+// ---- combine ----------------------------------------------------------------
+struct CombineArgs {
+    const void *yp;           // [P, H] packed expert outputs
+    const int32_t *inv_perm;  // [T*K]
+    const void *w;            // [T, K]
+    void *y;                  // [T, H]
+    int64_t T;
+    int32_t K;
+    int64_t H;
+    int32_t act;              // 0 bf16, 1 f16
+    int32_t w_f32;            // gate weights are fp32 (DeepSeek shim) instead of act dtype
+};
+void launch_combine(const CombineArgs &a, hipStream_t s);
+
+// ---- weight ingestion -------------------------------------------------------
+// src [N, K] row-major of src_dtype (ek_dtype numbering) -> chunked layout at
+// dst, matrix m of an nmat-group.  dst_dtype: 0 bf16, 1 f16, 3 int8.
+void launch_tile_weights(const void *src, int src_dtype, int64_t N, int64_t K, uint8_t *dst,
+                         int dst_dtype, int m, int nmat, hipStream_t s);
+void launch_scales_to_f32(const void *src, int src_dtype, int64_t n, float *dst, hipStream_t s);
+
+}  // namespace ek

@@ -1,0 +1,130 @@
+// Weighted scatter-combine and weight ingestion kernels (HBM-bound copies).
+#include "ek_internal.h"
+
+namespace ek {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// y[t, :] = sum_k w[t,k] * Yp[inv_perm[t*K + k], :], k ascending.
+// Follows the shim's weighted sum (qwen3_moe.py:102-104): the product tensor
+// has the promoted dtype of its operands, torch.sum accumulates in fp32 and
+// rounds once.  WF32 = gate weights kept in fp32 (deepseek_v3/model.py:97-103),
+// so the product is not rounded.  The scatter back to [T,K,H]
+// (controller/executor.rs:203-252) is folded into the indexed read.
+// Fixed summation order, no atomics: bit-reproducible.
+template <typename T, bool WF32>
+__global__ __launch_bounds__(256) void combine_kernel(CombineArgs a)
+{
+    typedef T V8 __attribute__((ext_vector_type(8)));
+    const int64_t t = blockIdx.x;
+    const int64_t c = ((int64_t)blockIdx.y * 256 + threadIdx.x) * 8;
+    if (c >= a.H) return;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    for (int k = 0; k < a.K; ++k) {
+        const int32_t pos = a.inv_perm[t * a.K + k];
+        if (pos < 0) continue;
+        const float wv = WF32 ? ((const float *)a.w)[t * a.K + k] : (float)((const T *)a.w)[t * a.K + k];
+        const V8 v = *(const V8 *)((const T *)a.yp + (int64_t)pos * a.H + c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float p = wv * (float)v[i];
+            if (!WF32) p = (float)(T)p;
+            acc[i] = acc[i] + p;
+        }
+    }
+    V8 o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = (T)acc[i];
+    *(V8 *)((T *)a.y + t * a.H + c) = o;
+}
+
+void launch_combine(const CombineArgs &a, hipStream_t s)
+{
+    if (a.T <= 0) return;
+    dim3 grid((unsigned)a.T, (unsigned)((a.H / 8 + 255) / 256));
+    if (a.act == 0) {
+        if (a.w_f32) hipLaunchKernelGGL((combine_kernel<__bf16, true>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((combine_kernel<__bf16, false>), grid, dim3(256), 0, s, a);
+    } else {
+        if (a.w_f32) hipLaunchKernelGGL((combine_kernel<_Float16, true>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((combine_kernel<_Float16, false>), grid, dim3(256), 0, s, a);
+    }
+}
+
+// ---- weight ingestion ---------------------------------------------------------
+
+__device__ __forceinline__ float load_src(const void *src, int dt, int64_t i)
+{
+    switch (dt) {
+    case 0: return (float)((const __bf16 *)src)[i];
+    case 1: return (float)((const _Float16 *)src)[i];
+    default: return ((const float *)src)[i];
+    }
+}
+
+// One thread writes one lane's 16 bytes of one chunk.
+template <typename T>
+__global__ __launch_bounds__(256) void tile_weights16_kernel(const void *src, int src_dt, int64_t N,
+                                                            int64_t K, uint8_t *dst, int m, int nmat)
+{
+    typedef T V8 __attribute__((ext_vector_type(8)));
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t KT = K / 32, total = (N / 16) * KT * 64;
+    if (idx >= total) return;
+    const int l = idx & 63;
+    const int64_t chunk = idx >> 6, nt = chunk / KT, kt = chunk % KT;
+    const int64_t row = nt * 16 + (l & 15), col = kt * 32 + (l >> 4) * 8;
+    V8 v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (T)load_src(src, src_dt, row * K + col + i);
+    *(V8 *)(dst + (chunk * nmat + m) * kChunkBytes + l * 16) = v;
+}
+
+__global__ __launch_bounds__(256) void tile_weights8_kernel(const uint8_t *src, int64_t N, int64_t K,
+                                                           uint8_t *dst, int m, int nmat)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t KT = K / 64, total = (N / 16) * KT * 64;
+    if (idx >= total) return;
+    const int l = idx & 63;
+    const int64_t chunk = idx >> 6, nt = chunk / KT, kt = chunk % KT;
+    const int64_t row = nt * 16 + (l & 15), col = kt * 64 + (l >> 4) * 16;
+    uint4 v = *(const uint4 *)(src + row * K + col);
+    v.x ^= 0x80808080u; v.y ^= 0x80808080u; v.z ^= 0x80808080u; v.w ^= 0x80808080u;
+    *(uint4 *)(dst + (chunk * nmat + m) * kChunkBytes + l * 16) = v;
+}
+
+void launch_tile_weights(const void *src, int src_dtype, int64_t N, int64_t K, uint8_t *dst,
+                         int dst_dtype, int m, int nmat, hipStream_t s)
+{
+    if (dst_dtype == 3) {
+        const int64_t total = (N / 16) * (K / 64) * 64;
+        hipLaunchKernelGGL(tile_weights8_kernel, dim3((total + 255) / 256), dim3(256), 0, s,
+                           (const uint8_t *)src, N, K, dst, m, nmat);
+    } else {
+        const int64_t total = (N / 16) * (K / 32) * 64;
+        if (dst_dtype == 0)
+            hipLaunchKernelGGL(tile_weights16_kernel<__bf16>, dim3((total + 255) / 256), dim3(256), 0,
+                               s, src, src_dtype, N, K, dst, m, nmat);
+        else
+            hipLaunchKernelGGL(tile_weights16_kernel<_Float16>, dim3((total + 255) / 256), dim3(256),
+                               0, s, src, src_dtype, N, K, dst, m, nmat);
+    }
+}
+
+__global__ void scales_to_f32_kernel(const void *src, int dt, int64_t n, float *dst)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = load_src(src, dt, i);
+}
+
+void launch_scales_to_f32(const void *src, int src_dtype, int64_t n, float *dst, hipStream_t s)
+{
+    hipLaunchKernelGGL(scales_to_f32_kernel, dim3((n + 255) / 256), dim3(256), 0, s, src, src_dtype,
+                       n, dst);
+}
+
+}  // namespace ek

@@ -1,0 +1,173 @@
+// Routing / pack kernels: (token, slot) -> per-expert contiguous segments.
+//
+// Reproduces, as a stable counting sort, the grouping that
+// NaiveExecutor::break_down_to_egress builds with per-expert push lists
+// (ek-computation/src/controller/executor.rs:283-304): within an expert's
+// segment the pairs keep ascending flat index t*K + k.
+//
+// Three launches, all integer work, all HBM/LDS bound:
+//   pack_hist : one LDS histogram per 4096-pair chunk
+//   pack_scan : per-expert exclusive scan over chunks, then a wavefront
+//               prefix scan over experts -> counts, offsets
+//   pack_rank : stable rank of every pair inside its chunk by wave-level
+//               match (ballots over the id bits) -> perm, inv_perm, row_token
+// plus a coalesced row gather (assemble_seq_tensors, executor.rs:112-133).
+#include "ek_internal.h"
+
+namespace ek {
+
+__global__ __launch_bounds__(kPackThreads) void pack_hist_kernel(PackArgs a)
+{
+    __shared__ int32_t hist[kMaxExperts];
+    for (int i = threadIdx.x; i < a.E; i += kPackThreads) hist[i] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * kPackChunk;
+    const int64_t end = min(base + (int64_t)kPackChunk, a.P);
+    bool bad = false;
+    for (int64_t p = base + threadIdx.x; p < end; p += kPackThreads) {
+        const int32_t id = a.ids[p];
+        if ((uint32_t)id < (uint32_t)a.E) atomicAdd(&hist[id], 1);
+        else bad = true;
+    }
+    if (bad) atomicOr(a.err, 1);
+    __syncthreads();
+    for (int i = threadIdx.x; i < a.E; i += kPackThreads)
+        a.block_hist[(int64_t)blockIdx.x * a.E + i] = hist[i];
+}
+
+// One workgroup of 1024 threads; thread e owns expert e.
+__global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
+{
+    __shared__ int32_t wave_tot[16];
+    const int e = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int32_t total = 0;
+    if (e < a.E) {
+        for (int b = 0; b < a.nblocks; ++b) {
+            const int64_t idx = (int64_t)b * a.E + e;
+            const int32_t t = a.block_hist[idx];
+            a.block_hist[idx] = total;   // exclusive prefix over chunks
+            total += t;
+        }
+        a.counts[e] = total;
+        if (total > 0 && a.slabs != nullptr && a.slabs[e].upgate == nullptr) atomicOr(a.err, 2);
+    }
+    // inclusive prefix scan across the wavefront
+    int32_t incl = total;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int32_t up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+    }
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    int32_t wave_base = 0;
+    for (int w = 0; w < wave; ++w) wave_base += wave_tot[w];
+    if (e < a.E) a.offsets[e] = wave_base + incl - total;
+    if (e == a.E - 1) a.offsets[a.E] = wave_base + incl;
+}
+
+__global__ __launch_bounds__(kPackThreads) void pack_rank_kernel(PackArgs a, int nbits)
+{
+    constexpr int kWaves = kPackThreads / 64;
+    constexpr int kSub = kPackChunk / kWaves;   // pairs per wave, consecutive
+    __shared__ int32_t wbase[kWaves][kMaxExperts];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < kWaves * kMaxExperts; i += kPackThreads) (&wbase[0][0])[i] = 0;
+    __syncthreads();
+    const int64_t start = (int64_t)blockIdx.x * kPackChunk + (int64_t)wave * kSub;
+    for (int it = 0; it < kSub / 64; ++it) {
+        const int64_t p = start + it * 64 + lane;
+        if (p < a.P) {
+            const int32_t id = a.ids[p];
+            if ((uint32_t)id < (uint32_t)a.E) atomicAdd(&wbase[wave][id], 1);
+        }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < a.E; e += kPackThreads) {
+        int32_t run = a.offsets[e] + a.block_hist[(int64_t)blockIdx.x * a.E + e];
+        for (int w = 0; w < kWaves; ++w) {
+            const int32_t t = wbase[w][e];
+            wbase[w][e] = run;
+            run += t;
+        }
+    }
+    __syncthreads();
+    // Each wave walks its own consecutive pairs 64 at a time; lanes holding
+    // the same expert id find each other with one ballot per id bit, so the
+    // rank inside the group is the number of lower lanes in the group.
+    for (int it = 0; it < kSub / 64; ++it) {
+        const int64_t p = start + it * 64 + lane;
+        int32_t id = 0;
+        bool valid = false;
+        if (p < a.P) {
+            id = a.ids[p];
+            valid = (uint32_t)id < (uint32_t)a.E;
+            if (!valid) a.inv_perm[p] = -1;
+        }
+        uint64_t m = __ballot(valid);
+        for (int b = 0; b < nbits; ++b) {
+            const bool bit = (id >> b) & 1;
+            const uint64_t bb = __ballot(bit);
+            m &= bit ? bb : ~bb;
+        }
+        if (valid) {
+            const int32_t rank = __popcll(m & ((1ull << lane) - 1ull));
+            const int32_t pos = wbase[wave][id] + rank;
+            const bool leader = (m >> lane) == 1ull;   // highest lane of the group
+            if (leader) wbase[wave][id] = pos + 1;
+            a.perm[pos] = (int32_t)p;
+            a.inv_perm[p] = pos;
+            a.row_token[pos] = (int32_t)(p / a.K);
+        }
+    }
+}
+
+__global__ void clear_err_kernel(int32_t *err) { err[0] = 0; }
+
+void launch_clear_err(int32_t *err, hipStream_t s)
+{
+    hipLaunchKernelGGL(clear_err_kernel, dim3(1), dim3(1), 0, s, err);
+}
+
+void launch_pack(const PackArgs &a, hipStream_t s)
+{
+    if (a.P <= 0) {
+        // offsets and counts must still be defined (all zero)
+        PackArgs z = a;
+        z.nblocks = 0;
+        hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(1024), 0, s, z);
+        return;
+    }
+    int nbits = 0;
+    while ((1 << nbits) < a.E) ++nbits;
+    hipLaunchKernelGGL(pack_hist_kernel, dim3(a.nblocks), dim3(kPackThreads), 0, s, a);
+    hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(1024), 0, s, a);
+    hipLaunchKernelGGL(pack_rank_kernel, dim3(a.nblocks), dim3(kPackThreads), 0, s, a, nbits);
+}
+
+// Xp[j, :] = x[row_token[j], :], 16 bytes per lane, one workgroup per row slice.
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint4 *x, const int32_t *row_token,
+                                                         int64_t P, int64_t row_vec, uint4 *xp)
+{
+    const int64_t j = blockIdx.y;
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (j >= P || c >= row_vec) return;
+    xp[j * row_vec + c] = x[(int64_t)row_token[j] * row_vec + c];
+}
+
+void launch_gather(const void *x, const int32_t *row_token, int64_t P, int64_t row_bytes, void *xp,
+                   hipStream_t s)
+{
+    if (P <= 0) return;
+    const int64_t row_vec = row_bytes / 16;
+    // grid.y is limited to 65535: walk P in slabs
+    for (int64_t j0 = 0; j0 < P; j0 += 65535) {
+        const int64_t nj = (P - j0) < 65535 ? (P - j0) : 65535;
+        hipLaunchKernelGGL(gather_rows_kernel, dim3((row_vec + 255) / 256, nj), dim3(256), 0, s,
+                           (const uint4 *)x, row_token + j0, nj, row_vec,
+                           (uint4 *)xp + j0 * row_vec);
+    }
+}
+
+}  // namespace ek

@@ -1,0 +1,292 @@
+"""Host-side mirror of the reference's worker-side expert interface, over the C ABI.
+
+Names, argument meaning and error behaviour follow the Rust items they stand
+for, so the parity tests read like the reference's own:
+
+  EKInstance     ek-computation/src/x.rs:27-32
+  ExpertWeight   ek-computation/src/ffn/meta.rs:10-23, loader :56-75
+  HipFFN         a third implementation of trait Expert<T> (ffn/meta.rs:30-39),
+                 next to TorchFFN (ffn/expert_torch.rs:94-128)
+  ExpertBackend  ek-computation/src/ffn/mod.rs:17-53
+  HipLayer       the worker's ExpertDB for one layer (worker/manager.rs:14-88)
+                 plus the fused pack -> FFN -> combine call
+
+Everything here is plumbing: torch supplies buffers and streams, all
+arithmetic happens inside libek_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import Dict, Optional, Sequence
+
+import torch
+
+from . import _capi as C
+
+_DT = {torch.bfloat16: C.EK_BF16, torch.float16: C.EK_F16, torch.float32: C.EK_F32, torch.int8: C.EK_I8}
+
+
+def _mem(t: torch.Tensor) -> int:
+    return C.EK_DEVICE if t.is_cuda else C.EK_HOST
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream_ptr(stream) -> ctypes.c_void_p:
+    if stream is None:
+        return ctypes.c_void_p(0)
+    return ctypes.c_void_p(stream.cuda_stream if hasattr(stream, "cuda_stream") else int(stream))
+
+
+@dataclass
+class EKInstance:
+    hidden: int
+    intermediate: int
+    backend: str = "hip"
+
+
+@dataclass
+class ExpertWeight:
+    """up/gate [I,H], down [H,I]; *_scale: per-output-channel scales for int8."""
+    up_w: torch.Tensor
+    gate_w: torch.Tensor
+    down_w: torch.Tensor
+    up_scale: Optional[torch.Tensor] = None
+    gate_scale: Optional[torch.Tensor] = None
+    down_scale: Optional[torch.Tensor] = None
+
+    @staticmethod
+    def _lookup_suffix(tensors: Dict[str, torch.Tensor], suffixes: Sequence[str]):
+        for name in sorted(tensors):
+            if any(name.endswith(s) for s in suffixes):
+                return tensors[name]
+        return None
+
+    @classmethod
+    def from_safetensor(cls, tensors: Dict[str, torch.Tensor]) -> "ExpertWeight":
+        """Suffix lookup of ffn/meta.rs:56-75 (w1 = up, w2 = down, w3 = gate)."""
+        up = cls._lookup_suffix(tensors, ["w1.weight", "up_proj.weight"])
+        if up is None:
+            raise C.EKError(C.EK_WEIGHT_NOT_FOUND, "w1/up_w")
+        down = cls._lookup_suffix(tensors, ["w2.weight", "down_proj.weight"])
+        if down is None:
+            raise C.EKError(C.EK_WEIGHT_NOT_FOUND, "w2/down_w")
+        gate = cls._lookup_suffix(tensors, ["w3.weight", "gate_proj.weight"])
+        if gate is None:
+            raise C.EKError(C.EK_WEIGHT_NOT_FOUND, "w3/gate_w")
+        return cls(up_w=up, gate_w=gate, down_w=down,
+                   up_scale=cls._lookup_suffix(tensors, ["w1.weight_scale", "up_proj.weight_scale"]),
+                   gate_scale=cls._lookup_suffix(tensors, ["w3.weight_scale", "gate_proj.weight_scale"]),
+                   down_scale=cls._lookup_suffix(tensors, ["w2.weight_scale", "down_proj.weight_scale"]))
+
+    @classmethod
+    def from_rand_linear(cls, hidden: int, intermediate: int, dtype=torch.bfloat16, device="cpu"):
+        """ffn/meta.rs:77-89."""
+        return cls(up_w=torch.rand(intermediate, hidden, device=device).to(dtype),
+                   gate_w=torch.rand(intermediate, hidden, device=device).to(dtype),
+                   down_w=torch.rand(hidden, intermediate, device=device).to(dtype))
+
+
+def _desc(w: Optional[torch.Tensor], scale: Optional[torch.Tensor]):
+    """Builds an ek_weight_desc; returns (desc or None, keepalive)."""
+    if w is None:
+        return None, ()
+    w = w.contiguous()
+    d = C.ek_weight_desc()
+    d.ptr = w.data_ptr()
+    d.rows, d.cols = w.shape
+    d.dtype = _DT[w.dtype]
+    d.mem = _mem(w)
+    keep = [w]
+    if scale is not None:
+        scale = scale.contiguous()
+        if scale.is_cuda != w.is_cuda:
+            scale = scale.to(w.device)
+        d.scale = scale.data_ptr()
+        d.scale_dtype = _DT[scale.dtype]
+        d.scale_kind = C.EK_SCALE_PER_CHANNEL
+        keep.append(scale)
+    else:
+        d.scale = None
+        d.scale_dtype = C.EK_F32
+        d.scale_kind = C.EK_SCALE_NONE
+    return d, keep
+
+
+@dataclass
+class RouteTables:
+    counts: torch.Tensor
+    offsets: torch.Tensor
+    perm: torch.Tensor
+    inv_perm: torch.Tensor
+
+
+class HipLayer:
+    """The experts of one MoE layer, resident in HBM, with the fused layer call."""
+
+    def __init__(self, hidden: int, inter: int, n_experts: int, top_k: int, act_dtype=torch.bfloat16,
+                 w_dtype=None, max_tokens: int = 1024, device_id: int = 0):
+        self._lib = C.load()
+        self.cfg = C.ek_cfg(hidden=hidden, inter=inter, n_experts=n_experts, top_k=top_k,
+                            act_dtype=_DT[act_dtype], w_dtype=_DT[w_dtype or act_dtype],
+                            max_tokens=max_tokens, device_id=device_id, flags=0)
+        self.act_dtype = act_dtype
+        self._h = ctypes.c_void_p()
+        C.check(self._lib.ek_layer_create(ctypes.byref(self.cfg), ctypes.byref(self._h)))
+
+    # -- ExpertDB ---------------------------------------------------------
+    def set_expert(self, e: int, weight: ExpertWeight) -> None:
+        up, k1 = _desc(weight.up_w, weight.up_scale)
+        gate, k2 = _desc(weight.gate_w, weight.gate_scale)
+        down, k3 = _desc(weight.down_w, weight.down_scale)
+        ref = lambda d: ctypes.byref(d) if d is not None else None
+        C.check(self._lib.ek_layer_set_expert(self._h, e, ref(up), ref(gate), ref(down)))
+        del k1, k2, k3
+
+    def remove_expert(self, e: int) -> None:
+        C.check(self._lib.ek_layer_remove_expert(self._h, e))
+
+    def has_expert(self, e: int) -> bool:
+        out = ctypes.c_int32(0)
+        C.check(self._lib.ek_layer_has_expert(self._h, e, ctypes.byref(out)))
+        return bool(out.value)
+
+    # -- compute ----------------------------------------------------------
+    def _route(self, T: int, device):
+        E, K = self.cfg.n_experts, self.cfg.top_k
+        rt = RouteTables(torch.empty(E, dtype=torch.int32, device=device),
+                         torch.empty(E + 1, dtype=torch.int32, device=device),
+                         torch.empty(T * K, dtype=torch.int32, device=device),
+                         torch.empty(T * K, dtype=torch.int32, device=device))
+        ro = C.ek_route_out(rt.counts.data_ptr(), rt.offsets.data_ptr(), rt.perm.data_ptr(),
+                            rt.inv_perm.data_ptr())
+        return rt, ro
+
+    def forward(self, x: torch.Tensor, ids: torch.Tensor, w: torch.Tensor, return_route: bool = False,
+                stream=None, out: Optional[torch.Tensor] = None):
+        """y[T,H] = sum_k w[t,k] * expert_{ids[t,k]}(x[t]); see ek_layer_forward."""
+        assert x.dim() == 2 and ids.dim() == 2 and w.shape == ids.shape
+        x, ids, w = x.contiguous(), ids.contiguous(), w.contiguous()
+        assert ids.dtype == torch.int32 and x.dtype == self.act_dtype
+        assert x.is_cuda == ids.is_cuda == w.is_cuda
+        T = x.shape[0]
+        y = out if out is not None else torch.empty_like(x)
+        rt, ro = self._route(T, x.device) if return_route else (None, None)
+        C.check(self._lib.ek_layer_forward(self._h, _ptr(x), _ptr(ids), _ptr(w), _DT[w.dtype], T, _ptr(y),
+                                           ctypes.byref(ro) if ro is not None else None, _mem(x),
+                                           _stream_ptr(stream)))
+        return (y, rt) if return_route else y
+
+    def pack(self, ids: torch.Tensor, x: Optional[torch.Tensor] = None, stream=None):
+        """Routing tables (and the gathered rows Xp if x is given)."""
+        ids = ids.contiguous()
+        T = ids.shape[0]
+        rt, ro = self._route(T, ids.device)
+        xp = None
+        if x is not None:
+            x = x.contiguous()
+            xp = torch.empty(T * self.cfg.top_k, x.shape[1], dtype=x.dtype, device=x.device)
+        C.check(self._lib.ek_layer_pack(self._h, _ptr(ids), T, ctypes.byref(ro), _ptr(x), _ptr(xp),
+                                        _mem(ids), _stream_ptr(stream)))
+        return (rt, xp) if x is not None else rt
+
+    def expert_forward(self, e: int, x: torch.Tensor, stream=None) -> torch.Tensor:
+        assert x.dim() == 2, "input must be rank 2 (ffn/mod.rs:45)"
+        x = x.contiguous()
+        out = torch.empty_like(x)
+        C.check(self._lib.ek_layer_expert_forward(self._h, e, _ptr(x), x.shape[0], _ptr(out), _mem(x),
+                                                  _stream_ptr(stream)))
+        return out
+
+    def profile(self, enable: bool) -> None:
+        C.check(self._lib.ek_layer_profile(self._h, int(enable)))
+
+    def stats(self) -> dict:
+        s = C.ek_stats()
+        C.check(self._lib.ek_layer_get_stats(self._h, ctypes.byref(s)))
+        d = {f: getattr(s, f) for f, _ in s._fields_}
+        d["kernel_us"] = list(s.kernel_us)
+        return d
+
+    def close(self) -> None:
+        if getattr(self, "_h", None) is not None and self._h.value:
+            self._lib.ek_layer_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class HipFFN:
+    """One expert behind trait Expert<T> (ffn/meta.rs:30-39)."""
+
+    def __init__(self, handle, lib, instance: EKInstance, act_dtype, device: str):
+        self._h, self._lib, self._instance, self._act_dtype, self._device = handle, lib, instance, act_dtype, device
+
+    @classmethod
+    def construct(cls, x: EKInstance, weight: ExpertWeight, act_dtype=torch.bfloat16, max_rows: int = 4096,
+                  device_id: int = 0) -> "HipFFN":
+        lib = C.load()
+        w_dtype = torch.int8 if weight.up_w is not None and weight.up_w.dtype == torch.int8 else act_dtype
+        cfg = C.ek_cfg(hidden=x.hidden, inter=x.intermediate, n_experts=1, top_k=1, act_dtype=_DT[act_dtype],
+                       w_dtype=_DT[w_dtype], max_tokens=max_rows, device_id=device_id, flags=0)
+        up, k1 = _desc(weight.up_w, weight.up_scale)
+        gate, k2 = _desc(weight.gate_w, weight.gate_scale)
+        down, k3 = _desc(weight.down_w, weight.down_scale)
+        ref = lambda d: ctypes.byref(d) if d is not None else None
+        h = ctypes.c_void_p()
+        C.check(lib.ek_expert_create(ctypes.byref(cfg), max_rows, ref(up), ref(gate), ref(down), ctypes.byref(h)))
+        del k1, k2, k3
+        return cls(h, lib, x, act_dtype, f"cuda:{device_id}")
+
+    def backend(self) -> str:
+        return self._lib.ek_backend_name().decode()
+
+    def shape(self):
+        hidden, inter = ctypes.c_int64(), ctypes.c_int64()
+        C.check(self._lib.ek_expert_shape(self._h, ctypes.byref(hidden), ctypes.byref(inter)))
+        return hidden.value, inter.value
+
+    def rand_input(self, batch: int) -> torch.Tensor:
+        return torch.rand(batch, self._instance.hidden).to(self._act_dtype)
+
+    def forward(self, x: torch.Tensor, stream=None) -> torch.Tensor:
+        x = x.contiguous()
+        out = torch.empty_like(x)
+        C.check(self._lib.ek_expert_forward(self._h, _ptr(x), x.shape[0], _ptr(out), _mem(x), _stream_ptr(stream)))
+        return out
+
+    def close(self):
+        if getattr(self, "_h", None) is not None and self._h.value:
+            self._lib.ek_expert_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class ExpertBackend:
+    """enum ExpertBackend { Torch, OnnxF32 } + the new Hip variant (ffn/mod.rs:17-53)."""
+
+    def __init__(self, exp: HipFFN):
+        self.exp = exp
+
+    @classmethod
+    def build(cls, instance: EKInstance, tensors: Dict[str, torch.Tensor], **kw) -> "ExpertBackend":
+        if instance.backend != "hip":
+            raise NotImplementedError(f"backend {instance.backend!r} (x.rs:18-24 knows torch/ort; this library adds hip)")
+        weight = ExpertWeight.from_safetensor(tensors)
+        return cls(HipFFN.construct(instance, weight, **kw))
+
+    def forward(self, view: torch.Tensor) -> torch.Tensor:
+        assert view.dim() == 2  # ffn/mod.rs:45
+        return self.exp.forward(view)

@@ -1,0 +1,196 @@
+/*
+ * ek_hip.h -- C ABI of libek_hip.so, an MI355X (gfx950) expert-computation
+ * backend for Expert Kit.
+ *
+ * The reference has no FFI on this path: the seam is the Rust trait
+ * `Expert<T>` (ek-computation/src/ffn/meta.rs:30-39), the dispatch enum
+ * `ExpertBackend` (ek-computation/src/ffn/mod.rs:17-53) and the worker's
+ * registry `ExpertDB` (ek-computation/src/worker/manager.rs:14-88).  Every
+ * entry point below names the reference item it stands behind, so that a Rust
+ * `HipFFN` can implement the trait with `extern "C"` calls only.
+ *
+ * Conventions
+ *  - plain C types only; handles are opaque and never dereferenced by callers;
+ *  - every function returns ek_status and never throws, aborts or unwinds;
+ *    ek_last_error() gives a thread-local message for the last failure;
+ *  - tensors are row-major and contiguous; `mem` says whether the pointers of
+ *    a call are host (EK_HOST) or device (EK_DEVICE) addresses;
+ *  - the caller owns every input/output buffer, the library owns weights and
+ *    workspace; weight bytes are copied (and re-tiled) by set_expert, so the
+ *    source buffer may be released as soon as the call returns;
+ *  - `stream` is a hipStream_t passed as void*.  NULL means "run on the
+ *    library's own stream and return after the work has completed".  With a
+ *    non-NULL stream and device pointers the call only enqueues work;
+ *  - all entry points may be called from any thread.  Calls that use the same
+ *    layer's workspace are serialised internally.
+ */
+#ifndef EK_HIP_H
+#define EK_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Mirrors the variants of EKError that this path can raise
+ * (ek-base/src/error.rs:12-72). */
+typedef enum ek_status {
+    EK_OK = 0,
+    EK_INVALID_INPUT = 1,    /* EKError::InvalidInput: bad shape / dtype / pointer / id */
+    EK_EXPERT_NOT_FOUND = 2, /* EKError::ExpertNotFound: pair routed to an unloaded expert */
+    EK_WEIGHT_NOT_FOUND = 3, /* EKError::ExpertWeightNotFound: missing up/gate/down or scale */
+    EK_OOM = 4,              /* device or host allocation failed */
+    EK_HIP_ERROR = 5,        /* a HIP runtime call failed */
+    EK_INTERNAL = 6          /* anything else (caught exception, broken invariant) */
+} ek_status;
+
+/* Element types (ek-computation/src/backend/mod.rs:7-16 and
+ * backend/torch/tch_safetensors.rs:12-46 list the reference's). */
+typedef enum ek_dtype { EK_BF16 = 0, EK_F16 = 1, EK_F32 = 2, EK_I8 = 3 } ek_dtype;
+
+typedef enum ek_mem { EK_HOST = 0, EK_DEVICE = 1 } ek_mem;
+
+typedef enum ek_scale_kind {
+    EK_SCALE_NONE = 0,
+    EK_SCALE_PER_CHANNEL = 1 /* one scale per output row: W[n,:] = q[n,:] * scale[n] */
+} ek_scale_kind;
+
+/* Stands for EKInstance{hidden, intermediate, backend} (ek-computation/src/x.rs:27-32)
+ * plus the inference settings it is filled from (ek-base/src/config.rs:26-31). */
+typedef struct ek_cfg {
+    int64_t hidden;     /* H */
+    int64_t inter;      /* I  (moe_intermediate_size) */
+    int32_t n_experts;  /* E  experts owned by one layer object */
+    int32_t top_k;      /* K  slots per token */
+    int32_t act_dtype;  /* ek_dtype of x, y and the gate weights: EK_BF16 or EK_F16 */
+    int32_t w_dtype;    /* ek_dtype weights are kept in: act_dtype, or EK_I8 (W8A16) */
+    int64_t max_tokens; /* largest T a forward call will pass */
+    int32_t device_id;  /* HIP device ordinal */
+    int32_t flags;      /* reserved, 0 */
+} ek_cfg;
+
+/* One weight matrix of ExpertWeight<T> (ek-computation/src/ffn/meta.rs:10-23),
+ * row-major [rows = out_features, cols = in_features] as HF nn.Linear stores
+ * it.  For EK_I8 weights `scale` holds `rows` per-output-channel scales. */
+typedef struct ek_weight_desc {
+    const void *ptr;
+    int64_t rows;
+    int64_t cols;
+    int32_t dtype;       /* EK_BF16 / EK_F16 / EK_F32 (cast on load, as
+                            TorchFFN::load_module does, ffn/expert_torch.rs:61-78) or EK_I8 */
+    int32_t mem;         /* ek_mem of ptr and scale */
+    const void *scale;   /* NULL unless scale_kind != EK_SCALE_NONE */
+    int32_t scale_dtype; /* EK_BF16 or EK_F32 */
+    int32_t scale_kind;  /* ek_scale_kind */
+} ek_weight_desc;
+
+/* Optional routing tables of a forward call: the dense form of
+ * NaiveExecutor::pending_egress (ek-computation/src/controller/executor.rs:54,283-299).
+ * Any pointer may be NULL.  Memory space = the call's `mem`. */
+typedef struct ek_route_out {
+    int32_t *counts;   /* [E]   pairs per expert */
+    int32_t *offsets;  /* [E+1] exclusive scan of counts */
+    int32_t *perm;     /* [T*K] packed position -> flat pair index t*K+k */
+    int32_t *inv_perm; /* [T*K] flat pair index -> packed position */
+} ek_route_out;
+
+/* Counters the worker shell feeds into its Prometheus series
+ * (ek-computation/src/metrics.rs:47-71; worker/server.rs:39-63). */
+typedef struct ek_stats {
+    int64_t forward_calls;
+    int64_t tokens;
+    int64_t pairs;
+    int64_t expert_forward_calls;
+    double last_forward_us; /* host wall time of the last blocking forward */
+    /* filled only while profiling is on (ek_layer_profile): device time between
+     * HIP events recorded around the four phases of ek_layer_forward, summed
+     * over profiled_calls calls.  [0] pack, [1] up/gate + SwiGLU, [2] down, [3] combine */
+    double kernel_us[4];
+    int64_t profiled_calls;
+} ek_stats;
+
+typedef struct ek_layer ek_layer;
+typedef struct ek_expert ek_expert;
+
+/* Expert::backend() (ffn/meta.rs:34): returns "hip". */
+const char *ek_backend_name(void);
+
+/* Thread-local text of the last error raised on the calling thread. */
+const char *ek_last_error(void);
+
+/* Number of visible HIP devices (0 if none); never fails. */
+int32_t ek_device_count(void);
+
+/* ---- layer object: the E experts of one MoE layer, resident in HBM --------
+ * Stands for the worker's ExpertDB (worker/manager.rs:14-88) restricted to one
+ * layer: insert = set_expert, remove = remove_expert, has/loaded = has_expert. */
+ek_status ek_layer_create(const ek_cfg *cfg, ek_layer **out);
+ek_status ek_layer_destroy(ek_layer *layer);
+
+/* ExpertDB::insert after ExpertBackend::build (ffn/mod.rs:23-36;
+ * worker/x.rs:13-34): copies the three matrices to HBM in the kernels' tiled
+ * layout, casting to cfg.w_dtype.  Shapes must be up,gate [I,H], down [H,I].
+ * A NULL descriptor or NULL data pointer gives EK_WEIGHT_NOT_FOUND
+ * (ExpertWeight::from_safetensor, ffn/meta.rs:56-75). */
+ek_status ek_layer_set_expert(ek_layer *layer, int32_t expert, const ek_weight_desc *up,
+                              const ek_weight_desc *gate, const ek_weight_desc *down);
+
+/* ExpertDB::remove (worker/manager.rs:69-72). */
+ek_status ek_layer_remove_expert(ek_layer *layer, int32_t expert);
+
+/* ExpertDB::has (worker/manager.rs:52-55): *loaded = 1 or 0. */
+ek_status ek_layer_has_expert(ek_layer *layer, int32_t expert, int32_t *loaded);
+
+/* Whole layer in one call: what today is spread over
+ * break_down_to_egress + assemble_seq_tensors (controller/executor.rs:283-299,112-133),
+ * one EKInstanceGate::forward per expert (worker/core.rs:47-74 ->
+ * ffn/expert_torch.rs:80-85), the collection loop + output
+ * (controller/executor.rs:203-252) and the weighted sum (qwen3_moe.py:102-104).
+ *   x   [T,H] act_dtype        ids [T,K] int32 in [0,E)
+ *   w   [T,K] w_dtype: act_dtype (Qwen3 shim) or EK_F32 (DeepSeek shim)
+ *   y   [T,H] act_dtype        route: optional routing tables (may be NULL)
+ * T == 0 is legal and does nothing.  An id outside [0,E) gives
+ * EK_INVALID_INPUT, a pair routed to an unloaded expert EK_EXPERT_NOT_FOUND
+ * (both reported by blocking calls; y is then unspecified). */
+ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, const void *w,
+                           int32_t w_dtype, int64_t T, void *y, const ek_route_out *route,
+                           int32_t mem, void *stream);
+
+/* Routing only: the pack step of ek_layer_forward, plus (if xp != NULL) the
+ * gather Xp[j,:] = x[perm[j]/K,:] of assemble_seq_tensors
+ * (controller/executor.rs:112-133).  x may be NULL when xp is NULL. */
+ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek_route_out *route,
+                        const void *x, void *xp, int32_t mem, void *stream);
+
+/* One expert, one call: ExpertBackend::forward -> Expert::forward
+ * (ffn/mod.rs:39-53; ffn/meta.rs:37) as EKInstanceGate::forward uses it
+ * (worker/core.rs:55-59).  x [n,H] -> out [n,H], both act_dtype.  n may
+ * exceed cfg.max_tokens * top_k only if it still fits the workspace. */
+ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x, int64_t n,
+                                  void *out, int32_t mem, void *stream);
+
+/* Turns per-phase HIP-event timing of ek_layer_forward on (1) or off (0) and
+ * clears the accumulated kernel_us.  Stands for the PerfTimer checkpoints of
+ * the reference (ek-base/src/utils.rs:4-45; controller/executor.rs:136,201,228).
+ * At most 1024 calls are recorded between two ek_layer_get_stats calls. */
+ek_status ek_layer_profile(ek_layer *layer, int32_t enable);
+
+/* Snapshot of the layer's counters (waits for recorded events to complete). */
+ek_status ek_layer_get_stats(ek_layer *layer, ek_stats *out);
+
+/* ---- single expert object: the literal shape of trait Expert<T> ----------
+ * construct (ffn/meta.rs:38), forward (:37), shape (:35).  Implemented as a
+ * one-expert layer; max_rows bounds n of forward. */
+ek_status ek_expert_create(const ek_cfg *cfg, int64_t max_rows, const ek_weight_desc *up,
+                           const ek_weight_desc *gate, const ek_weight_desc *down,
+                           ek_expert **out);
+ek_status ek_expert_forward(ek_expert *expert, const void *x, int64_t n, void *out, int32_t mem,
+                            void *stream);
+ek_status ek_expert_shape(ek_expert *expert, int64_t *hidden, int64_t *inter);
+ek_status ek_expert_destroy(ek_expert *expert);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EK_HIP_H */

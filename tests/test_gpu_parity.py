@@ -1,0 +1,257 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI.
+
+Bars: routing tables and the gather are bit-exact; FFN / layer outputs satisfy
+max|y - y_ref| <= 2e-2 * rms(y_ref), y_ref = the oracle's reference-rounded
+form (fp32-equivalent accumulation, storage rounding after every op).
+"""
+import pytest
+import torch
+
+from ek_hip import workloads as wl
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+
+
+def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
+    ref = ref.float()
+    rms = float(ref.pow(2).mean().sqrt())
+    return float((got.float().cpu() - ref).abs().max()) / max(rms, 1e-30)
+
+
+def load_layer(ek, w: wl.Workload, experts=None, max_tokens=None, device="cpu"):
+    layer = ek.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype,
+                        w_dtype=torch.int8 if w.w8 else w.act_dtype, max_tokens=max_tokens or max(w.tokens, 1))
+    ws = {}
+    for e in (range(w.n_experts) if experts is None else experts):
+        ws[e] = wl.make_expert(w, e, device=device)
+        layer.set_expert(e, ws[e])
+    return layer, ws
+
+
+def oracle_weights(oracle, ws, E):
+    wu, wg, wd = [None] * E, [None] * E, [None] * E
+    for e, ew in ws.items():
+        if ew.up_w.dtype == torch.int8:
+            wu[e] = oracle.dequant_channel(ew.up_w.cpu(), ew.up_scale.cpu())
+            wg[e] = oracle.dequant_channel(ew.gate_w.cpu(), ew.gate_scale.cpu())
+            wd[e] = oracle.dequant_channel(ew.down_w.cpu(), ew.down_scale.cpu())
+        else:
+            wu[e], wg[e], wd[e] = ew.up_w.cpu(), ew.gate_w.cpu(), ew.down_w.cpu()
+    return wu, wg, wd
+
+
+# ----------------------------------------------------------------- routing
+
+PACK_CASES = [(0, 2, 16), (1, 1, 1), (1, 8, 256), (63, 1, 3), (64, 2, 16), (65, 3, 5), (128, 8, 256), (256, 8, 128),
+              (511, 8, 128), (513, 8, 1000), (4099, 2, 33), (8192, 8, 256)]
+
+
+@pytest.mark.parametrize("T,K,E", PACK_CASES)
+def test_pack_bit_exact(ek, oracle, cuda, T, K, E):
+    print(f"pack T={T} K={K} E={E}", flush=True)
+    g = torch.Generator().manual_seed(T * 7919 + K * 31 + E)
+    ids = torch.randint(0, E, (T, K), generator=g, dtype=torch.int32)
+    if T > 100:                                   # skew: half the pairs to a few hot experts
+        hot = torch.randint(0, min(E, 3), (T, K), generator=g, dtype=torch.int32)
+        ids = torch.where(torch.rand(T, K, generator=g) < 0.5, hot, ids)
+    layer = ek.HipLayer(64, 64, E, K, max_tokens=max(T, 1))
+    rt = layer.pack(ids.to(cuda))
+    ref = oracle.pack(ids, E)
+    for name, a, b in zip(("counts", "offsets", "perm", "inv_perm"), (rt.counts, rt.offsets, rt.perm, rt.inv_perm), ref):
+        assert torch.equal(a.cpu(), b), name
+    # host-memory call gives the same tables
+    rt_h = layer.pack(ids)
+    assert torch.equal(rt_h.perm, ref[2]) and torch.equal(rt_h.offsets, ref[1])
+    layer.close()
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_pack_benchmark_routing(ek, oracle, cuda, name):
+    w = wl.resolve(wl.CONFIGS[name])
+    print(f"pack {w.name} T={w.tokens}", flush=True)
+    ids, _ = wl.make_routing(w)
+    layer = ek.HipLayer(64, 64, w.n_experts, w.top_k, max_tokens=w.tokens)
+    rt = layer.pack(ids.to(cuda))
+    ref = oracle.pack(ids, w.n_experts)
+    for a, b in zip((rt.counts, rt.offsets, rt.perm, rt.inv_perm), ref):
+        assert torch.equal(a.cpu(), b)
+    layer.close()
+
+
+def test_gather_bit_exact(ek, oracle, cuda):
+    g = torch.Generator().manual_seed(5)
+    T, K, E, H = 300, 4, 20, 128
+    ids = torch.randint(0, E, (T, K), generator=g, dtype=torch.int32)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    layer = ek.HipLayer(H, 64, E, K, max_tokens=T)
+    rt, xp = layer.pack(ids.to(cuda), x.to(cuda))
+    ref = oracle.gather(x, oracle.pack(ids, E)[2], K)
+    assert torch.equal(xp.cpu().view(torch.int16), ref.view(torch.int16))
+    rt_h, xp_h = layer.pack(ids, x)
+    assert torch.equal(xp_h.view(torch.int16), ref.view(torch.int16))
+    layer.close()
+
+
+# ------------------------------------------------------------ one expert
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w8", [False, True])
+@pytest.mark.parametrize("n", [1, 5, 16, 17, 40])
+def test_expert_forward(ek, oracle, cuda, dt, w8, n):
+    print(f"expert_forward dt={dt} w8={w8} n={n}", flush=True)
+    w = wl.Workload("t", 256, 192, 1, 1, n, dt, w8=w8)
+    ew = wl.make_expert(w, 0)
+    if not w8:   # larger weights than the benchmark's so that silu is exercised off its linear part
+        ew = ek.ExpertWeight(ew.up_w * 4, ew.gate_w * 4, ew.down_w * 4)
+    ffn = ek.HipFFN.construct(ek.EKInstance(w.hidden, w.inter), ew, act_dtype=dt, max_rows=64)
+    assert ffn.backend() == "hip" and ffn.shape() == (256, 192)
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(n, w.hidden, generator=g).to(dt)
+    wu, wg, wd = oracle_weights(oracle, {0: ew}, 1)
+    if w8 and dt == torch.float16:
+        wu, wg, wd = wu[0].to(dt), wg[0].to(dt), wd[0].to(dt)
+    else:
+        wu, wg, wd = wu[0], wg[0], wd[0]
+    ref = oracle.ffn(x, wu, wg, wd, mode=0)
+    got_dev = ffn.forward(x.to(cuda))
+    got_host = ffn.forward(x)
+    assert rel_err(got_dev, ref) <= TOL, rel_err(got_dev, ref)
+    assert torch.equal(got_dev.cpu().view(torch.int16), got_host.view(torch.int16))
+    ffn.close()
+
+
+def test_expert_forward_special_cases(ek, cuda):
+    w = wl.Workload("t", 128, 64, 1, 1, 8, torch.bfloat16)
+    ew = wl.make_expert(w, 0)
+    ffn = ek.HipFFN.construct(ek.EKInstance(128, 64), ew, max_rows=32)
+    x = torch.randn(8, 128).to(torch.bfloat16)
+    assert not ffn.forward(torch.zeros_like(x).to(cuda)).float().any()
+    full = ffn.forward(x.to(cuda)).cpu()
+    for r in (0, 3, 7):                                   # rows are independent; batching changes nothing
+        one = ffn.forward(x[r:r + 1].to(cuda)).cpu()
+        assert torch.equal(one.view(torch.int16), full[r:r + 1].view(torch.int16))
+    assert ffn.forward(x[:0].to(cuda)).shape == (0, 128)  # empty batch
+    zg = ek.HipFFN.construct(ek.EKInstance(128, 64), ek.ExpertWeight(ew.up_w, torch.zeros_like(ew.gate_w), ew.down_w))
+    assert not zg.forward(x.to(cuda)).float().any()       # silu(0) = 0
+    ffn.close(); zg.close()
+
+
+# ------------------------------------------------------------ whole layer
+
+def run_layer_parity(ek, oracle, cuda, w, w_f32=False):
+    w = wl.resolve(w)
+    layer, ws = load_layer(ek, w)
+    x = wl.make_x(w)
+    ids, gw = wl.make_routing(w)
+    if w_f32:
+        gw = gw.float()
+    y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
+    wu, wg, wd = oracle_weights(oracle, ws, w.n_experts)
+    ref, counts, offsets, perm, inv = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=0)
+    for a, b in zip((rt.counts, rt.offsets, rt.perm, rt.inv_perm), (counts, offsets, perm, inv)):
+        assert torch.equal(a.cpu(), b)
+    err = rel_err(y, ref)
+    print(f"{w.name}: max|err|/rms = {err:.3e}", flush=True)
+    assert err <= TOL
+    y_host = layer.forward(x, ids, gw)
+    assert torch.equal(y_host.view(torch.int16), y.cpu().view(torch.int16))
+    st = layer.stats()
+    assert st["forward_calls"] == 2 and st["pairs"] == 2 * w.pairs
+    layer.close()
+    return err
+
+
+def test_layer_c1(ek, oracle, cuda):
+    run_layer_parity(ek, oracle, cuda, wl.C1)
+
+
+def test_layer_c1_fp32_gate_weights(ek, oracle, cuda):
+    run_layer_parity(ek, oracle, cuda, wl.C1, w_f32=True)
+
+
+def test_layer_small_fp16_skewed(ek, oracle, cuda):
+    run_layer_parity(ek, oracle, cuda, wl.Workload("qwen3ish_small", 512, 192, 32, 8, 96, torch.float16, zipf_s=1.0))
+
+
+def test_layer_small_w8(ek, oracle, cuda):
+    run_layer_parity(ek, oracle, cuda, wl.Workload("dsv3ish_small", 512, 256, 32, 4, 70, torch.bfloat16, w8=True, zipf_s=0.8))
+
+
+def test_layer_ragged_lengths(ek, oracle, cuda):
+    """Segment lengths from 0 to a few hundred in one call (hot expert + empty experts)."""
+    w = wl.Workload("ragged", 256, 128, 24, 2, 400, torch.bfloat16, zipf_s=2.0)
+    run_layer_parity(ek, oracle, cuda, w)
+
+
+def test_layer_c3_sampled(ek, oracle, cuda):
+    """Full DeepSeek-V3 decode shape; weights drawn on the GPU, a sample of experts
+    is copied back and their rows are checked against the oracle via K=8 combine of
+    reference rows for tokens fully covered by the sample... here: the per-expert
+    rows themselves, through ek_layer_expert_forward, plus the routing tables."""
+    w = wl.C3
+    sample = [0, 37, 101, 255]
+    layer, ws = load_layer(ek, w, experts=sample, device="cuda")
+    x = wl.make_x(w)
+    ids, gw = wl.make_routing(w)
+    ref_rt = oracle.pack(ids, w.n_experts)
+    rt = layer.pack(ids.to(cuda))
+    for a, b in zip((rt.counts, rt.offsets, rt.perm, rt.inv_perm), ref_rt):
+        assert torch.equal(a.cpu(), b)
+    for e in sample:
+        n = int(ref_rt[0][e])
+        rows = (ref_rt[2][int(ref_rt[1][e]):int(ref_rt[1][e + 1])] // w.top_k).long()
+        xe = x[rows] if n else x[:3]
+        got = layer.expert_forward(e, xe.to(cuda))
+        wu, wg, wd = oracle_weights(oracle, {e: ws[e]}, w.n_experts)
+        ref = oracle.ffn(xe, wu[e], wg[e], wd[e], mode=0)
+        err = rel_err(got, ref)
+        print(f"c3 expert {e}: rows={xe.shape[0]} max|err|/rms = {err:.3e}", flush=True)
+        assert err <= TOL
+    layer.close()
+
+
+# ------------------------------------------------------------ error paths
+
+def test_error_paths(ek, cuda):
+    from ek_hip import _capi as C
+    w = wl.Workload("t", 128, 64, 8, 2, 16, torch.bfloat16)
+    layer, ws = load_layer(ek, w, experts=[0, 1, 2, 3])
+    x = torch.randn(16, 128).to(torch.bfloat16).to(cuda)
+    gw = torch.full((16, 2), 0.5).to(torch.bfloat16).to(cuda)
+    ok_ids = torch.tensor([[0, 1]] * 16, dtype=torch.int32, device=cuda)
+    layer.forward(x, ok_ids, gw)
+    with pytest.raises(ek.EKError) as ei:                       # pair routed to an unloaded expert
+        layer.forward(x, torch.tensor([[0, 7]] * 16, dtype=torch.int32, device=cuda), gw)
+    assert ei.value.status == C.EK_EXPERT_NOT_FOUND
+    for bad in (8, -1, 1 << 20):                                # id outside [0, E)
+        with pytest.raises(ek.EKError) as ei:
+            layer.forward(x, torch.tensor([[0, bad]] * 16, dtype=torch.int32, device=cuda), gw)
+        assert ei.value.status == C.EK_INVALID_INPUT
+    with pytest.raises(ek.EKError) as ei:                       # T > max_tokens
+        layer.forward(torch.cat([x, x]), torch.cat([ok_ids, ok_ids]), torch.cat([gw, gw]))
+    assert ei.value.status == C.EK_INVALID_INPUT
+    with pytest.raises(ek.EKError) as ei:
+        layer.expert_forward(5, x)
+    assert ei.value.status == C.EK_EXPERT_NOT_FOUND
+    with pytest.raises(ek.EKError) as ei:                       # wrong weight shape
+        layer.set_expert(4, ek.ExpertWeight(ws[0].up_w[:32], ws[0].gate_w, ws[0].down_w))
+    assert ei.value.status == C.EK_INVALID_INPUT
+    with pytest.raises(ek.EKError) as ei:                       # missing matrix
+        layer.set_expert(4, ek.ExpertWeight(None, ws[0].gate_w, ws[0].down_w))
+    assert ei.value.status == C.EK_WEIGHT_NOT_FOUND
+    # registry semantics
+    assert layer.has_expert(0) and not layer.has_expert(4)
+    layer.remove_expert(0)
+    assert not layer.has_expert(0)
+    with pytest.raises(ek.EKError):
+        layer.remove_expert(0)
+    with pytest.raises(ek.EKError) as ei:
+        layer.forward(x, ok_ids, gw)
+    assert ei.value.status == C.EK_EXPERT_NOT_FOUND
+    layer.set_expert(0, ws[0])                                  # reload, then the call works again
+    y = layer.forward(x, ok_ids, gw)
+    assert y.shape == x.shape
+    assert layer.forward(x[:0], ok_ids[:0], gw[:0]).shape == (0, 128)   # T = 0
+    layer.close()
+    layer.close()                                               # idempotent
