@@ -282,6 +282,10 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
         L->st_raw_bytes = need;
     }
 
+    // device-resident sources may still be being written on the caller's streams
+    if (up->mem == EK_DEVICE || gate->mem == EK_DEVICE || down->mem == EK_DEVICE)
+        EK_HIP(hipDeviceSynchronize());
+
     void *mem = nullptr;
     EK_TRY(dev_alloc(&mem, total, "expert weights"));
     uint8_t *base = (uint8_t *)mem;
@@ -575,6 +579,8 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
         std::lock_guard<std::mutex> lk(layer->mu);
         hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
         ek_status st = EK_OK;
+        // a blocking call on device buffers sees everything submitted before it
+        if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
         if (mem == EK_DEVICE) {
             EK_TRY(enqueue_forward(layer, x, ids, w, w_f32, T, y, s));
             EK_TRY(copy_route_out(layer, route, P, mem, s));
@@ -621,6 +627,7 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
         const int64_t H = layer->cfg.hidden, K = layer->cfg.top_k, P = T * K;
         std::lock_guard<std::mutex> lk(layer->mu);
         hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+        if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
         const int32_t *d_ids = ids;
         const void *d_x = x;
         void *d_xp = xp;
@@ -667,6 +674,7 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
         if (!layer->expert_mem[expert])
             return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", expert);
         hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+        if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
         if (n > 0) {
             const void *d_x = x;
             void *d_out = out;

@@ -15,10 +15,12 @@
 //   - the <= 16 activation rows of the segment are the "B" operand (32 k x 16
 //     rows), re-read from L2 by every wave;
 //   - D loads deep software prefetch keeps >= D KiB per wave in flight.
-// int8 weights are stored offset-binary (q + 128): v_cvt_f32_ubyteN +
-// v_cvt_pk_bf16_f32 turn 4 bytes into 4 exact bf16 integers, one extra MFMA
-// against an all-ones A operand accumulates sum_k x[k], and the epilogue
-// forms (acc - 128 * sum_x) * scale[channel].
+// int8 weights are dequantised in registers to exactly the tensor a CPU backend
+// would hold, W[n,k] = rne_16bit(f32(q[n,k]) * f32(scale[n])): they are stored
+// offset-binary (u = q + 128) so v_cvt_f32_ubyteN converts them, one
+// fma(u, s, -128 s) per element gives the exact fp32 product q*s (16
+// significant bits), and v_cvt_pk_bf16_f32 rounds two of them to nearest even.
+// Each lane owns one output channel of the A operand, so s is a lane scalar.
 #include "ek_internal.h"
 
 namespace ek {
@@ -45,19 +47,20 @@ template <> struct Act<_Float16> {
 
 template <typename T> __device__ __forceinline__ float rnd(float v) { return (float)(T)v; }
 
-// 8 offset-binary bytes (two dwords) -> 8 exact integers in T
+// 8 offset-binary bytes (two dwords) of one output channel -> 8 dequantised
+// weights rne_T((u - 128) * s); c = -128 * s
 template <typename T>
-__device__ __forceinline__ typename Act<T>::V8 cvt_u8x8(uint32_t lo, uint32_t hi)
+__device__ __forceinline__ typename Act<T>::V8 dequant_u8x8(uint32_t lo, uint32_t hi, float s, float c)
 {
     typename Act<T>::V8 r;
-    r[0] = (T)(float)(lo & 0xffu);
-    r[1] = (T)(float)((lo >> 8) & 0xffu);
-    r[2] = (T)(float)((lo >> 16) & 0xffu);
-    r[3] = (T)(float)(lo >> 24);
-    r[4] = (T)(float)(hi & 0xffu);
-    r[5] = (T)(float)((hi >> 8) & 0xffu);
-    r[6] = (T)(float)((hi >> 16) & 0xffu);
-    r[7] = (T)(float)(hi >> 24);
+    r[0] = (T)__builtin_fmaf((float)(lo & 0xffu), s, c);
+    r[1] = (T)__builtin_fmaf((float)((lo >> 8) & 0xffu), s, c);
+    r[2] = (T)__builtin_fmaf((float)((lo >> 16) & 0xffu), s, c);
+    r[3] = (T)__builtin_fmaf((float)(lo >> 24), s, c);
+    r[4] = (T)__builtin_fmaf((float)(hi & 0xffu), s, c);
+    r[5] = (T)__builtin_fmaf((float)((hi >> 8) & 0xffu), s, c);
+    r[6] = (T)__builtin_fmaf((float)((hi >> 16) & 0xffu), s, c);
+    r[7] = (T)__builtin_fmaf((float)(hi >> 24), s, c);
     return r;
 }
 
@@ -93,9 +96,20 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
     for (int gi = 0; gi < NG; ++gi)
         wp[gi] = wmat + (int64_t)(nt0 + gi) * KT * (NMAT * kChunkBytes) + lane * 16;
 
-    V8 ones;
+    // per-lane dequantisation constants: the lane's channel of each A operand
+    float ws[NW], wc[NW];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) ones[i] = (T)1.0f;
+    for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+        for (int m = 0; m < NMAT; ++m) {
+            float sv = 1.f;
+            if constexpr (W8) {
+                const int ch = (nt0 + gi) * 16 + j;
+                sv = NMAT == 2 ? (m == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
+            }
+            ws[gi * NMAT + m] = sv;
+            wc[gi * NMAT + m] = -128.f * sv;
+        }
 
     for (int r0 = 0; r0 < n; r0 += 16) {
         const int jr = min(r0 + j, n - 1);   // lanes past the segment re-read its last row
@@ -103,7 +117,6 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
         const T *xp = (const T *)a.x + row * a.x_stride + g * (KE / 4);
 
         f32x4 acc[NMAT][NG];
-        f32x4 accs = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int m = 0; m < NMAT; ++m)
 #pragma unroll
@@ -131,15 +144,14 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
                 if constexpr (W8) {
                     const V8 x0 = __builtin_bit_cast(V8, xq[d][0]);
                     const V8 x1 = __builtin_bit_cast(V8, xq[d][1]);
-                    accs = Act<T>::mfma(ones, x0, accs);
-                    accs = Act<T>::mfma(ones, x1, accs);
 #pragma unroll
                     for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
                         for (int m = 0; m < NMAT; ++m) {
                             const uint4 q = wq[d][gi * NMAT + m];
-                            acc[m][gi] = Act<T>::mfma(cvt_u8x8<T>(q.x, q.y), x0, acc[m][gi]);
-                            acc[m][gi] = Act<T>::mfma(cvt_u8x8<T>(q.z, q.w), x1, acc[m][gi]);
+                            const float sv = ws[gi * NMAT + m], cv = wc[gi * NMAT + m];
+                            acc[m][gi] = Act<T>::mfma(dequant_u8x8<T>(q.x, q.y, sv, cv), x0, acc[m][gi]);
+                            acc[m][gi] = Act<T>::mfma(dequant_u8x8<T>(q.z, q.w, sv, cv), x1, acc[m][gi]);
                         }
                 } else {
                     const V8 x0 = __builtin_bit_cast(V8, xq[d][0]);
@@ -176,19 +188,12 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     if constexpr (NMAT == 2) {
-                        float up = acc[0][gi][r], gate = acc[1][gi][r];
-                        if constexpr (W8) {
-                            up = (up - 128.f * accs[r]) * slab.s_up[ch + r];
-                            gate = (gate - 128.f * accs[r]) * slab.s_gate[ch + r];
-                        }
-                        up = rnd<T>(up);
-                        gate = rnd<T>(gate);
+                        const float up = rnd<T>(acc[0][gi][r]);
+                        const float gate = rnd<T>(acc[1][gi][r]);
                         const float sg = rnd<T>(gate / (1.0f + expf(-gate)));
                         o[r] = (T)(up * sg);
                     } else {
-                        float v = acc[0][gi][r];
-                        if constexpr (W8) v = (v - 128.f * accs[r]) * slab.s_down[ch + r];
-                        o[r] = (T)v;
+                        o[r] = (T)acc[0][gi][r];
                     }
                 }
                 *(uint2 *)(orow + ch) = __builtin_bit_cast(uint2, o);

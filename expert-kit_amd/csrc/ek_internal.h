@@ -16,7 +16,8 @@ namespace ek {
 // (up and gate are one group, so one wave streams one contiguous range):
 //   byte offset of chunk (nt, kt, m) = ((nt*KT + kt)*NMAT + m) * 1024.
 // int8 values are stored offset-binary (q + 128, i.e. q ^ 0x80) so that
-// v_cvt_f32_ubyte* converts them; the kernels subtract 128 * sum_k x[k].
+// v_cvt_f32_ubyte* converts them; the kernels fold the -128 into the
+// dequantisation fma.
 constexpr int kChunkBytes = 1024;
 
 struct ExpertSlab {           // device addresses of one expert's tensors

@@ -139,14 +139,12 @@ int eko_router_softmax_topk(const float *logits, int64_t T, int E, int K, int re
         for (int e = 0; e < E; ++e) p[e] = p[e] / s;
         memset(used, 0, (size_t)E);
         float ws = 0.f;
-        float top[64];
         for (int k = 0; k < K; ++k) {
             int best = -1;
             for (int e = 0; e < E; ++e)
                 if (!used[e] && (best < 0 || p[e] > p[best])) best = e;
             used[best] = 1;
             ids[t * K + k] = best;
-            top[k < 64 ? k : 63] = p[best];
             ws += p[best];
         }
         for (int k = 0; k < K; ++k) {
@@ -154,7 +152,6 @@ int eko_router_softmax_topk(const float *logits, int64_t T, int E, int K, int re
             if (renorm) v = v / ws;
             store_act(w, t * K + k, v, w_dt);
         }
-        (void)top;
     }
     free(p); free(used);
     return 0;
@@ -243,18 +240,19 @@ void eko_scatter(const void *yp, int64_t H, int elem_size, const int32_t *perm, 
 /* --------------------------------------------------------------- dequant */
 
 /*
- * Per-output-channel W8A16 dequantisation (the BASELINE definition):
- * W[n,c] = bf16( f32(q[n,c]) * f32(scale[n]) ), scale given as bf16 bits.
+ * Per-output-channel W8A16 dequantisation (the benchmark's definition):
+ * W[n,c] = rne_dt( f32(q[n,c]) * f32(scale[n]) ), scale given as bf16 bits,
+ * dt = bf16 (the definition) or fp16 (its analogue for fp16 activations).
  * The product of an int8 and a bf16 has at most 15 significant bits, so it is
  * exact in fp32 and the only rounding is the final one.
  */
 void eko_dequant_channel(const int8_t *q, const uint16_t *scale_bf16, int64_t N, int64_t C,
-                         uint16_t *w_bf16)
+                         int dt, uint16_t *w)
 {
     for (int64_t n = 0; n < N; ++n) {
         float s = bf16_to_f32(scale_bf16[n]);
         for (int64_t c = 0; c < C; ++c)
-            w_bf16[n * C + c] = f32_to_bf16((float)q[n * C + c] * s);
+            store_act(w, n * C + c, (float)q[n * C + c] * s, dt);
     }
 }
 
@@ -297,10 +295,15 @@ static inline double silu_d(double v) { return v / (1.0 + exp(-v)); }
  * the rounded gate.
  * mode 1 ("ideal"): no intermediate rounding; everything in double, the
  * result written as fp32 regardless of dt.
+ * mode 2 ("reference-rounded, last rounding left out"): as mode 0, but `out`
+ * is written as fp32 before its storage rounding.  A bf16 ulp at 4-5 sigma of
+ * the output distribution is up to 3.5e-2 x RMS, so a max-norm gate against
+ * the rounded output would be decided by 1-ulp coin flips of the last
+ * rounding; this mode gives the value those flips are taken around.
  *
  * x [n,H] (dt), w_* 16-bit of type dt (or fp32 if dt==EKO_F32).
- * out: dt in mode 0, fp32 in mode 1.  h_out (optional, may be NULL): [n,I]
- * same typing rule as out.
+ * out: dt in mode 0, fp32 in modes 1 and 2.  h_out (optional, may be NULL):
+ * [n,I], dt in modes 0 and 2, fp32 in mode 1.
  */
 void eko_ffn(const void *x, int64_t n, int64_t H, int64_t I, const void *w_up, const void *w_gate,
              const void *w_down, int dt, int mode, void *out, void *h_out)
@@ -318,7 +321,7 @@ void eko_ffn(const void *x, int64_t n, int64_t H, int64_t I, const void *w_up, c
                 au += (double)xr[k] * (double)load_act(w_up, c * H + k, dt);
                 ag += (double)xr[k] * (double)load_act(w_gate, c * H + k, dt);
             }
-            if (mode == 0) {
+            if (mode != 1) {
                 float up = round_act((float)au, dt);
                 float gate = round_act((float)ag, dt);
                 float sg = round_act(gate / (1.0f + expf(-gate)), dt);
@@ -330,7 +333,7 @@ void eko_ffn(const void *x, int64_t n, int64_t H, int64_t I, const void *w_up, c
     }
     if (h_out) {
         for (int64_t i = 0; i < n * I; ++i) {
-            if (mode == 0) store_act(h_out, i, (float)h[i], dt);
+            if (mode != 1) store_act(h_out, i, (float)h[i], dt);
             else ((float *)h_out)[i] = (float)h[i];
         }
     }
@@ -359,10 +362,11 @@ void eko_ffn(const void *x, int64_t n, int64_t H, int64_t I, const void *w_up, c
  *                   product rounded to dt, then summed.
  *   w_dt == EKO_F32 (DeepSeek shim, deepseek_v3/model.py:97-103): product and
  *                   sum stay fp32, one rounding to dt at the end.
- * y3 [T,K,H] (dt), w [T,K] (w_dt) -> y [T,H] (dt).
+ * y3 [T,K,H] (dt), w [T,K] (w_dt) -> y [T,H]: dt if round_out, else the fp32
+ * sum before its storage rounding.
  */
 void eko_combine(const void *y3, const void *w, int64_t T, int K, int64_t H, int dt, int w_dt,
-                 void *y)
+                 int round_out, void *y)
 {
     for (int64_t t = 0; t < T; ++t)
         for (int64_t c = 0; c < H; ++c) {
@@ -374,7 +378,8 @@ void eko_combine(const void *y3, const void *w, int64_t T, int K, int64_t H, int
                 if (w_dt != EKO_F32) p = round_act(p, dt);
                 acc += p;
             }
-            store_act(y, t * H + c, acc, dt);
+            if (round_out) store_act(y, t * H + c, acc, dt);
+            else ((float *)y)[t * H + c] = acc;
         }
 }
 
@@ -388,14 +393,18 @@ void eko_combine(const void *y3, const void *w, int64_t T, int K, int64_t H, int
  *
  * weights: arrays of E pointers (NULL allowed for experts that receive no
  * pair); mode as in eko_ffn.  In mode 1 the combine is done in double and y is
- * written as fp32 [T,H]; in mode 0 y has dtype dt.
+ * written as fp32 [T,H]; in mode 0 y has dtype dt; in mode 2 every tensor of
+ * the reference is rounded as in mode 0 except y itself, written as fp32.
  * route outputs (counts, offsets, perm, inv_perm) may each be NULL.
+ * y3_o (may be NULL): the [T,K,H] tensor the controller hands back before the
+ * weighted sum (dt in modes 0 and 2, fp32 in mode 1).
  * Returns 0; -1 bad id; -3 pair routed to an expert without weights.
  */
 int eko_layer_forward(const void *x, const int32_t *ids, const void *w, int64_t T, int K, int E,
                       int64_t H, int64_t I, const void *const *w_up, const void *const *w_gate,
                       const void *const *w_down, int dt, int w_dt, int mode, void *y,
-                      int32_t *counts_o, int32_t *offsets_o, int32_t *perm_o, int32_t *inv_o)
+                      int32_t *counts_o, int32_t *offsets_o, int32_t *perm_o, int32_t *inv_o,
+                      void *y3_o)
 {
     int64_t P = T * K;
     int es = act_size(dt);
@@ -406,7 +415,8 @@ int eko_layer_forward(const void *x, const int32_t *ids, const void *w, int64_t 
     int rc = eko_pack(ids, P, E, counts, offsets, perm, inv);
     if (rc) { free(counts); free(offsets); free(perm); free(inv); return rc; }
 
-    int oes = mode == 0 ? es : 4;
+    int ffn_mode = mode == 1 ? 1 : 0;
+    int oes = ffn_mode == 0 ? es : 4;
     char *xp = (char *)malloc((size_t)(P * H + 1) * (size_t)es);
     char *yp = (char *)malloc((size_t)(P * H + 1) * (size_t)oes);
     char *y3 = (char *)malloc((size_t)(P * H + 1) * (size_t)oes);
@@ -415,13 +425,13 @@ int eko_layer_forward(const void *x, const int32_t *ids, const void *w, int64_t 
         if (!counts[e]) continue;
         if (!w_up[e] || !w_gate[e] || !w_down[e]) { rc = -3; break; }
         eko_ffn(xp + (size_t)offsets[e] * (size_t)H * (size_t)es, counts[e], H, I, w_up[e],
-                w_gate[e], w_down[e], dt, mode, yp + (size_t)offsets[e] * (size_t)H * (size_t)oes,
+                w_gate[e], w_down[e], dt, ffn_mode, yp + (size_t)offsets[e] * (size_t)H * (size_t)oes,
                 NULL);
     }
     if (rc == 0) {
         eko_scatter(yp, H, oes, perm, P, y3);
-        if (mode == 0) {
-            eko_combine(y3, w, T, K, H, dt, w_dt, y);
+        if (mode != 1) {
+            eko_combine(y3, w, T, K, H, dt, w_dt, mode == 0, y);
         } else {
             for (int64_t t = 0; t < T; ++t)
                 for (int64_t c = 0; c < H; ++c) {
@@ -432,6 +442,7 @@ int eko_layer_forward(const void *x, const int32_t *ids, const void *w, int64_t 
                     ((float *)y)[t * H + c] = (float)acc;
                 }
         }
+        if (y3_o) memcpy(y3_o, y3, (size_t)(P * H) * (size_t)oes);
         if (counts_o) memcpy(counts_o, counts, sizeof(int32_t) * (size_t)E);
         if (offsets_o) memcpy(offsets_o, offsets, sizeof(int32_t) * (size_t)(E + 1));
         if (perm_o) memcpy(perm_o, perm, sizeof(int32_t) * (size_t)P);

@@ -122,14 +122,14 @@ def scatter(yp: torch.Tensor, perm: torch.Tensor, T: int, k: int) -> torch.Tenso
     return y3
 
 
-def dequant_channel(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
-    """W[n,:] = bf16(f32(q[n,:]) * f32(scale[n])); q int8 [N,C], scale bf16 [N]."""
+def dequant_channel(q: torch.Tensor, scale: torch.Tensor, dtype=torch.bfloat16) -> torch.Tensor:
+    """W[n,:] = rne_dtype(f32(q[n,:]) * f32(scale[n])); q int8 [N,C], scale bf16 [N]."""
     q = q.contiguous()
     scale = scale.contiguous()
     assert q.dtype == torch.int8 and scale.dtype == torch.bfloat16
     N, C = q.shape
-    w = torch.empty(N, C, dtype=torch.bfloat16)
-    lib().eko_dequant_channel(_p(q), _p(scale), _i64(N), _i64(C), _p(w))
+    w = torch.empty(N, C, dtype=dtype)
+    lib().eko_dequant_channel(_p(q), _p(scale), _i64(N), _i64(C), _DT[dtype], _p(w))
     return w
 
 
@@ -148,6 +148,7 @@ def ffn(x, w_up, w_gate, w_down, mode: int = 0, return_h: bool = False):
 
     mode 0: reference rounding points, result in x.dtype.
     mode 1: ideal (double, unrounded), result fp32.
+    mode 2: as mode 0 with the last storage rounding left out, result fp32.
     """
     dt = _DT[x.dtype]
     assert w_up.dtype == x.dtype and w_gate.dtype == x.dtype and w_down.dtype == x.dtype
@@ -155,28 +156,31 @@ def ffn(x, w_up, w_gate, w_down, mode: int = 0, return_h: bool = False):
     n, H = x.shape
     I = w_up.shape[0]
     assert tuple(w_up.shape) == (I, H) and tuple(w_gate.shape) == (I, H) and tuple(w_down.shape) == (H, I)
-    odt = x.dtype if mode == 0 else torch.float32
-    out = torch.empty(n, H, dtype=odt)
-    h = torch.empty(n, I, dtype=odt) if return_h else None
+    out = torch.empty(n, H, dtype=x.dtype if mode == 0 else torch.float32)
+    h = torch.empty(n, I, dtype=torch.float32 if mode == 1 else x.dtype) if return_h else None
     lib().eko_ffn(_p(x), _i64(n), _i64(H), _i64(I), _p(w_up.contiguous()), _p(w_gate.contiguous()),
                   _p(w_down.contiguous()), dt, mode, _p(out), _p(h))
     return (out, h) if return_h else out
 
 
-def combine(y3: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """y[t] = sum_k w[t,k] * Y[t,k] (qwen3_moe.py:102-104; deepseek_v3/model.py:97-103)."""
+def combine(y3: torch.Tensor, w: torch.Tensor, round_out: bool = True) -> torch.Tensor:
+    """y[t] = sum_k w[t,k] * Y[t,k] (qwen3_moe.py:102-104; deepseek_v3/model.py:97-103).
+
+    round_out=False returns the fp32 sum before its storage rounding."""
     y3 = y3.contiguous()
     w = w.contiguous()
     T, K, H = y3.shape
-    y = torch.empty(T, H, dtype=y3.dtype)
-    lib().eko_combine(_p(y3), _p(w), _i64(T), K, _i64(H), _DT[y3.dtype], _DT[w.dtype], _p(y))
+    y = torch.empty(T, H, dtype=y3.dtype if round_out else torch.float32)
+    lib().eko_combine(_p(y3), _p(w), _i64(T), K, _i64(H), _DT[y3.dtype], _DT[w.dtype], int(round_out), _p(y))
     return y
 
 
-def layer_forward(x, ids, w, w_up, w_gate, w_down, mode: int = 0):
+def layer_forward(x, ids, w, w_up, w_gate, w_down, mode: int = 0, return_y3: bool = False):
     """Whole layer, Expert Kit form.  w_* are lists of E tensors (None allowed).
 
-    Returns (y, counts, offsets, perm, inv_perm); y is x.dtype (mode 0) or fp32.
+    Returns (y, counts, offsets, perm, inv_perm); y is x.dtype (mode 0) or fp32
+    (mode 1 ideal; mode 2 reference-rounded except for y's own storage rounding).
+    With return_y3 the [T,K,H] tensor before the weighted sum is appended.
     """
     x = x.contiguous()
     T, H = x.shape
@@ -191,15 +195,16 @@ def layer_forward(x, ids, w, w_up, w_gate, w_down, mode: int = 0):
     offsets = torch.empty(E + 1, dtype=torch.int32)
     perm = torch.empty(P, dtype=torch.int32)
     inv = torch.empty(P, dtype=torch.int32)
+    y3 = torch.empty(T, K, H, dtype=torch.float32 if mode == 1 else x.dtype) if return_y3 else None
     wu = [None if t is None else t.contiguous() for t in w_up]
     wg = [None if t is None else t.contiguous() for t in w_gate]
     wd = [None if t is None else t.contiguous() for t in w_down]
     rc = lib().eko_layer_forward(_p(x), _p(ids), _p(w), _i64(T), K, E, _i64(H), _i64(I), _ptr_array(wu),
                                  _ptr_array(wg), _ptr_array(wd), _DT[x.dtype], _DT[w.dtype], mode, _p(y),
-                                 _p(counts), _p(offsets), _p(perm), _p(inv))
+                                 _p(counts), _p(offsets), _p(perm), _p(inv), _p(y3))
     if rc:
         raise ValueError(f"eko_layer_forward rc={rc}")
-    return y, counts, offsets, perm, inv
+    return (y, counts, offsets, perm, inv, y3) if return_y3 else (y, counts, offsets, perm, inv)
 
 
 def layer_loop_form(x, ids, w, w_up, w_gate, w_down):
@@ -234,12 +239,12 @@ def torch_router(logits: torch.Tensor, k: int, renorm: bool = True, w_dtype=torc
     return sel.to(torch.int32), rw.to(w_dtype)
 
 
-def torch_dequant_channel(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
-    """bf16(f32(q) * f32(scale[n])) with libtorch ops: what a CPU backend holds
-    after load_module's cast to bf16 (ffn/expert_torch.rs:61-78)."""
+def torch_dequant_channel(q: torch.Tensor, scale: torch.Tensor, dtype=torch.bfloat16) -> torch.Tensor:
+    """rne(f32(q) * f32(scale[n])) with libtorch ops: what a CPU backend holds
+    after load_module's cast to its compute dtype (ffn/expert_torch.rs:61-78)."""
     if q.dtype != torch.int8:
         return q.cpu()
-    return (q.cpu().float() * scale.cpu().float().unsqueeze(1)).to(torch.bfloat16)
+    return (q.cpu().float() * scale.cpu().float().unsqueeze(1)).to(dtype)
 
 
 def torch_ffn(x, w_up, w_gate, w_down):
