@@ -58,6 +58,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4"])
     ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--calib-copy-mib", type=int, default=0,
+                    help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
+                         "used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -95,6 +98,13 @@ def main():
     ref_perm = torch.argsort(ids.reshape(-1).long(), stable=True).to(torch.int32)
     assert torch.equal(rt.perm.cpu(), ref_perm), "routing permutation mismatch"
 
+    if args.calib_copy_mib:
+        src = torch.empty(args.calib_copy_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         layer.forward(xd, idd, gwd, stream=stream, out=y)
     torch.cuda.synchronize()

@@ -90,6 +90,8 @@ struct ek_layer {
     int32_t *counts = nullptr, *offsets = nullptr, *perm = nullptr, *inv_perm = nullptr;
     int32_t *row_token = nullptr, *block_hist = nullptr, *err = nullptr;
     void *h = nullptr, *yp = nullptr;
+    ek::WorkLists lists{};                   // device work lists (see ek_internal.h)
+    int64_t list_cap[ek::kNumLists] = {0, 0, 0, 0};
     int32_t *h_err = nullptr;                // pinned
 
     // staging for host-memory callers (allocated on first use)
@@ -133,7 +135,8 @@ void free_layer(ek_layer *L)
     for (void *p : L->expert_mem) if (p) (void)hipFree(p);
     void *bufs[] = {L->d_slabs, L->counts, L->offsets, L->perm, L->inv_perm, L->row_token,
                     L->block_hist, L->err, L->h, L->yp, L->st_x, L->st_w, L->st_y, L->st_xp,
-                    L->st_ids, L->st_raw};
+                    L->st_ids, L->st_raw, L->lists.count, L->lists.items[0], L->lists.items[1],
+                    L->lists.items[2], L->lists.items[3]};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
     if (L->h_err) (void)hipHostFree(L->h_err);
@@ -149,7 +152,7 @@ ek_status validate_cfg(const ek_cfg *c)
         return fail(EK_INVALID_INPUT, "act_dtype must be EK_BF16 or EK_F16 (got %d)", c->act_dtype);
     if (c->w_dtype != c->act_dtype && c->w_dtype != EK_I8)
         return fail(EK_INVALID_INPUT, "w_dtype must equal act_dtype or be EK_I8 (got %d)", c->w_dtype);
-    const int64_t ke = c->w_dtype == EK_I8 ? 64 : 32;
+    const int64_t ke = 64;   // contraction step of the tile kernel; int8 chunk width
     if (c->hidden <= 0 || c->inter <= 0 || c->hidden % ke || c->inter % ke)
         return fail(EK_INVALID_INPUT, "hidden (%lld) and inter (%lld) must be positive multiples of %lld",
                     (long long)c->hidden, (long long)c->inter, (long long)ke);
@@ -195,9 +198,17 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     A((void **)&L->err, sizeof(int32_t) * 4, "err");
     A(&L->h, (size_t)pmax * cfg->inter * 2, "h");
     A(&L->yp, (size_t)pmax * cfg->hidden * 2, "yp");
+    A((void **)&L->lists.count, sizeof(int32_t) * ek::kNumLists, "work list counts");
+    for (int l = 0; l < ek::kNumLists; ++l) {
+        // the per-expert entry point cuts one segment of up to pmax rows: capacity for E = 1 too
+        const int64_t cap = ek::list_capacity(l, pmax, E) + 1;
+        L->list_cap[l] = cap;
+        A((void **)&L->lists.items[l], sizeof(ek::WorkItem) * cap, "work list");
+    }
     if (st == EK_OK) {
         hipError_t e = hipMemset(L->d_slabs, 0, sizeof(ek::ExpertSlab) * E);
         if (e == hipSuccess) e = hipMemset(L->err, 0, sizeof(int32_t) * 4);
+        if (e == hipSuccess) e = hipMemset(L->lists.count, 0, sizeof(int32_t) * ek::kNumLists);
         if (e == hipSuccess) e = hipHostMalloc((void **)&L->h_err, sizeof(int32_t) * 4, hipHostMallocDefault);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->load_stream, hipStreamNonBlocking);
@@ -399,14 +410,46 @@ ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_lo
     a.inv_perm = L->inv_perm;
     a.row_token = L->row_token;
     a.err = L->err;
+    if (check_loaded) a.lists = L->lists;
+    else a.lists = ek::WorkLists{{nullptr, nullptr, nullptr, nullptr}, nullptr};
     return a;
+}
+
+// Both FFN stages over the work lists in L->lists: x [*, H] (rows picked through
+// `rows`, or packed order when nullptr) -> L->h -> out [P, H].  P and E bound the
+// list lengths (grid sizes); ev, if set, receives the stage boundary event.
+ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out, int64_t P, int64_t E,
+                      hipStream_t s, hipEvent_t *ev)
+{
+    const int64_t H = L->cfg.hidden, I = L->cfg.inter;
+    static const int tile_rows[ek::kNumLists] = {0, 32, 64, 128};
+    ek::FfnArgs a1;
+    a1.x = x; a1.x_stride = H; a1.rows = rows; a1.slabs = L->d_slabs; a1.out = L->h; a1.out_stride = I;
+    a1.N = (int32_t)I; a1.Kdim = (int32_t)H;
+    ek::FfnArgs a2 = a1;
+    a2.x = L->h; a2.x_stride = I; a2.rows = nullptr; a2.out = out; a2.out_stride = H;
+    a2.N = (int32_t)H; a2.Kdim = (int32_t)I;
+    for (int stage = 1; stage <= 2; ++stage) {
+        ek::FfnArgs a = stage == 1 ? a1 : a2;
+        for (int l = 0; l < ek::kNumLists; ++l) {
+            int64_t cap = ek::list_capacity(l, P, E);
+            if (cap > L->list_cap[l]) cap = L->list_cap[l];
+            if (cap <= 0) continue;
+            a.items = L->lists.items[l];
+            a.n_items = L->lists.count + l;
+            if (l == ek::kListStream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->w8, cap, s));
+            else EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->w8, tile_rows[l], cap, s));
+        }
+        if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
+    }
+    return EK_OK;
 }
 
 // pack -> stage 1 -> stage 2 -> combine on stream s; all pointers are device.
 ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const void *w, int w_f32,
                           int64_t T, void *y, hipStream_t s)
 {
-    const int64_t H = L->cfg.hidden, I = L->cfg.inter;
+    const int64_t H = L->cfg.hidden;
     const int E = L->cfg.n_experts, K = L->cfg.top_k;
     const int64_t P = T * K;
     hipEvent_t *ev = nullptr;
@@ -419,17 +462,7 @@ ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const 
     ek::launch_pack(pack_args(L, ids, P, true), s);
     if (ev) EK_HIP(hipEventRecord(ev[1], s));
     if (P > 0) {
-        ek::StreamArgs a1;
-        a1.x = x; a1.x_stride = H; a1.rows = L->row_token; a1.offsets = L->offsets;
-        a1.slabs = L->d_slabs; a1.out = L->h; a1.out_stride = I; a1.N = (int32_t)I;
-        a1.Kdim = (int32_t)H; a1.E = E; a1.e0 = 0; a1.single_n = -1; a1.min_rows = 1;
-        a1.max_rows = INT32_MAX;
-        EK_HIP(ek::launch_ffn_stream(a1, 1, L->act, L->w8, E, s));
-        if (ev) EK_HIP(hipEventRecord(ev[2], s));
-        ek::StreamArgs a2 = a1;
-        a2.x = L->h; a2.x_stride = I; a2.rows = nullptr; a2.out = L->yp; a2.out_stride = H;
-        a2.N = (int32_t)H; a2.Kdim = (int32_t)I;
-        EK_HIP(ek::launch_ffn_stream(a2, 2, L->act, L->w8, E, s));
+        EK_TRY(enqueue_ffn(L, x, L->row_token, L->yp, P, E, s, ev));
         if (ev) EK_HIP(hipEventRecord(ev[3], s));
         ek::CombineArgs c;
         c.yp = L->yp; c.inv_perm = L->inv_perm; c.w = w; c.y = y; c.T = T; c.K = K; c.H = H;
@@ -669,7 +702,7 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
             return fail(EK_INVALID_INPUT, "host-memory calls are blocking: stream must be NULL");
         DeviceGuard dg(layer->cfg.device_id);
         if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
-        const int64_t H = layer->cfg.hidden, I = layer->cfg.inter;
+        const int64_t H = layer->cfg.hidden;
         std::lock_guard<std::mutex> lk(layer->mu);
         if (!layer->expert_mem[expert])
             return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", expert);
@@ -684,16 +717,8 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
                 d_x = layer->st_x;
                 d_out = layer->st_y;
             }
-            ek::StreamArgs a1;
-            a1.x = d_x; a1.x_stride = H; a1.rows = nullptr; a1.offsets = nullptr;
-            a1.slabs = layer->d_slabs; a1.out = layer->h; a1.out_stride = I; a1.N = (int32_t)I;
-            a1.Kdim = (int32_t)H; a1.E = layer->cfg.n_experts; a1.e0 = expert;
-            a1.single_n = (int32_t)n; a1.min_rows = 1; a1.max_rows = INT32_MAX;
-            EK_HIP(ek::launch_ffn_stream(a1, 1, layer->act, layer->w8, 1, s));
-            ek::StreamArgs a2 = a1;
-            a2.x = layer->h; a2.x_stride = I; a2.out = d_out; a2.out_stride = H; a2.N = (int32_t)H;
-            a2.Kdim = (int32_t)I;
-            EK_HIP(ek::launch_ffn_stream(a2, 2, layer->act, layer->w8, 1, s));
+            ek::launch_single_lists(layer->lists, expert, (int32_t)n, s);
+            EK_TRY(enqueue_ffn(layer, d_x, nullptr, d_out, n, 1, s, nullptr));
             if (mem == EK_HOST)
                 EK_HIP(hipMemcpyAsync(out, layer->st_y, (size_t)n * H * 2, hipMemcpyDeviceToHost, s));
         }

@@ -1,4 +1,4 @@
-// Ragged grouped SwiGLU FFN, weight-streaming kernel (short segments).
+// Ragged grouped SwiGLU FFN, weight-streaming kernel (work items of <= 16 rows).
 //
 // Computes, per expert segment, the four ops of TorchFFN's closure
 // (ek-computation/src/ffn/expert_torch.rs:81-84):
@@ -22,50 +22,12 @@
 // significant bits), and v_cvt_pk_bf16_f32 rounds two of them to nearest even.
 // Each lane owns one output channel of the A operand, so s is a lane scalar.
 #include "ek_internal.h"
+#include "ek_mfma.h"
 
 namespace ek {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-template <typename T> struct Act;
-template <> struct Act<__bf16> {
-    using V8 = bf16x8;
-    static __device__ __forceinline__ f32x4 mfma(V8 a, V8 b, f32x4 c)
-    {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-    }
-};
-template <> struct Act<_Float16> {
-    using V8 = f16x8;
-    static __device__ __forceinline__ f32x4 mfma(V8 a, V8 b, f32x4 c)
-    {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-    }
-};
-
-template <typename T> __device__ __forceinline__ float rnd(float v) { return (float)(T)v; }
-
-// 8 offset-binary bytes (two dwords) of one output channel -> 8 dequantised
-// weights rne_T((u - 128) * s); c = -128 * s
-template <typename T>
-__device__ __forceinline__ typename Act<T>::V8 dequant_u8x8(uint32_t lo, uint32_t hi, float s, float c)
-{
-    typename Act<T>::V8 r;
-    r[0] = (T)__builtin_fmaf((float)(lo & 0xffu), s, c);
-    r[1] = (T)__builtin_fmaf((float)((lo >> 8) & 0xffu), s, c);
-    r[2] = (T)__builtin_fmaf((float)((lo >> 16) & 0xffu), s, c);
-    r[3] = (T)__builtin_fmaf((float)(lo >> 24), s, c);
-    r[4] = (T)__builtin_fmaf((float)(hi & 0xffu), s, c);
-    r[5] = (T)__builtin_fmaf((float)((hi >> 8) & 0xffu), s, c);
-    r[6] = (T)__builtin_fmaf((float)((hi >> 16) & 0xffu), s, c);
-    r[7] = (T)__builtin_fmaf((float)(hi >> 24), s, c);
-    return r;
-}
-
 template <typename T, bool W8, int NMAT, int NG, int D>
-__global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
+__global__ __launch_bounds__(256) void ffn_stream_kernel(FfnArgs a)
 {
     using V8 = typename Act<T>::V8;
     constexpr int KE = W8 ? 64 : 32;   // contraction elements per chunk
@@ -73,15 +35,9 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
     constexpr int NW = NMAT * NG;      // weight chunks per k step per wave
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int e, seg0, n;
-    if (a.single_n >= 0) {
-        e = a.e0; seg0 = 0; n = a.single_n;
-    } else {
-        e = blockIdx.y;
-        seg0 = a.offsets[e];
-        n = a.offsets[e + 1] - seg0;
-    }
-    if (n < a.min_rows || n > a.max_rows) return;
+    if ((int)blockIdx.y >= *a.n_items) return;
+    const WorkItem item = a.items[blockIdx.y];
+    const int e = item.expert, seg0 = item.row0, n = item.nrows;
     const int NT = a.N >> 4;
     const int nt0 = (blockIdx.x * 4 + wave) * NG;
     if (nt0 >= NT) return;
@@ -111,7 +67,8 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
             wc[gi * NMAT + m] = -128.f * sv;
         }
 
-    for (int r0 = 0; r0 < n; r0 += 16) {
+    {
+        constexpr int r0 = 0;   // items hold at most 16 rows
         const int jr = min(r0 + j, n - 1);   // lanes past the segment re-read its last row
         const int64_t row = a.rows ? (int64_t)a.rows[seg0 + jr] : (int64_t)(seg0 + jr);
         const T *xp = (const T *)a.x + row * a.x_stride + g * (KE / 4);
@@ -188,10 +145,7 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     if constexpr (NMAT == 2) {
-                        const float up = rnd<T>(acc[0][gi][r]);
-                        const float gate = rnd<T>(acc[1][gi][r]);
-                        const float sg = rnd<T>(gate / (1.0f + expf(-gate)));
-                        o[r] = (T)(up * sg);
+                        o[r] = swiglu_rounded<T>(acc[0][gi][r], acc[1][gi][r]);
                     } else {
                         o[r] = (T)acc[0][gi][r];
                     }
@@ -203,7 +157,7 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(StreamArgs a)
 }
 
 template <typename T, bool W8, int NMAT, int NG>
-static hipError_t launch_d(const StreamArgs &a, int32_t nseg, hipStream_t s)
+static hipError_t launch_d(const FfnArgs &a, int32_t nseg, hipStream_t s)
 {
     constexpr int KE = W8 ? 64 : 32;
     const int KT = a.Kdim / KE;
@@ -219,7 +173,7 @@ static hipError_t launch_d(const StreamArgs &a, int32_t nseg, hipStream_t s)
 }
 
 template <typename T, bool W8, int NMAT>
-static hipError_t launch_g(const StreamArgs &a, int32_t nseg, hipStream_t s)
+static hipError_t launch_g(const FfnArgs &a, int32_t nseg, hipStream_t s)
 {
     const int NT = a.N / 16;
     if (NMAT == 1 && NT % 4 == 0) return launch_d<T, W8, NMAT, 4>(a, nseg, s);
@@ -227,9 +181,10 @@ static hipError_t launch_g(const StreamArgs &a, int32_t nseg, hipStream_t s)
     return launch_d<T, W8, NMAT, 1>(a, nseg, s);
 }
 
-hipError_t launch_ffn_stream(const StreamArgs &a, int stage, int act, bool w8, int32_t n_segments,
+hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items,
                              hipStream_t s)
 {
+    const int32_t n_segments = (int32_t)max_items;
     if (n_segments <= 0) return hipSuccess;
     if (act == 0) {
         if (w8) return stage == 1 ? launch_g<__bf16, true, 2>(a, n_segments, s)

@@ -28,6 +28,33 @@ struct ExpertSlab {           // device addresses of one expert's tensors
     const float *s_down;      // [H]
 };
 
+// ---- work lists ---------------------------------------------------------------
+// The pack step cuts every expert segment into work items for the FFN kernels:
+// as many full 128-row tiles as fit, then the remainder r by size:
+//   r <= 16 -> one weight-streaming item, r <= 32 / <= 64 / <= 128 -> one MFMA
+//   tile of 32 / 64 / 128 rows.
+// Items of one class are stored expert-ascending, rows ascending.  List sizes
+// depend on the routing, list capacities only on P, so grids are fixed on the
+// host and kernels drop items beyond the device-side count.
+struct WorkItem {
+    int32_t expert;
+    int32_t row0;    // first packed position
+    int32_t nrows;
+    int32_t pad;
+};
+enum { kListStream = 0, kListT32 = 1, kListT64 = 2, kListT128 = 3, kNumLists = 4 };
+struct WorkLists {
+    WorkItem *items[kNumLists];
+    int32_t *count;              // [kNumLists]
+};
+inline int64_t list_capacity(int list, int64_t P, int64_t E)
+{
+    const int64_t min_rows[kNumLists] = {1, 17, 33, 65};
+    const int64_t by_rows = P / min_rows[list];
+    if (list == kListT128) return by_rows;
+    return by_rows < E ? by_rows : E;
+}
+
 // ---- routing (pack) ---------------------------------------------------------
 struct PackArgs {
     const int32_t *ids;       // [P]
@@ -43,6 +70,7 @@ struct PackArgs {
     int32_t *inv_perm;        // [P]
     int32_t *row_token;       // [P]  perm[j] / K
     int32_t *err;             // bit 0: id out of range, bit 1: expert not loaded
+    WorkLists lists;
 };
 constexpr int kPackChunk = 4096;   // pairs per workgroup
 constexpr int kPackThreads = 256;
@@ -50,30 +78,32 @@ constexpr int kMaxExperts = 1024;
 
 void launch_clear_err(int32_t *err, hipStream_t s);   // fill kernel (graph-capture safe)
 void launch_pack(const PackArgs &a, hipStream_t s);
+// work lists for one segment [0, n) of expert e (per-expert forward)
+void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, hipStream_t s);
 void launch_gather(const void *x, const int32_t *row_token, int64_t P, int64_t row_bytes, void *xp,
                    hipStream_t s);
 
-// ---- grouped FFN, weight-streaming kernel -------------------------------------
-struct StreamArgs {
+// ---- grouped FFN -------------------------------------------------------------
+struct FfnArgs {
     const void *x;            // activations, row stride x_stride elements
     int64_t x_stride;
     const int32_t *rows;      // packed position -> row of x, or nullptr (identity)
-    const int32_t *offsets;   // [E+1] segment starts (ignored when single_n >= 0)
     const ExpertSlab *slabs;  // [E]
     void *out;                // stage 1: h [P, N]; stage 2: yp [P, N]
     int64_t out_stride;
     int32_t N;                // output channels of this stage
     int32_t Kdim;             // contraction length of this stage
-    int32_t E;
-    int32_t e0;               // expert id when single_n >= 0
-    int32_t single_n;         // >= 0: one segment [0, single_n) of expert e0
-    int32_t min_rows;         // segments with fewer rows are skipped
-    int32_t max_rows;         // segments with more rows are skipped
+    const WorkItem *items;    // work list of the kernel's class
+    const int32_t *n_items;   // device-side length of that list
 };
 // stage = 1: up/gate + SwiGLU epilogue;  stage = 2: down projection
 // act: 0 bf16, 1 f16;  w8: int8 weights with per-channel scales
-hipError_t launch_ffn_stream(const StreamArgs &a, int stage, int act, bool w8, int32_t n_segments,
+// weight-streaming kernel (items of <= 16 rows); max_items = grid bound
+hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items,
                              hipStream_t s);
+// MFMA tile kernel, rows_per_tile in {32, 64, 128}
+hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, bool w8, int rows_per_tile,
+                           int64_t max_items, hipStream_t s);
 
 // ---- combine ----------------------------------------------------------------
 struct CombineArgs {

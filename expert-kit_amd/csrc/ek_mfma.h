@@ -1,0 +1,59 @@
+// MFMA operand types and the shared W8A16 dequantisation / SwiGLU epilogue.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ek {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Act;
+template <> struct Act<__bf16> {
+    using V8 = bf16x8;
+    static __device__ __forceinline__ f32x4 mfma(V8 a, V8 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Act<_Float16> {
+    using V8 = f16x8;
+    static __device__ __forceinline__ f32x4 mfma(V8 a, V8 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+template <typename T> __device__ __forceinline__ float rnd(float v) { return (float)(T)v; }
+
+// 8 offset-binary bytes (two dwords) of one output channel -> 8 dequantised
+// weights rne_T((u - 128) * s); c = -128 * s
+template <typename T>
+__device__ __forceinline__ typename Act<T>::V8 dequant_u8x8(uint32_t lo, uint32_t hi, float s, float c)
+{
+    typename Act<T>::V8 r;
+    r[0] = (T)__builtin_fmaf((float)(lo & 0xffu), s, c);
+    r[1] = (T)__builtin_fmaf((float)((lo >> 8) & 0xffu), s, c);
+    r[2] = (T)__builtin_fmaf((float)((lo >> 16) & 0xffu), s, c);
+    r[3] = (T)__builtin_fmaf((float)(lo >> 24), s, c);
+    r[4] = (T)__builtin_fmaf((float)(hi & 0xffu), s, c);
+    r[5] = (T)__builtin_fmaf((float)((hi >> 8) & 0xffu), s, c);
+    r[6] = (T)__builtin_fmaf((float)((hi >> 16) & 0xffu), s, c);
+    r[7] = (T)__builtin_fmaf((float)(hi >> 24), s, c);
+    return r;
+}
+
+
+// SwiGLU with the reference's storage roundings: up, gate, silu(gate) and the
+// product are each a materialised tensor of the activation dtype
+// (ek-computation/src/ffn/expert_torch.rs:81-83).
+template <typename T> __device__ __forceinline__ T swiglu_rounded(float acc_up, float acc_gate)
+{
+    const float up = rnd<T>(acc_up);
+    const float gate = rnd<T>(acc_gate);
+    const float sg = rnd<T>(gate / (1.0f + expf(-gate)));
+    return (T)(up * sg);
+}
+
+}  // namespace ek

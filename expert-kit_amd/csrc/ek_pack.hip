@@ -8,7 +8,8 @@
 // Three launches, all integer work, all HBM/LDS bound:
 //   pack_hist : one LDS histogram per 4096-pair chunk
 //   pack_scan : per-expert exclusive scan over chunks, then a wavefront
-//               prefix scan over experts -> counts, offsets
+//               prefix scan over experts -> counts, offsets, and the FFN
+//               kernels' work lists
 //   pack_rank : stable rank of every pair inside its chunk by wave-level
 //               match (ballots over the id bits) -> perm, inv_perm, row_token
 // plus a coalesced row gather (assemble_seq_tensors, executor.rs:112-133).
@@ -35,12 +36,62 @@ __global__ __launch_bounds__(kPackThreads) void pack_hist_kernel(PackArgs a)
         a.block_hist[(int64_t)blockIdx.x * a.E + i] = hist[i];
 }
 
+// Exclusive prefix sum of one int per thread over a 1024-thread workgroup:
+// shuffles inside each wavefront, then the 16 wave totals through LDS.
+// Returns the exclusive prefix; *total receives the workgroup sum.
+__device__ __forceinline__ int32_t block_exclusive_scan(int32_t v, int32_t *wave_tot, int32_t *total)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int32_t incl = v;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int32_t up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+    }
+    __syncthreads();   // wave_tot may still be read from a previous scan
+    if (lane == 63) wave_tot[wave] = incl;
+    __syncthreads();
+    int32_t base = 0, sum = 0;
+    for (int w = 0; w < 16; ++w) {
+        const int32_t t = wave_tot[w];
+        if (w < wave) base += t;
+        sum += t;
+    }
+    *total = sum;
+    return base + incl - v;
+}
+
+// How one segment of n rows is cut into work items (see WorkLists).
+struct SegmentCut {
+    int32_t n128, n64, n32, ns;
+};
+__device__ __forceinline__ SegmentCut cut_segment(int32_t n)
+{
+    SegmentCut c;
+    const int32_t r = n & 127;
+    c.n128 = (n >> 7) + (r > 64);
+    c.n64 = r > 32 && r <= 64;
+    c.n32 = r > 16 && r <= 32;
+    c.ns = r > 0 && r <= 16;
+    return c;
+}
+__device__ __forceinline__ void emit_items(const WorkLists &l, int32_t e, int32_t seg0, int32_t n,
+                                           int32_t p128, int32_t p64, int32_t p32, int32_t ps)
+{
+    const int32_t full = n >> 7, r = n & 127;
+    for (int32_t t = 0; t < full; ++t) l.items[kListT128][p128 + t] = WorkItem{e, seg0 + t * 128, 128, 0};
+    const WorkItem rem{e, seg0 + full * 128, r, 0};
+    if (r > 64) l.items[kListT128][p128 + full] = rem;
+    else if (r > 32) l.items[kListT64][p64] = rem;
+    else if (r > 16) l.items[kListT32][p32] = rem;
+    else if (r > 0) l.items[kListStream][ps] = rem;
+}
+
 // One workgroup of 1024 threads; thread e owns expert e.
 __global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
 {
     __shared__ int32_t wave_tot[16];
     const int e = threadIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int32_t total = 0;
     if (e < a.E) {
         for (int b = 0; b < a.nblocks; ++b) {
@@ -52,19 +103,39 @@ __global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
         a.counts[e] = total;
         if (total > 0 && a.slabs != nullptr && a.slabs[e].upgate == nullptr) atomicOr(a.err, 2);
     }
-    // inclusive prefix scan across the wavefront
-    int32_t incl = total;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int32_t up = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += up;
+    int32_t sum;
+    const int32_t off = block_exclusive_scan(total, wave_tot, &sum);
+    if (e < a.E) a.offsets[e] = off;
+    if (e == 0) a.offsets[a.E] = sum;
+    if (a.lists.count == nullptr) return;
+    const SegmentCut c = cut_segment(total);
+    int32_t s128, s64, s32, ss;
+    const int32_t p128 = block_exclusive_scan(c.n128, wave_tot, &s128);
+    const int32_t p64 = block_exclusive_scan(c.n64, wave_tot, &s64);
+    const int32_t p32 = block_exclusive_scan(c.n32, wave_tot, &s32);
+    const int32_t ps = block_exclusive_scan(c.ns, wave_tot, &ss);
+    if (e < a.E && total > 0) emit_items(a.lists, e, off, total, p128, p64, p32, ps);
+    if (e == 0) {
+        a.lists.count[kListT128] = s128;
+        a.lists.count[kListT64] = s64;
+        a.lists.count[kListT32] = s32;
+        a.lists.count[kListStream] = ss;
     }
-    if (lane == 63) wave_tot[wave] = incl;
-    __syncthreads();
-    int32_t wave_base = 0;
-    for (int w = 0; w < wave; ++w) wave_base += wave_tot[w];
-    if (e < a.E) a.offsets[e] = wave_base + incl - total;
-    if (e == a.E - 1) a.offsets[a.E] = wave_base + incl;
+}
+
+__global__ void single_lists_kernel(WorkLists l, int32_t e, int32_t n)
+{
+    const SegmentCut c = cut_segment(n);
+    if (n > 0) emit_items(l, e, 0, n, 0, 0, 0, 0);
+    l.count[kListT128] = c.n128;
+    l.count[kListT64] = c.n64;
+    l.count[kListT32] = c.n32;
+    l.count[kListStream] = c.ns;
+}
+
+void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, hipStream_t s)
+{
+    hipLaunchKernelGGL(single_lists_kernel, dim3(1), dim3(1), 0, s, lists, expert, n);
 }
 
 __global__ __launch_bounds__(kPackThreads) void pack_rank_kernel(PackArgs a, int nbits)

@@ -1,13 +1,16 @@
 """Parity of the HIP path against the CPU oracle, through the C ABI.
 
 Bars: routing tables and the gather are bit-exact; FFN / layer outputs satisfy
-max|y - y_ref| <= 2e-2 * rms(y_ref).  y_ref is the oracle's reference-rounded
-form (fp32-equivalent accumulation, storage rounding after every op) taken
-*before its last storage rounding* (oracle mode 2): one bf16 ulp at 4-5 sigma of
-the output distribution is up to 3.5e-2 x RMS, so a max-norm gate against the
-rounded tensor would be decided by coin flips of that last rounding.  The
-distance to the fully rounded form is reported and bounded by the gate plus
-one ulp.
+|y - y_ref| <= 2e-2 * rms(y_ref) + q, where q is the storage quantum of the
+16-bit output type.  y_ref is the oracle's reference-rounded form
+(fp32-equivalent accumulation, storage rounding after every op) taken *before
+its last storage rounding* (oracle mode 2).  Why q: the output is stored in
+bf16 / fp16, so even the exactly computed value sits up to half an ulp from
+y_ref; a bf16 ulp is 2^-7..2^-8 of the value, i.e. up to 3.5e-2 x RMS at 4.5
+sigma, so without q the gate would be decided by the last storage rounding and
+by how far the tail of the distribution reaches, not by the arithmetic.  Every
+test also asserts that the plain bound 2e-2 * rms holds for all but 1e-4 of the
+elements and prints the plain max|err| / rms.
 """
 import pytest
 import torch
@@ -22,6 +25,24 @@ def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
     ref = ref.float()
     rms = float(ref.pow(2).mean().sqrt())
     return float((got.float().cpu() - ref).abs().max()) / max(rms, 1e-30)
+
+
+def ulp_of(v: torch.Tensor, dtype) -> torch.Tensor:
+    """Spacing of `dtype` at the magnitude of each element of v (normal range)."""
+    bits = 7 if dtype == torch.bfloat16 else 10
+    return torch.exp2(torch.floor(torch.log2(v.float().abs().clamp_min(1e-30))) - bits)
+
+
+def ffn_gate(got: torch.Tensor, ref32: torch.Tensor, name: str) -> float:
+    """One expert's gate: 2e-2 * rms plus half an output ulp (the output's own storage rounding)."""
+    rms = float(ref32.pow(2).mean().sqrt())
+    err = (got.float().cpu() - ref32).abs()
+    strict_viol = float((err > TOL * rms).float().mean())
+    worst = float(err.max()) / rms
+    print(f"{name}: max|err|/rms = {worst:.3e}, elements over 2e-2*rms: {strict_viol:.2e}", flush=True)
+    assert bool((err <= TOL * rms + 0.5 * ulp_of(ref32, got.dtype) * 1.0001).all()), worst
+    assert strict_viol <= 1e-4
+    return worst
 
 
 def check_vs_rounded(got: torch.Tensor, ref32: torch.Tensor, name: str = ""):
@@ -42,18 +63,19 @@ def layer_gate(y: torch.Tensor, ref32: torch.Tensor, y3: torch.Tensor, gw: torch
 
     strict : max|y - y_ref| <= 2e-2 * rms(y_ref) -- must hold for all but 1e-4 of the
              elements, and is reported;
-    always : every element is within the strict bound plus ONE ulp flip of a stored
-             intermediate, 2^-7 (bf16; 2^-10 fp16) * max_k |w[t,k] * Y[t,k,c]|.  The
-             reference materialises Y[T,K,H] and w*Y in the 16-bit type; fp32
-             accumulation order alone decides on which side of a rounding boundary
-             such a stored value falls, and for K <= 2 (gate weight near 1) one such
-             flip at 3-4 sigma already exceeds 2e-2 * RMS.
+    always : every element is within the strict bound plus the storage quanta of the
+             16-bit tensors involved: half an ulp of y itself (its own storage
+             rounding) and ONE ulp flip of a stored intermediate,
+             ulp(max_k |w[t,k] * Y[t,k,c]|).  The reference materialises Y[T,K,H] and
+             w*Y in the 16-bit type; fp32 accumulation order alone decides on which
+             side of a rounding boundary such a stored value falls, and for K <= 2
+             (gate weight near 1) one such flip at 3-4 sigma already exceeds 2e-2 * RMS.
     """
     y = y.float().cpu()
     rms = float(ref32.pow(2).mean().sqrt())
     err = (y - ref32).abs()
-    ulp = 2.0 ** (-7 if y3.dtype == torch.bfloat16 else -10)
-    flip = ulp * (gw.float().unsqueeze(-1) * y3.float()).abs().amax(dim=1)
+    flip = ulp_of((gw.float().unsqueeze(-1) * y3.float()).abs().amax(dim=1), y3.dtype) \
+        + 0.5 * ulp_of(ref32, y3.dtype) * 1.0001
     strict_viol = float((err > TOL * rms).float().mean())
     worst = float(err.max()) / rms
     print(f"{name}: max|err|/rms = {worst:.3e}, elements over 2e-2*rms: {strict_viol:.2e}", flush=True)
@@ -140,14 +162,14 @@ def test_gather_bit_exact(ek, oracle, cuda):
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("w8", [False, True])
-@pytest.mark.parametrize("n", [1, 5, 16, 17, 40])
+@pytest.mark.parametrize("n", [1, 5, 16, 17, 32, 33, 64, 65, 128, 129, 145, 300])
 def test_expert_forward(ek, oracle, cuda, dt, w8, n):
     print(f"expert_forward dt={dt} w8={w8} n={n}", flush=True)
     w = wl.Workload("t", 256, 192, 1, 1, n, dt, w8=w8)
     ew = wl.make_expert(w, 0)
     if not w8:   # larger weights than the benchmark's so that silu is exercised off its linear part
         ew = ek.ExpertWeight(ew.up_w * 4, ew.gate_w * 4, ew.down_w * 4)
-    ffn = ek.HipFFN.construct(ek.EKInstance(w.hidden, w.inter), ew, act_dtype=dt, max_rows=64)
+    ffn = ek.HipFFN.construct(ek.EKInstance(w.hidden, w.inter), ew, act_dtype=dt, max_rows=512)
     assert ffn.backend() == "hip" and ffn.shape() == (256, 192)
     g = torch.Generator().manual_seed(n)
     x = torch.randn(n, w.hidden, generator=g).to(dt)
@@ -155,7 +177,7 @@ def test_expert_forward(ek, oracle, cuda, dt, w8, n):
     ref = oracle.ffn(x, wu, wg, wd, mode=2)
     got_dev = ffn.forward(x.to(cuda))
     got_host = ffn.forward(x)
-    assert rel_err(got_dev, ref) <= TOL, rel_err(got_dev, ref)
+    ffn_gate(got_dev, ref, f"expert_forward dt={dt} w8={w8} n={n}")
     same = check_vs_rounded(got_dev, ref, f"expert_forward dt={dt} w8={w8} n={n}")
     assert same > 0.9   # same weights bit for bit (int8 ones after dequantisation): only accumulation order differs
     assert torch.equal(got_dev.cpu().view(torch.int16), got_host.view(torch.int16))
@@ -245,9 +267,7 @@ def test_layer_c3_sampled(ek, oracle, cuda):
         got = layer.expert_forward(e, xe.to(cuda))
         wu, wg, wd = oracle_weights(oracle, {e: ws[e]}, w.n_experts)
         ref = oracle.ffn(xe, wu[e], wg[e], wd[e], mode=2)
-        err = rel_err(got, ref)
-        print(f"c3 expert {e}: rows={xe.shape[0]} max|err|/rms = {err:.3e}", flush=True)
-        assert err <= TOL
+        ffn_gate(got, ref, f"c3 expert {e}: rows={xe.shape[0]}")
     layer.close()
 
 
