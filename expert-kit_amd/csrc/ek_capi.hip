@@ -422,24 +422,22 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
                       hipStream_t s, hipEvent_t *ev)
 {
     const int64_t H = L->cfg.hidden, I = L->cfg.inter;
-    static const int tile_rows[ek::kNumLists] = {0, 32, 64, 128};
     ek::FfnArgs a1;
     a1.x = x; a1.x_stride = H; a1.rows = rows; a1.slabs = L->d_slabs; a1.out = L->h; a1.out_stride = I;
-    a1.N = (int32_t)I; a1.Kdim = (int32_t)H;
+    a1.N = (int32_t)I; a1.Kdim = (int32_t)H; a1.lists = L->lists;
     ek::FfnArgs a2 = a1;
     a2.x = L->h; a2.x_stride = I; a2.rows = nullptr; a2.out = out; a2.out_stride = H;
     a2.N = (int32_t)H; a2.Kdim = (int32_t)I;
+    int64_t cap[ek::kNumLists];
+    for (int l = 0; l < ek::kNumLists; ++l) {
+        cap[l] = ek::list_capacity(l, P, E);
+        if (cap[l] > L->list_cap[l]) cap[l] = L->list_cap[l];
+        if (cap[l] < 0) cap[l] = 0;
+    }
     for (int stage = 1; stage <= 2; ++stage) {
-        ek::FfnArgs a = stage == 1 ? a1 : a2;
-        for (int l = 0; l < ek::kNumLists; ++l) {
-            int64_t cap = ek::list_capacity(l, P, E);
-            if (cap > L->list_cap[l]) cap = L->list_cap[l];
-            if (cap <= 0) continue;
-            a.items = L->lists.items[l];
-            a.n_items = L->lists.count + l;
-            if (l == ek::kListStream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->w8, cap, s));
-            else EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->w8, tile_rows[l], cap, s));
-        }
+        const ek::FfnArgs &a = stage == 1 ? a1 : a2;
+        EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->w8, cap[ek::kListStream], s));
+        EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->w8, cap, s));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
     }
     return EK_OK;
@@ -458,7 +456,6 @@ ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const 
         L->events_used += 5;
     }
     if (ev) EK_HIP(hipEventRecord(ev[0], s));
-    ek::launch_clear_err(L->err, s);
     ek::launch_pack(pack_args(L, ids, P, true), s);
     if (ev) EK_HIP(hipEventRecord(ev[1], s));
     if (P > 0) {
@@ -674,7 +671,6 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
                 d_xp = layer->yp;   // [Pmax, H] scratch of the right size
             }
         }
-        ek::launch_clear_err(layer->err, s);
         ek::launch_pack(pack_args(layer, d_ids, P, false), s);
         if (xp) ek::launch_gather(d_x, layer->row_token, P, H * 2, d_xp, s);
         EK_HIP(hipGetLastError());

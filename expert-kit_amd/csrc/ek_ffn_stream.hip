@@ -35,8 +35,8 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(FfnArgs a)
     constexpr int NW = NMAT * NG;      // weight chunks per k step per wave
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if ((int)blockIdx.y >= *a.n_items) return;
-    const WorkItem item = a.items[blockIdx.y];
+    if ((int)blockIdx.y >= a.lists.count[kListStream]) return;
+    const WorkItem item = a.lists.items[kListStream][blockIdx.y];
     const int e = item.expert, seg0 = item.row0, n = item.nrows;
     const int NT = a.N >> 4;
     const int nt0 = (blockIdx.x * 4 + wave) * NG;
@@ -87,10 +87,9 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(FfnArgs a)
             for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
                 for (int m = 0; m < NMAT; ++m)
-                    wq[d][gi * NMAT + m] =
-                        *(const uint4 *)(wp[gi] + (int64_t)(d * NMAT + m) * kChunkBytes);
+                    wq[d][gi * NMAT + m] = ldg16(wp[gi] + (int64_t)(d * NMAT + m) * kChunkBytes);
 #pragma unroll
-            for (int v = 0; v < XV; ++v) xq[d][v] = *(const uint4 *)(xp + d * KE + v * 8);
+            for (int v = 0; v < XV; ++v) xq[d][v] = ldg16(xp + d * KE + v * 8);
         }
 
         for (int kt0 = 0; kt0 < KT; kt0 += D) {
@@ -125,11 +124,11 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(FfnArgs a)
                     for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
                         for (int m = 0; m < NMAT; ++m)
-                            wq[d][gi * NMAT + m] = *(const uint4 *)(
-                                wp[gi] + (int64_t)((kt + D) * NMAT + m) * kChunkBytes);
+                            wq[d][gi * NMAT + m] =
+                                ldg16(wp[gi] + (int64_t)((kt + D) * NMAT + m) * kChunkBytes);
 #pragma unroll
                     for (int v = 0; v < XV; ++v)
-                        xq[d][v] = *(const uint4 *)(xp + (int64_t)(kt + D) * KE + v * 8);
+                        xq[d][v] = ldg16(xp + (int64_t)(kt + D) * KE + v * 8);
                 }
             }
         }

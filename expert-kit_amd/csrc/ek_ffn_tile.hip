@@ -23,7 +23,7 @@
 namespace ek {
 
 template <typename T, bool W8, int NMAT, int MR>
-__global__ __launch_bounds__(256, 2) void ffn_tile_kernel(FfnArgs a, int nb_count)
+__device__ __forceinline__ void tile_body(const FfnArgs &a, const WorkItem item, const int nb, T *smem)
 {
     using V8 = typename Act<T>::V8;
     constexpr int NR = NMAT == 2 ? 2 : 4;      // channel tiles per wave and matrix
@@ -34,18 +34,9 @@ __global__ __launch_bounds__(256, 2) void ffn_tile_kernel(FfnArgs a, int nb_coun
     constexpr int CPS = BK / KE;                // weight chunks per step, channel tile and matrix
     constexpr int XP = BM * 8 / 256;            // 16-byte pieces of the x tile per thread and step
     constexpr int NWC = NR * NMAT * CPS;        // weight chunks per step per wave
-    __shared__ __attribute__((aligned(16))) T sX[2][BM][LDK];
+    typedef T XTile[BM][LDK];
+    XTile *sX = reinterpret_cast<XTile *>(smem);   // [2][BM][LDK]
 
-    // ---- which (item, channel block) -----------------------------------------
-    const int n_items = *a.n_items;
-    const int nvalid = n_items * nb_count;
-    const int per_xcd = (nvalid + 7) >> 3;
-    const int xi = blockIdx.x >> 3;
-    if (xi >= per_xcd) return;
-    const int logical = (blockIdx.x & 7) * per_xcd + xi;
-    if (logical >= nvalid) return;
-    const WorkItem item = a.items[logical / nb_count];
-    const int nb = logical % nb_count;
     const int e = item.expert, row0 = item.row0, nrows = item.nrows;
     const ExpertSlab slab = a.slabs[e];
     const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
@@ -105,10 +96,10 @@ __global__ __launch_bounds__(256, 2) void ffn_tile_kernel(FfnArgs a, int nb_coun
     _Pragma("unroll") for (int nr = 0; nr < NR; ++nr)                                          \
     _Pragma("unroll") for (int c = 0; c < CPS; ++c)                                            \
     _Pragma("unroll") for (int m = 0; m < NMAT; ++m)                                           \
-        dst[(nr * CPS + c) * NMAT + m] = *(const uint4 *)(                                     \
-            wp[nr] + (int64_t)(((step) * CPS + c) * NMAT + m) * kChunkBytes)
+        dst[(nr * CPS + c) * NMAT + m] =                                                       \
+            ldg16(wp[nr] + (int64_t)(((step) * CPS + c) * NMAT + m) * kChunkBytes)
 #define EK_LOAD_X(step)                                                                        \
-    _Pragma("unroll") for (int i = 0; i < XP; ++i) xreg[i] = *(const uint4 *)(xsrc[i] + (step) * BK)
+    _Pragma("unroll") for (int i = 0; i < XP; ++i) xreg[i] = ldg16(xsrc[i] + (step) * BK)
 #define EK_STORE_X(buf)                                                                        \
     _Pragma("unroll") for (int i = 0; i < XP; ++i) *(uint4 *)(&sX[buf][0][0] + xdst[i]) = xreg[i]
 
@@ -185,37 +176,63 @@ __global__ __launch_bounds__(256, 2) void ffn_tile_kernel(FfnArgs a, int nb_coun
 #undef EK_LOAD_X
 #undef EK_STORE_X
 
+// One launch covers the three tile lists.  Workgroup b runs on XCD b % 8
+// (round-robin dispatch), so each XCD is given a contiguous eighth of every
+// list: first its 128-row items, then its 64-row, then its 32-row ones, each
+// times nb_count channel blocks.  Neighbouring workgroups of an XCD then share
+// the activation tile (same item) and mostly the expert's weights in its L2,
+// and every XCD gets the same mix of long and short items.
 template <typename T, bool W8, int NMAT>
-static hipError_t launch_mr(const FfnArgs &a, int rows_per_tile, int64_t max_items, hipStream_t s)
+__global__ __launch_bounds__(256, 2) void ffn_tile_kernel(FfnArgs a, int nb_count)
+{
+    __shared__ __attribute__((aligned(16))) T smem[2 * 128 * (64 + 8)];
+    const int x = blockIdx.x & 7;
+    int i = blockIdx.x >> 3;
+    const int n128 = a.lists.count[kListT128], n64 = a.lists.count[kListT64], n32 = a.lists.count[kListT32];
+    const int lo128 = x * n128 / 8, s128 = (x + 1) * n128 / 8 - lo128;
+    const int lo64 = x * n64 / 8, s64 = (x + 1) * n64 / 8 - lo64;
+    const int lo32 = x * n32 / 8, s32 = (x + 1) * n32 / 8 - lo32;
+    if (i < s128 * nb_count) {
+        tile_body<T, W8, NMAT, 8>(a, a.lists.items[kListT128][lo128 + i / nb_count], i % nb_count, smem);
+        return;
+    }
+    i -= s128 * nb_count;
+    if (i < s64 * nb_count) {
+        tile_body<T, W8, NMAT, 4>(a, a.lists.items[kListT64][lo64 + i / nb_count], i % nb_count, smem);
+        return;
+    }
+    i -= s64 * nb_count;
+    if (i < s32 * nb_count)
+        tile_body<T, W8, NMAT, 2>(a, a.lists.items[kListT32][lo32 + i / nb_count], i % nb_count, smem);
+}
+
+template <typename T, bool W8, int NMAT>
+static hipError_t launch_t(const FfnArgs &a, const int64_t max_items[kNumLists], hipStream_t s)
 {
     constexpr int NR = NMAT == 2 ? 2 : 4;
     const int NT = a.N / 16;
     const int nb_count = (NT + 4 * NR - 1) / (4 * NR);
-    const int64_t blocks = ((max_items * nb_count + 7) / 8) * 8;
+    const int64_t per_xcd = (max_items[kListT128] + 7) / 8 + (max_items[kListT64] + 7) / 8 +
+                            (max_items[kListT32] + 7) / 8;
+    const int64_t blocks = per_xcd * nb_count * 8;
     if (blocks <= 0) return hipSuccess;
-    dim3 grid((unsigned)blocks);
-    switch (rows_per_tile) {
-    case 128: hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT, 8>), grid, dim3(256), 0, s, a, nb_count); break;
-    case 64: hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT, 4>), grid, dim3(256), 0, s, a, nb_count); break;
-    default: hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT, 2>), grid, dim3(256), 0, s, a, nb_count); break;
-    }
+    hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT>), dim3((unsigned)blocks), dim3(256), 0, s, a, nb_count);
     return hipGetLastError();
 }
 
-hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, bool w8, int rows_per_tile,
-                           int64_t max_items, hipStream_t s)
+hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, bool w8,
+                           const int64_t max_items[kNumLists], hipStream_t s)
 {
-    if (max_items <= 0) return hipSuccess;
     if (act == 0) {
-        if (w8) return stage == 1 ? launch_mr<__bf16, true, 2>(a, rows_per_tile, max_items, s)
-                                  : launch_mr<__bf16, true, 1>(a, rows_per_tile, max_items, s);
-        return stage == 1 ? launch_mr<__bf16, false, 2>(a, rows_per_tile, max_items, s)
-                          : launch_mr<__bf16, false, 1>(a, rows_per_tile, max_items, s);
+        if (w8) return stage == 1 ? launch_t<__bf16, true, 2>(a, max_items, s)
+                                  : launch_t<__bf16, true, 1>(a, max_items, s);
+        return stage == 1 ? launch_t<__bf16, false, 2>(a, max_items, s)
+                          : launch_t<__bf16, false, 1>(a, max_items, s);
     }
-    if (w8) return stage == 1 ? launch_mr<_Float16, true, 2>(a, rows_per_tile, max_items, s)
-                              : launch_mr<_Float16, true, 1>(a, rows_per_tile, max_items, s);
-    return stage == 1 ? launch_mr<_Float16, false, 2>(a, rows_per_tile, max_items, s)
-                      : launch_mr<_Float16, false, 1>(a, rows_per_tile, max_items, s);
+    if (w8) return stage == 1 ? launch_t<_Float16, true, 2>(a, max_items, s)
+                              : launch_t<_Float16, true, 1>(a, max_items, s);
+    return stage == 1 ? launch_t<_Float16, false, 2>(a, max_items, s)
+                      : launch_t<_Float16, false, 1>(a, max_items, s);
 }
 
 }  // namespace ek

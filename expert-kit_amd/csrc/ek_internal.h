@@ -76,7 +76,7 @@ constexpr int kPackChunk = 4096;   // pairs per workgroup
 constexpr int kPackThreads = 256;
 constexpr int kMaxExperts = 1024;
 
-void launch_clear_err(int32_t *err, hipStream_t s);   // fill kernel (graph-capture safe)
+// clears *err itself (with a fill kernel, never a memset node: graph-capture safe)
 void launch_pack(const PackArgs &a, hipStream_t s);
 // work lists for one segment [0, n) of expert e (per-expert forward)
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, hipStream_t s);
@@ -93,17 +93,17 @@ struct FfnArgs {
     int64_t out_stride;
     int32_t N;                // output channels of this stage
     int32_t Kdim;             // contraction length of this stage
-    const WorkItem *items;    // work list of the kernel's class
-    const int32_t *n_items;   // device-side length of that list
+    WorkLists lists;          // device work lists and their lengths
 };
 // stage = 1: up/gate + SwiGLU epilogue;  stage = 2: down projection
 // act: 0 bf16, 1 f16;  w8: int8 weights with per-channel scales
-// weight-streaming kernel (items of <= 16 rows); max_items = grid bound
+// weight-streaming kernel over lists.items[kListStream]; max_items = grid bound
 hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items,
                              hipStream_t s);
-// MFMA tile kernel, rows_per_tile in {32, 64, 128}
-hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, bool w8, int rows_per_tile,
-                           int64_t max_items, hipStream_t s);
+// MFMA tile kernel over the three tile lists (128-row items first, then 64,
+// then 32); max_items[l] bounds list l
+hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, bool w8,
+                           const int64_t max_items[kNumLists], hipStream_t s);
 
 // ---- combine ----------------------------------------------------------------
 struct CombineArgs {

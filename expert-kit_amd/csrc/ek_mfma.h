@@ -25,6 +25,17 @@ template <> struct Act<_Float16> {
     }
 };
 
+// 16-byte load through the global (not flat) path.  Pointers that come out of
+// a struct in memory have no known address space, and a flat load also ties
+// up the LDS counter that the fragment reads wait on.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ldg16(const void *p)
+{
+    typedef const __attribute__((address_space(1))) u32x4 *gptr;
+    const u32x4 v = *(gptr)(uintptr_t)p;
+    return __builtin_bit_cast(uint4, v);
+}
+
 template <typename T> __device__ __forceinline__ float rnd(float v) { return (float)(T)v; }
 
 // 8 offset-binary bytes (two dwords) of one output channel -> 8 dequantised

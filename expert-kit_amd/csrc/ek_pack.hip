@@ -12,6 +12,7 @@
 //               kernels' work lists
 //   pack_rank : stable rank of every pair inside its chunk by wave-level
 //               match (ballots over the id bits) -> perm, inv_perm, row_token
+// (calls of at most 4096 pairs run all of it in one workgroup, pack_fused)
 // plus a coalesced row gather (assemble_seq_tensors, executor.rs:112-133).
 #include "ek_internal.h"
 
@@ -194,6 +195,94 @@ __global__ __launch_bounds__(kPackThreads) void pack_rank_kernel(PackArgs a, int
     }
 }
 
+// Whole pack step in one workgroup, for calls of at most kPackFusedMax pairs
+// (decode batches): histogram, scans, work lists and stable ranks without
+// leaving LDS, and no separate clear of the error word.  16 wavefronts; wave w
+// owns the consecutive pairs [w*sub, (w+1)*sub) and keeps them in registers.
+constexpr int kPackFusedMax = 4096;
+__global__ __launch_bounds__(1024) void pack_fused_kernel(PackArgs a, int nbits)
+{
+    extern __shared__ int32_t lds[];          // wbase[16][E], then wave_tot[16], err
+    int32_t *wave_tot = lds + 16 * a.E;
+    int32_t *lerr = wave_tot + 16;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr int kIter = kPackFusedMax / 1024;   // 64-pair groups per wave
+    for (int i = threadIdx.x; i < 16 * a.E; i += 1024) lds[i] = 0;
+    if (threadIdx.x == 0) *lerr = 0;
+    const int64_t start = (int64_t)wave * (kIter * 64);
+    int32_t id[kIter];
+    bool bad = false;
+#pragma unroll
+    for (int it = 0; it < kIter; ++it) {
+        const int64_t p = start + it * 64 + lane;
+        id[it] = p < a.P ? a.ids[p] : -1;
+        if (p < a.P && (uint32_t)id[it] >= (uint32_t)a.E) { bad = true; id[it] = -1; }
+    }
+    __syncthreads();
+    if (bad) atomicOr(lerr, 1);
+#pragma unroll
+    for (int it = 0; it < kIter; ++it)
+        if (id[it] >= 0) atomicAdd(&lds[wave * a.E + id[it]], 1);
+    __syncthreads();
+    const int e = threadIdx.x;
+    int32_t total = 0;
+    if (e < a.E) {
+        for (int w = 0; w < 16; ++w) total += lds[w * a.E + e];
+        a.counts[e] = total;
+        if (total > 0 && a.slabs != nullptr && a.slabs[e].upgate == nullptr) atomicOr(lerr, 2);
+    }
+    int32_t sum;
+    const int32_t off = block_exclusive_scan(total, wave_tot, &sum);
+    if (e < a.E) {
+        a.offsets[e] = off;
+        int32_t run = off;
+        for (int w = 0; w < 16; ++w) {
+            const int32_t t = lds[w * a.E + e];
+            lds[w * a.E + e] = run;
+            run += t;
+        }
+    }
+    if (e == 0) a.offsets[a.E] = sum;
+    if (a.lists.count != nullptr) {
+        const SegmentCut c = cut_segment(total);
+        int32_t s128, s64, s32, ss;
+        const int32_t p128 = block_exclusive_scan(c.n128, wave_tot, &s128);
+        const int32_t p64 = block_exclusive_scan(c.n64, wave_tot, &s64);
+        const int32_t p32 = block_exclusive_scan(c.n32, wave_tot, &s32);
+        const int32_t ps = block_exclusive_scan(c.ns, wave_tot, &ss);
+        if (e < a.E && total > 0) emit_items(a.lists, e, off, total, p128, p64, p32, ps);
+        if (e == 0) {
+            a.lists.count[kListT128] = s128;
+            a.lists.count[kListT64] = s64;
+            a.lists.count[kListT32] = s32;
+            a.lists.count[kListStream] = ss;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) a.err[0] = *lerr;
+#pragma unroll
+    for (int it = 0; it < kIter; ++it) {
+        const int64_t p = start + it * 64 + lane;
+        const bool valid = id[it] >= 0;
+        if (p < a.P && !valid) a.inv_perm[p] = -1;
+        uint64_t m = __ballot(valid);
+        for (int b = 0; b < nbits; ++b) {
+            const bool bit = (id[it] >> b) & 1;
+            const uint64_t bb = __ballot(bit);
+            m &= bit ? bb : ~bb;
+        }
+        if (valid) {
+            const int32_t rank = __popcll(m & ((1ull << lane) - 1ull));
+            const int32_t pos = lds[wave * a.E + id[it]] + rank;
+            const bool leader = (m >> lane) == 1ull;
+            if (leader) lds[wave * a.E + id[it]] = pos + 1;
+            a.perm[pos] = (int32_t)p;
+            a.inv_perm[p] = pos;
+            a.row_token[pos] = (int32_t)(p / a.K);
+        }
+    }
+}
+
 __global__ void clear_err_kernel(int32_t *err) { err[0] = 0; }
 
 void launch_clear_err(int32_t *err, hipStream_t s)
@@ -207,11 +296,18 @@ void launch_pack(const PackArgs &a, hipStream_t s)
         // offsets and counts must still be defined (all zero)
         PackArgs z = a;
         z.nblocks = 0;
+        launch_clear_err(a.err, s);
         hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(1024), 0, s, z);
         return;
     }
     int nbits = 0;
     while ((1 << nbits) < a.E) ++nbits;
+    if (a.P <= kPackFusedMax) {
+        const size_t lds_bytes = sizeof(int32_t) * (16 * (size_t)a.E + 32);
+        hipLaunchKernelGGL(pack_fused_kernel, dim3(1), dim3(1024), lds_bytes, s, a, nbits);
+        return;
+    }
+    launch_clear_err(a.err, s);
     hipLaunchKernelGGL(pack_hist_kernel, dim3(a.nblocks), dim3(kPackThreads), 0, s, a);
     hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(1024), 0, s, a);
     hipLaunchKernelGGL(pack_rank_kernel, dim3(a.nblocks), dim3(kPackThreads), 0, s, a, nbits);
