@@ -51,12 +51,70 @@ def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
     return pairs / med, pairs, len(times)
 
 
+def bench_chain(args, w, dev):
+    """The ragged continuous-batching mix over n_layers consecutive layers, one hipGraph."""
+    import torch
+    import ek_hip
+    from ek_hip import workloads as wl
+    layers = []
+    for l in range(w.n_layers):
+        layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype,
+                                w_dtype=torch.int8 if w.w8 else w.act_dtype, max_tokens=w.tokens)
+        for e in range(w.n_experts):
+            layer.set_expert(e, wl.make_expert(w, e, layer=l, device="cuda"))
+        layers.append(layer)
+    routing = [wl.make_routing(w, layer=l) for l in range(w.n_layers)]
+    ids = torch.stack([r[0] for r in routing]).to(dev)
+    gw = torch.stack([r[1] for r in routing]).to(dev)
+    xd = wl.make_x(w).to(dev)
+    y = torch.empty_like(xd)
+    chain = ek_hip.HipChain(layers)
+    stream = torch.cuda.current_stream()
+    y_eager = chain.forward(xd, ids, gw, use_graph=False).clone()
+    res = {}
+    for mode, use_graph in (("eager", False), ("graph", True)):
+        for _ in range(args.warmup):
+            chain.forward(xd, ids, gw, use_graph=use_graph, stream=stream, out=y)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for _ in range(args.steps):
+            chain.forward(xd, ids, gw, use_graph=use_graph, stream=stream, out=y)
+        ev1.record(stream)
+        torch.cuda.synchronize()
+        res[mode] = max(time.perf_counter() - t0, ev0.elapsed_time(ev1) * 1e-3) / args.steps
+        assert torch.equal(y.view(torch.int16), y_eager.view(torch.int16)), f"{mode} chain output changed"
+    step_s = res["graph"]
+    pairs = w.pairs * w.n_layers
+    counts = [torch.bincount(r[0].reshape(-1).long(), minlength=w.n_experts) for r in routing]
+    b = sum(wl.algorithmic_bytes(w, c) for c in counts)
+    f = pairs * w.flops_per_pair()
+    out = {
+        "metric": "token-expert pairs/s on 1 MI355X (DSv3 W8A16 layer); % HBM / MFMA roofline",
+        "value": pairs / step_s, "unit": "pairs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": step_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": str(w.act_dtype).replace("torch.", "") + ", fp32 accumulate", "data": "synthetic",
+        "config": {"workload": w.name, "hidden": w.hidden, "moe_intermediate": w.inter, "experts": w.n_experts,
+                   "top_k": w.top_k, "tokens": w.tokens, "pairs_per_layer": w.pairs, "layers": w.n_layers,
+                   "requests": len(wl.request_lengths()), "zipf_s": w.zipf_s, "launch": "one hipGraph per chain"},
+        "roofline": {"bound": "mfma" if f / MFMA_PEAK_16 > b / HBM_PEAK else "hbm",
+                     "achieved": f / step_s / 1e12, "peak": MFMA_PEAK_16 / 1e12, "unit": "TFLOP/s",
+                     "frac": f / step_s / MFMA_PEAK_16, "traffic": None, "kernel": "whole chain"},
+        "layer": {"algorithmic_bytes": b, "algorithmic_flops": f, "hbm_frac": b / step_s / HBM_PEAK,
+                  "mfma_frac": f / step_s / MFMA_PEAK_16, "eager_ms_per_step": res["eager"] * 1e3,
+                  "graph_ms_per_step": res["graph"] * 1e3},
+    }
+    chain.close()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
@@ -74,6 +132,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     w = wl.resolve(wl.CONFIGS[args.workload])
+    if w.n_layers > 1:
+        return bench_chain(args, w, dev)
     layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype,
                             w_dtype=torch.int8 if w.w8 else w.act_dtype, max_tokens=w.tokens)
     ids, gw = wl.make_routing(w)

@@ -114,6 +114,22 @@ struct ek_expert {
     ek_layer *layer = nullptr;
 };
 
+struct ek_chain {
+    std::vector<ek_layer *> layers;
+    void *act[2] = {nullptr, nullptr};       // ping-pong activations [max_tokens, H]
+    int32_t *d_err = nullptr;                // [L] per-layer routing error words, gathered
+    int32_t *h_err = nullptr;                // pinned
+    hipStream_t stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    // key of the captured graph
+    const void *k_x = nullptr, *k_ids = nullptr, *k_w = nullptr;
+    void *k_y = nullptr;
+    int64_t k_T = -1;
+    int32_t k_wdt = -1;
+    std::mutex mu;
+};
+
 namespace {
 
 ek_status dev_alloc(void **p, size_t bytes, const char *what)
@@ -770,6 +786,155 @@ ek_status ek_layer_get_stats(ek_layer *layer, ek_stats *out)
         }
         layer->events_used = 0;
         *out = layer->stats;
+        return EK_OK;
+    )
+}
+
+static void free_chain(ek_chain *c)
+{
+    if (!c) return;
+    (void)hipDeviceSynchronize();
+    if (c->exec) (void)hipGraphExecDestroy(c->exec);
+    if (c->graph) (void)hipGraphDestroy(c->graph);
+    if (c->act[0]) (void)hipFree(c->act[0]);
+    if (c->act[1]) (void)hipFree(c->act[1]);
+    if (c->d_err) (void)hipFree(c->d_err);
+    if (c->h_err) (void)hipHostFree(c->h_err);
+    if (c->stream) (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+ek_status ek_chain_create(ek_layer *const *layers, int32_t n_layers, ek_chain **out)
+{
+    EK_GUARDED(
+        if (!out) return fail(EK_INVALID_INPUT, "out is NULL");
+        *out = nullptr;
+        if (!layers || n_layers < 1 || n_layers > 1024)
+            return fail(EK_INVALID_INPUT, "n_layers must be in [1, 1024]");
+        for (int i = 0; i < n_layers; ++i) {
+            if (!layers[i]) return fail(EK_INVALID_INPUT, "layer %d is NULL", i);
+            const ek_cfg &a = layers[0]->cfg, &b = layers[i]->cfg;
+            if (a.hidden != b.hidden || a.top_k != b.top_k || a.act_dtype != b.act_dtype ||
+                a.device_id != b.device_id || a.max_tokens != b.max_tokens)
+                return fail(EK_INVALID_INPUT, "layer %d differs from layer 0 in hidden / top_k / "
+                            "act_dtype / device / max_tokens", i);
+        }
+        DeviceGuard dg(layers[0]->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layers[0]->cfg.device_id);
+        ek_chain *c = new (std::nothrow) ek_chain();
+        if (!c) return fail(EK_OOM, "host allocation failed");
+        c->layers.assign(layers, layers + n_layers);
+        const size_t act_bytes = (size_t)layers[0]->cfg.max_tokens * layers[0]->cfg.hidden * 2;
+        ek_status st = dev_alloc(&c->act[0], act_bytes, "chain activations");
+        if (st == EK_OK) st = dev_alloc(&c->act[1], act_bytes, "chain activations");
+        if (st == EK_OK) st = dev_alloc((void **)&c->d_err, sizeof(int32_t) * n_layers, "chain errors");
+        if (st == EK_OK) {
+            hipError_t e = hipHostMalloc((void **)&c->h_err, sizeof(int32_t) * n_layers, hipHostMallocDefault);
+            if (e == hipSuccess) e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+            if (e != hipSuccess) st = hip_fail(e, "chain setup");
+        }
+        if (st != EK_OK) {
+            std::string keep = g_last_error;
+            free_chain(c);
+            g_last_error = keep;
+            return st;
+        }
+        *out = c;
+        return EK_OK;
+    )
+}
+
+// All layer calls of the chain on stream s (eager or under capture).
+static ek_status enqueue_chain(ek_chain *c, const void *x, const int32_t *ids, const void *w, int w_f32,
+                               int64_t T, void *y, hipStream_t s)
+{
+    const int L = (int)c->layers.size();
+    const int64_t K = c->layers[0]->cfg.top_k;
+    const size_t w_es = w_f32 ? 4 : 2;
+    const void *in = x;
+    for (int l = 0; l < L; ++l) {
+        void *outp = l == L - 1 ? y : c->act[l & 1];
+        ek_layer *ly = c->layers[l];
+        const bool prof = ly->profiling;
+        ly->profiling = false;               // no event records inside a chain (capture-safe)
+        ek_status st = enqueue_forward(ly, in, ids + (size_t)l * T * K,
+                                       (const char *)w + (size_t)l * T * K * w_es, w_f32, T, outp, s);
+        ly->profiling = prof;
+        EK_TRY(st);
+        // collect the layer's error word with a copy kernel-free D2D memcpy node
+        EK_HIP(hipMemcpyAsync(c->d_err + l, ly->err, sizeof(int32_t), hipMemcpyDeviceToDevice, s));
+        in = outp;
+    }
+    return EK_OK;
+}
+
+ek_status ek_chain_forward(ek_chain *chain, const void *x, const int32_t *ids, const void *w,
+                           int32_t w_dtype, int64_t T, void *y, int32_t use_graph, void *stream)
+{
+    EK_GUARDED(
+        if (!chain) return fail(EK_INVALID_INPUT, "chain is NULL");
+        ek_layer *l0 = chain->layers[0];
+        if (T < 0 || T > l0->cfg.max_tokens)
+            return fail(EK_INVALID_INPUT, "T = %lld outside [0, max_tokens = %lld]", (long long)T,
+                        (long long)l0->cfg.max_tokens);
+        if (w_dtype != l0->cfg.act_dtype && w_dtype != EK_F32)
+            return fail(EK_INVALID_INPUT, "w_dtype must be the activation dtype or EK_F32 (got %d)", w_dtype);
+        if (T > 0 && (!x || !ids || !w || !y)) return fail(EK_INVALID_INPUT, "NULL tensor pointer");
+        DeviceGuard dg(l0->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", l0->cfg.device_id);
+        std::lock_guard<std::mutex> ck(chain->mu);
+        std::vector<std::unique_lock<std::mutex>> locks;
+        for (ek_layer *ly : chain->layers) locks.emplace_back(ly->mu);
+        hipStream_t s = stream ? (hipStream_t)stream : chain->stream;
+        const int w_f32 = w_dtype == EK_F32;
+        const int L = (int)chain->layers.size();
+        if (!stream) EK_HIP(hipDeviceSynchronize());
+        if (!use_graph) {
+            EK_TRY(enqueue_chain(chain, x, ids, w, w_f32, T, y, s));
+        } else {
+            const bool same = chain->exec && chain->k_x == x && chain->k_ids == ids && chain->k_w == w &&
+                              chain->k_y == y && chain->k_T == T && chain->k_wdt == w_dtype;
+            if (!same) {
+                if (chain->exec) { (void)hipGraphExecDestroy(chain->exec); chain->exec = nullptr; }
+                if (chain->graph) { (void)hipGraphDestroy(chain->graph); chain->graph = nullptr; }
+                // capture on the chain's own stream, never on the caller's
+                EK_HIP(hipStreamBeginCapture(chain->stream, hipStreamCaptureModeThreadLocal));
+                ek_status st = enqueue_chain(chain, x, ids, w, w_f32, T, y, chain->stream);
+                hipGraph_t g = nullptr;
+                hipError_t e = hipStreamEndCapture(chain->stream, &g);
+                if (st != EK_OK) { if (g) (void)hipGraphDestroy(g); return st; }
+                if (e != hipSuccess) return hip_fail(e, "hipStreamEndCapture");
+                chain->graph = g;
+                EK_HIP(hipGraphInstantiate(&chain->exec, g, nullptr, nullptr, 0));
+                chain->k_x = x; chain->k_ids = ids; chain->k_w = w; chain->k_y = y;
+                chain->k_T = T; chain->k_wdt = w_dtype;
+            }
+            EK_HIP(hipGraphLaunch(chain->exec, s));
+        }
+        for (ek_layer *ly : chain->layers) {
+            std::lock_guard<std::mutex> sl(ly->stats_mu);
+            ly->stats.forward_calls += 1;
+            ly->stats.tokens += T;
+            ly->stats.pairs += T * ly->cfg.top_k;
+        }
+        if (!stream) {
+            EK_HIP(hipMemcpyAsync(chain->h_err, chain->d_err, sizeof(int32_t) * L, hipMemcpyDeviceToHost, s));
+            EK_HIP(hipStreamSynchronize(s));
+            int32_t err = 0;
+            for (int l = 0; l < L; ++l) err |= chain->h_err[l];
+            return err_to_status(err);
+        }
+        return EK_OK;
+    )
+}
+
+ek_status ek_chain_destroy(ek_chain *chain)
+{
+    EK_GUARDED(
+        if (!chain) return fail(EK_INVALID_INPUT, "chain is NULL");
+        DeviceGuard dg(chain->layers[0]->cfg.device_id);
+        { std::lock_guard<std::mutex> ck(chain->mu); }
+        free_chain(chain);
         return EK_OK;
     )
 }

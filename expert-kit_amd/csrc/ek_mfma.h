@@ -38,23 +38,36 @@ __device__ __forceinline__ uint4 ldg16(const void *p)
 
 template <typename T> __device__ __forceinline__ float rnd(float v) { return (float)(T)v; }
 
+// Two fp32 values -> one dword holding their round-to-nearest-even 16-bit forms
+// (v_cvt_pk_bf16_f32 / v_cvt_pkrtz is not used: rtz would differ from the CPU cast).
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2<__bf16>(float lo, float hi)
+{
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+template <> __device__ __forceinline__ uint32_t pack2<_Float16>(float lo, float hi)
+{
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
 // 8 offset-binary bytes (two dwords) of one output channel -> 8 dequantised
 // weights rne_T((u - 128) * s); c = -128 * s
 template <typename T>
 __device__ __forceinline__ typename Act<T>::V8 dequant_u8x8(uint32_t lo, uint32_t hi, float s, float c)
 {
-    typename Act<T>::V8 r;
-    r[0] = (T)__builtin_fmaf((float)(lo & 0xffu), s, c);
-    r[1] = (T)__builtin_fmaf((float)((lo >> 8) & 0xffu), s, c);
-    r[2] = (T)__builtin_fmaf((float)((lo >> 16) & 0xffu), s, c);
-    r[3] = (T)__builtin_fmaf((float)(lo >> 24), s, c);
-    r[4] = (T)__builtin_fmaf((float)(hi & 0xffu), s, c);
-    r[5] = (T)__builtin_fmaf((float)((hi >> 8) & 0xffu), s, c);
-    r[6] = (T)__builtin_fmaf((float)((hi >> 16) & 0xffu), s, c);
-    r[7] = (T)__builtin_fmaf((float)(hi >> 24), s, c);
-    return r;
+    u32x4 r;
+    r[0] = pack2<T>(__builtin_fmaf((float)(lo & 0xffu), s, c), __builtin_fmaf((float)((lo >> 8) & 0xffu), s, c));
+    r[1] = pack2<T>(__builtin_fmaf((float)((lo >> 16) & 0xffu), s, c), __builtin_fmaf((float)(lo >> 24), s, c));
+    r[2] = pack2<T>(__builtin_fmaf((float)(hi & 0xffu), s, c), __builtin_fmaf((float)((hi >> 8) & 0xffu), s, c));
+    r[3] = pack2<T>(__builtin_fmaf((float)((hi >> 16) & 0xffu), s, c), __builtin_fmaf((float)(hi >> 24), s, c));
+    return __builtin_bit_cast(typename Act<T>::V8, r);
 }
-
 
 // SwiGLU with the reference's storage roundings: up, gate, silu(gate) and the
 // product are each a materialised tensor of the activation dtype

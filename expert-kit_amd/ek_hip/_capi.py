@@ -64,6 +64,9 @@ PROTOTYPES = {
     "ek_layer_expert_forward": (_I32, [_P, _I32, _P, _I64, _P, _I32, _P]),
     "ek_layer_profile": (_I32, [_P, _I32]),
     "ek_layer_get_stats": (_I32, [_P, ctypes.POINTER(ek_stats)]),
+    "ek_chain_create": (_I32, [_PP, _I32, _PP]),
+    "ek_chain_forward": (_I32, [_P, _P, _P, _P, _I32, _I64, _P, _I32, _P]),
+    "ek_chain_destroy": (_I32, [_P]),
     "ek_expert_create": (_I32, [ctypes.POINTER(ek_cfg), _I64, _DESC, _DESC, _DESC, _PP]),
     "ek_expert_forward": (_I32, [_P, _P, _I64, _P, _I32, _P]),
     "ek_expert_shape": (_I32, [_P, ctypes.POINTER(_I64), ctypes.POINTER(_I64)]),

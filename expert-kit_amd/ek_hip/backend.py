@@ -223,6 +223,39 @@ class HipLayer:
             pass
 
 
+class HipChain:
+    """L consecutive MoE layers (x_{l+1} = y_l) launched as one HIP graph."""
+
+    def __init__(self, layers: Sequence[HipLayer]):
+        self._lib = C.load()
+        self.layers = list(layers)
+        arr = (ctypes.c_void_p * len(self.layers))(*[l._h.value for l in self.layers])
+        self._h = ctypes.c_void_p()
+        C.check(self._lib.ek_chain_create(arr, len(self.layers), ctypes.byref(self._h)))
+
+    def forward(self, x: torch.Tensor, ids: torch.Tensor, w: torch.Tensor, use_graph: bool = True, stream=None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """ids, w: [L, T, K] on the device."""
+        assert x.is_cuda and ids.is_cuda and w.is_cuda and ids.dtype == torch.int32
+        assert x.is_contiguous() and ids.is_contiguous() and w.is_contiguous()
+        assert ids.dim() == 3 and ids.shape[0] == len(self.layers) and w.shape == ids.shape
+        y = out if out is not None else torch.empty_like(x)
+        C.check(self._lib.ek_chain_forward(self._h, _ptr(x), _ptr(ids), _ptr(w), _DT[w.dtype], x.shape[0], _ptr(y),
+                                           int(use_graph), _stream_ptr(stream)))
+        return y
+
+    def close(self) -> None:
+        if getattr(self, "_h", None) is not None and self._h.value:
+            self._lib.ek_chain_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class HipFFN:
     """One expert behind trait Expert<T> (ffn/meta.rs:30-39)."""
 

@@ -98,7 +98,7 @@ def make_routing(w: Workload, layer: int = 0):
     return sel.to(torch.int32).contiguous(), rw.to(w.act_dtype).contiguous()
 
 
-def make_expert(w: Workload, e: int, layer: int = 0, device: str = "cpu") -> ExpertWeight:
+def make_expert(w: Workload, e: int, layer: int = 0, device: str = "cpu", std: float = 0.02) -> ExpertWeight:
     """One expert's weights.  Each expert has its own generator stream, so any
     subset can be reproduced without drawing the others.  CPU and GPU generators
     give different values for the same seed; parity tests always move the very
@@ -117,7 +117,7 @@ def make_expert(w: Workload, e: int, layer: int = 0, device: str = "cpu") -> Exp
                             down_scale=s(H))
 
     def n(r, c):
-        return (torch.randn(r, c, generator=g, device=device) * 0.02).to(w.act_dtype)
+        return (torch.randn(r, c, generator=g, device=device) * std).to(w.act_dtype)
 
     return ExpertWeight(up_w=n(I, H), gate_w=n(I, H), down_w=n(H, I))
 

@@ -179,6 +179,25 @@ ek_status ek_layer_profile(ek_layer *layer, int32_t enable);
 /* Snapshot of the layer's counters (waits for recorded events to complete). */
 ek_status ek_layer_get_stats(ek_layer *layer, ek_stats *out);
 
+/* ---- chain of layers: consecutive MoE layers launched as one HIP graph ------
+ * The reference issues one ForwardReq per MoE layer from the attention side
+ * (qwen3_moe.py:89-104 is entered once per decoder layer); a chain runs L
+ * layer calls back to back on the device, x_{l+1} = y_l, with no host
+ * round trip: the calls are captured once into a hipGraph (grids depend only
+ * on T; segment lengths are read from device memory) and replayed.
+ *   layers [L]: same hidden / top_k / act_dtype / device; each keeps its own
+ *               experts and workspace and must outlive the chain
+ *   ids [L,T,K] int32, w [L,T,K] w_dtype, x [T,H] -> y [T,H]; device pointers.
+ * use_graph = 0 runs the same launches eagerly (the reference for graph tests).
+ * A graph is re-captured when T, a pointer or w_dtype changes.  stream as in
+ * ek_layer_forward (NULL = blocking on the library's stream); routing errors
+ * are reported by blocking calls. */
+typedef struct ek_chain ek_chain;
+ek_status ek_chain_create(ek_layer *const *layers, int32_t n_layers, ek_chain **out);
+ek_status ek_chain_forward(ek_chain *chain, const void *x, const int32_t *ids, const void *w,
+                           int32_t w_dtype, int64_t T, void *y, int32_t use_graph, void *stream);
+ek_status ek_chain_destroy(ek_chain *chain);
+
 /* ---- single expert object: the literal shape of trait Expert<T> ----------
  * construct (ffn/meta.rs:38), forward (:37), shape (:35).  Implemented as a
  * one-expert layer; max_rows bounds n of forward. */
