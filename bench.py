@@ -25,6 +25,24 @@ HBM_PEAK = 8.0e12        # B/s, MI355X HBM3E
 MFMA_PEAK_16 = 2.5e15    # FLOP/s, bf16/fp16 dense
 
 
+def measured_traffic(workload: str, stage: int, decode: bool):
+    """HBM bytes per launch of the dominant kernel, from the committed rocprofv3 --pmc
+    summary (FETCH_SIZE + WRITE_SIZE, scaled by a 1 GiB copy): profiles/pmc_traffic.json.
+    None when no profile of this workload has been committed."""
+    path = os.path.join(ROOT, "profiles", "pmc_traffic.json")
+    if not os.path.exists(path):
+        return None
+    table = json.load(open(path)).get(workload, {})
+    want = "ffn_stream_kernel" if decode else "ffn_tile_kernel"
+    nmat = ", 2" if stage == 1 else ", 1"
+    for name, t in table.items():
+        if want in name and name.split("E" + nmat)[0] != name and ("E" + nmat + ",") in name + ",":
+            return t["fetch_bytes"] + t["write_bytes"]
+        if want in name and ("E" + nmat + ">") in name:
+            return t["fetch_bytes"] + t["write_bytes"]
+    return None
+
+
 def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
     """Reference-equivalent CPU backend (libtorch ops of ffn/expert_torch.rs:81-84,
     grouped per expert, weighted sum of qwen3_moe.py:102-104) on the pairs routed to
@@ -208,6 +226,7 @@ def main():
                 "frac": dom_flops / dom_s / MFMA_PEAK_16, "traffic": None}
     roof.update({"kernel": dom_name, "kernel_us": k_us[dom], "algorithmic_bytes": dom_bytes,
                  "algorithmic_flops": dom_flops})
+    roof["traffic"] = measured_traffic(w.name, dom, decode=hbm_frac >= mfma_frac)
 
     out = {
         "metric": "token-expert pairs/s on 1 MI355X (DSv3 W8A16 layer); % HBM / MFMA roofline",

@@ -100,6 +100,9 @@ struct ek_layer {
     void *st_raw = nullptr;                  // raw weight bytes during ingestion
     size_t st_raw_bytes = 0;
     hipStream_t load_stream = nullptr;
+    // the two FFN kernel families work on disjoint items, so their chains run side by side
+    hipStream_t side_stream = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
 
     ek_stats stats{};
     std::mutex stats_mu;
@@ -158,6 +161,9 @@ void free_layer(ek_layer *L)
     if (L->h_err) (void)hipHostFree(L->h_err);
     if (L->stream) (void)hipStreamDestroy(L->stream);
     if (L->load_stream) (void)hipStreamDestroy(L->load_stream);
+    if (L->side_stream) (void)hipStreamDestroy(L->side_stream);
+    if (L->ev_fork) (void)hipEventDestroy(L->ev_fork);
+    if (L->ev_join) (void)hipEventDestroy(L->ev_join);
     delete L;
 }
 
@@ -228,6 +234,9 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         if (e == hipSuccess) e = hipHostMalloc((void **)&L->h_err, sizeof(int32_t) * 4, hipHostMallocDefault);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->load_stream, hipStreamNonBlocking);
+        if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->side_stream, hipStreamNonBlocking);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_fork, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_join, hipEventDisableTiming);
         if (e != hipSuccess) st = hip_fail(e, "layer setup");
     }
     if (st != EK_OK) {
@@ -450,11 +459,32 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
         if (cap[l] > L->list_cap[l]) cap[l] = L->list_cap[l];
         if (cap[l] < 0) cap[l] = 0;
     }
+    // Two independent chains: the weight-streaming kernel (items of <= 16 rows) and the
+    // MFMA tile kernel (longer items) touch disjoint rows of h and out.  In the middle
+    // regime (a few to a few dozen rows per expert on average) both have real work of
+    // similar size and run side by side: the tile chain is forked to the side stream and
+    // joined before returning.  In the decode regime the tile lists are (nearly) empty and
+    // in the prefill regime the streaming list is short, and measured on MI355X the
+    // fork/join then costs more than it hides, so those run in order on s.
+    const bool tiles_main = P > 16 * E;
+    const bool have_stream = cap[ek::kListStream] > 0;
+    const bool have_tiles = cap[ek::kListT32] + cap[ek::kListT64] + cap[ek::kListT128] > 0;
+    const bool fork = have_stream && have_tiles && P > 4 * E && P <= 64 * E;
+    hipStream_t s_stream = s, s_tiles = s;
+    if (fork) {
+        EK_HIP(hipEventRecord(L->ev_fork, s));
+        EK_HIP(hipStreamWaitEvent(L->side_stream, L->ev_fork, 0));
+        (tiles_main ? s_stream : s_tiles) = L->side_stream;
+    }
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
-        EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->w8, cap[ek::kListStream], s));
-        EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->w8, cap, s));
+        if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->w8, cap[ek::kListStream], s_stream));
+        if (have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->w8, cap, s_tiles));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
+    }
+    if (fork) {
+        EK_HIP(hipEventRecord(L->ev_join, L->side_stream));
+        EK_HIP(hipStreamWaitEvent(s, L->ev_join, 0));
     }
     return EK_OK;
 }

@@ -3,62 +3,114 @@
 // Same arithmetic as the weight-streaming kernel (TorchFFN's closure,
 // ek-computation/src/ffn/expert_torch.rs:81-84, with its storage roundings),
 // for segments long enough that the contraction, not weight traffic, is the
-// cost.  One workgroup of four wavefronts owns one work item (BM = 16*MR rows
-// of one expert) x BN output channels:
-//   - the four waves split the channels; each wave keeps every row of the
-//     tile, so a weight element is fetched and dequantised once per workgroup,
-//     straight from the chunked HBM layout into MFMA "A" operands (no LDS);
-//   - the activation rows (gathered through row_token for stage 1) are staged
-//     global -> registers -> LDS in 64-wide k steps, double buffered, one
-//     barrier per step, and read back as MFMA "B" operands by all four waves;
-//     rows are padded to 72 elements so the 16-byte fragment reads of 16 lanes
-//     fall in 16 distinct bank groups;
-//   - fp32 accumulators: MR x NR x NMAT tiles of 16x16 per wave.
-// Workgroups are numbered so that each XCD walks a contiguous range of
-// (item, channel block) pairs: neighbours share the activation tile and, for
-// the tiles of one expert, the weights, in that XCD's L2.
+// cost.  One workgroup of eight wavefronts (two per SIMD, one workgroup per CU)
+// owns one work item (BM = 16*MR rows of one expert) x BN output channels:
+//   - the eight waves split the channels; each wave keeps every row of the
+//     tile, so a weight element is fetched and dequantised once per workgroup;
+//   - everything is brought in by LDS-DMA (global_load_lds_dwordx4: global ->
+//     LDS without passing through registers), three stages deep: while step s
+//     is being multiplied, the loads of steps s+1 and s+2 are in flight.  The
+//     weight chunks of a wave land in a wave-private region in exactly the
+//     chunked HBM layout (lane l's 16 bytes at l*16), the activation rows
+//     (gathered through row_token for stage 1) in an XOR-swizzled tile whose
+//     16-byte fragment reads are bank-conflict free;
+//   - completion is tracked by hand: the DMA is issued from inline asm, so the
+//     only vector-memory operations of a wave in the main loop are its own
+//     DMAs, in program order, and `s_waitcnt vmcnt(n)` with n = the DMAs of
+//     the younger stage is exact; one s_barrier per step publishes the
+//     activation tile and retires the stage that is overwritten next;
+//   - MFMA 32x32x16 (weights as the A operand: 32 channels x 16 k; activation
+//     rows as B: 16 k x 32 rows): one wavefront alone keeps the matrix pipe
+//     full with it (one issue per 32 cycles), which 16x16x32 does not; fp32
+//     accumulators: (MR/2) x 2 tiles of 32x32 per wave;
+// Each XCD walks a contiguous eighth of every work list, so neighbouring
+// workgroups share the activation tile and mostly the expert's weights in
+// that XCD's L2.
 #include "ek_internal.h"
 #include "ek_mfma.h"
 
 namespace ek {
 
+typedef __attribute__((address_space(3))) void *lds_ptr;
+
+// One LDS-DMA of 16 bytes per lane: lane l's bytes land at lds_addr + l*16.
+// lds_addr must be wave-uniform (it travels in M0).
+__device__ __forceinline__ void dma16(const void *gaddr, uint32_t lds_addr)
+{
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(gaddr), "s"(lds_addr)
+                 : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_vmcnt()
+{
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+__device__ __forceinline__ void block_barrier()
+{
+    asm volatile("s_barrier" : : : "memory");
+}
+
+constexpr int kTileThreads = 512;
+constexpr int kTileWaves = 8;
+constexpr int kTileStages = 3;
+
+template <bool W8> struct TileGeom {
+    static constexpr int BK = W8 ? 64 : 32;          // contraction elements per step = per weight chunk
+    static constexpr int PPR = BK / 8;               // 16-byte pieces per activation row and step
+    static constexpr int XS = 128 * BK * 2;          // bytes of a 128-row activation stage
+    static constexpr int WS = kTileWaves * 4 * kChunkBytes;
+    static constexpr int STAGE = XS + WS;
+};
+
+// XOR key of a row: fragment reads of 16 consecutive rows and one piece index
+// hit 16 distinct 16-byte bank groups (also 8 distinct ones per half).
+template <int PPR> __device__ __forceinline__ int swizzle_key(int row)
+{
+    if constexpr (PPR == 8) return (row & 7) ^ ((row >> 3) & 1);
+    else return ((row >> 1) & 3) ^ ((row >> 3) & 1);
+}
+
 template <typename T, bool W8, int NMAT, int MR>
-__device__ __forceinline__ void tile_body(const FfnArgs &a, const WorkItem item, const int nb, T *smem)
+__device__ __forceinline__ void tile_body(const FfnArgs &a, const WorkItem item, const int nb,
+                                          uint8_t *lds, const uint32_t lds_base)
 {
     using V8 = typename Act<T>::V8;
+    using G = TileGeom<W8>;
     constexpr int NR = NMAT == 2 ? 2 : 4;      // channel tiles per wave and matrix
+    constexpr int NWC = NR * NMAT;             // weight chunks per wave and step (always 4)
     constexpr int BM = MR * 16;
-    constexpr int BK = 64;                      // contraction elements per step
-    constexpr int LDK = BK + 8;                 // padded LDS row
-    constexpr int KE = W8 ? 64 : 32;            // contraction elements per weight chunk
-    constexpr int CPS = BK / KE;                // weight chunks per step, channel tile and matrix
-    constexpr int XP = BM * 8 / 256;            // 16-byte pieces of the x tile per thread and step
-    constexpr int NWC = NR * NMAT * CPS;        // weight chunks per step per wave
-    typedef T XTile[BM][LDK];
-    XTile *sX = reinterpret_cast<XTile *>(smem);   // [2][BM][LDK]
+    constexpr int BK = G::BK, PPR = G::PPR;
+    constexpr int XINSTR = BM * PPR / 64;      // DMA instructions per activation stage
+    constexpr int LX = (XINSTR + kTileWaves - 1) / kTileWaves;   // ... per wave
+    constexpr int LOADS = NWC + LX;            // DMAs per wave and stage
+    static_assert(NWC == 4, "wave-private weight region holds 4 chunks");
 
     const int e = item.expert, row0 = item.row0, nrows = item.nrows;
     const ExpertSlab slab = a.slabs[e];
     const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
     if (wmat == nullptr) return;                // expert not loaded: pack has flagged the call
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int j = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15;
     const int NT = a.N >> 4;
-    const int KT = a.Kdim / KE;                 // chunks along k
-    const int nsteps = a.Kdim / BK;
+    const int KT = a.Kdim / BK;                 // chunks along k = steps
+    const int nsteps = KT;
 
-    // ---- x tile: global -> LDS assignment -------------------------------------
-    const T *xsrc[XP];
-    int xdst[XP];
+    // ---- activation tile: which 16 bytes this lane brings in ------------------
+    const T *xsrc[LX];
+    uint32_t xdst[LX];
 #pragma unroll
-    for (int i = 0; i < XP; ++i) {
-        const int p = tid + i * 256;
-        const int r = p >> 3, c = p & 7;
-        const int rr = min(r, nrows - 1);       // rows past the item re-read its last row
+    for (int i = 0; i < LX; ++i) {
+        const int q = (wave + i * kTileWaves) % XINSTR;    // surplus waves repeat an instruction
+        const int sidx = q * 64 + lane;
+        const int r = sidx / PPR, ps = sidx % PPR;
+        const int c = ps ^ swizzle_key<PPR>(r);
+        const int rr = min(r, nrows - 1);                   // rows past the item re-read its last row
         const int64_t row = a.rows ? (int64_t)a.rows[row0 + rr] : (int64_t)(row0 + rr);
         xsrc[i] = (const T *)a.x + row * a.x_stride + c * 8;
-        xdst[i] = r * LDK + c * 8;
+        xdst[i] = q * 1024;
     }
 
     // ---- weights: this wave's channel tiles -------------------------------------
@@ -67,7 +119,7 @@ __device__ __forceinline__ void tile_body(const FfnArgs &a, const WorkItem item,
     int ct[NR];
 #pragma unroll
     for (int nr = 0; nr < NR; ++nr) {
-        ct[nr] = (nb * 4 + wave) * NR + nr;
+        ct[nr] = (nb * kTileWaves + wave) * NR + nr;
         const int ctc = min(ct[nr], NT - 1);    // channel tiles past N recompute the last one
         wp[nr] = wmat + (int64_t)ctc * KT * (NMAT * kChunkBytes) + lane * 16;
 #pragma unroll
@@ -81,111 +133,181 @@ __device__ __forceinline__ void tile_body(const FfnArgs &a, const WorkItem item,
             wc[nr][m] = -128.f * sv;
         }
     }
+    const uint32_t w_off = G::XS + wave * (NWC * kChunkBytes);   // wave-private weight region
 
-    f32x4 acc[MR][NR][NMAT];
-#pragma unroll
-    for (int mr = 0; mr < MR; ++mr)
-#pragma unroll
-        for (int nr = 0; nr < NR; ++nr)
-#pragma unroll
-            for (int m = 0; m < NMAT; ++m) acc[mr][nr][m] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-    uint4 wcur[NWC], wnext[NWC], xreg[XP];
-
-#define EK_LOAD_W(dst, step)                                                                   \
-    _Pragma("unroll") for (int nr = 0; nr < NR; ++nr)                                          \
-    _Pragma("unroll") for (int c = 0; c < CPS; ++c)                                            \
-    _Pragma("unroll") for (int m = 0; m < NMAT; ++m)                                           \
-        dst[(nr * CPS + c) * NMAT + m] =                                                       \
-            ldg16(wp[nr] + (int64_t)(((step) * CPS + c) * NMAT + m) * kChunkBytes)
-#define EK_LOAD_X(step)                                                                        \
-    _Pragma("unroll") for (int i = 0; i < XP; ++i) xreg[i] = ldg16(xsrc[i] + (step) * BK)
-#define EK_STORE_X(buf)                                                                        \
-    _Pragma("unroll") for (int i = 0; i < XP; ++i) *(uint4 *)(&sX[buf][0][0] + xdst[i]) = xreg[i]
-
-    EK_LOAD_X(0);
-    EK_LOAD_W(wcur, 0);
-    EK_STORE_X(0);
-    __syncthreads();
-
-    for (int step = 0; step < nsteps; ++step) {
-        const int buf = step & 1;
-        const bool more = step + 1 < nsteps;
-        if (more) {
-            EK_LOAD_X(step + 1);
-            EK_LOAD_W(wnext, step + 1);
-        }
-        // two MFMA k-groups of 32 per step
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            V8 af[NR][NMAT];
-#pragma unroll
-            for (int nr = 0; nr < NR; ++nr)
-#pragma unroll
-                for (int m = 0; m < NMAT; ++m) {
-                    if constexpr (W8) {
-                        const uint4 q = wcur[nr * NMAT + m];
-                        af[nr][m] = h == 0 ? dequant_u8x8<T>(q.x, q.y, ws[nr][m], wc[nr][m])
-                                           : dequant_u8x8<T>(q.z, q.w, ws[nr][m], wc[nr][m]);
-                    } else {
-                        af[nr][m] = __builtin_bit_cast(V8, wcur[(nr * CPS + h) * NMAT + m]);
-                    }
-                }
-            // lane (j, g) supplies k = g*16 + h*8 .. +8 (int8 chunk order) or h*32 + g*8 .. +8
-            const int koff = W8 ? g * 16 + h * 8 : h * 32 + g * 8;
-#pragma unroll
-            for (int mr = 0; mr < MR; ++mr) {
-                const V8 bf = *(const V8 *)&sX[buf][mr * 16 + j][koff];
-#pragma unroll
-                for (int nr = 0; nr < NR; ++nr)
-#pragma unroll
-                    for (int m = 0; m < NMAT; ++m)
-                        acc[mr][nr][m] = Act<T>::mfma(af[nr][m], bf, acc[mr][nr][m]);
-            }
-        }
-        if (more) {
-            EK_STORE_X(buf ^ 1);
-#pragma unroll
-            for (int i = 0; i < NWC; ++i) wcur[i] = wnext[i];
-        }
-        __syncthreads();
+#define EK_ISSUE(step)                                                                          \
+    {                                                                                           \
+        const uint32_t st_ = lds_base + ((step) % kTileStages) * G::STAGE;                      \
+        _Pragma("unroll") for (int nr = 0; nr < NR; ++nr)                                       \
+        _Pragma("unroll") for (int m = 0; m < NMAT; ++m)                                        \
+            dma16(wp[nr] + (int64_t)((step) * NMAT + m) * kChunkBytes,                          \
+                  st_ + w_off + (nr * NMAT + m) * kChunkBytes);                                 \
+        _Pragma("unroll") for (int i = 0; i < LX; ++i) dma16(xsrc[i] + (step) * BK, st_ + xdst[i]); \
     }
 
-    // ---- epilogue: lane (g, j) holds channels ct*16 + 4g + r of row mr*16 + j ----
+    // ---- MFMA 32x32x16 geometry ----------------------------------------------------
+    // The wave's 4 weight chunks (16 channels each) form CB = 2 column blocks of 32
+    // channels: {up, gate} of the same 32 channels (stage 1) or 64 consecutive channels
+    // (stage 2).  Lane l feeds channel l%32 and k-half kg = l/32 of the A operand, and row
+    // l%32 of a 32-row block of the B operand.  A 16-byte LDS read of weight slot
+    // (2*tt + kg) gives the lane the A operands of two MFMAs (int8) or one (16-bit); the
+    // matching B operand is the 16-byte piece with the same k.
+    constexpr int CB = 2;
+    constexpr int RB = MR / 2;                 // 32-row blocks
+    constexpr int NGRP = BK / 16;              // MFMA k-groups per step (4 int8, 2 16-bit)
+    const int l32 = lane & 31, kg = lane >> 5, hh = l32 >> 4;
+    f32x16 acc[RB < 1 ? 1 : RB][CB];
+    constexpr int RBn = RB < 1 ? 1 : RB;
+#pragma unroll
+    for (int rb = 0; rb < RBn; ++rb)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.f;
+
+    int aoff[CB];
+    float as[CB], ac[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        // chunk (nr, m) sits at index nr*NMAT + m of the wave's region
+        const int nr = NMAT == 2 ? hh : cb * 2 + hh, m = NMAT == 2 ? cb : 0;
+        aoff[cb] = (nr * NMAT + m) * kChunkBytes + kg * 256 + j * 16;
+        // per-lane dequantisation constants of that channel
+        as[cb] = hh ? ws[NMAT == 2 ? 1 : cb * 2 + 1][m] : ws[NMAT == 2 ? 0 : cb * 2][m];
+        ac[cb] = -128.f * as[cb];
+    }
+    // B fragment offsets of the step's k-groups for row block 0 (bytes inside a stage)
+    int boff[NGRP];
+#pragma unroll
+    for (int grp = 0; grp < NGRP; ++grp) {
+        const int c = W8 ? ((grp >> 1) * 2 + kg) * 2 + (grp & 1) : grp * 2 + kg;
+        boff[grp] = (l32 * PPR + (c ^ swizzle_key<PPR>(j))) * 16;
+    }
+    constexpr int kRowBlockBytes = 32 * PPR * 16;
+
+    EK_ISSUE(0);
+    if (nsteps > 1) EK_ISSUE(1);
+
+    for (int step = 0; step < nsteps; ++step) {
+        // the DMAs of this step are older than those of step+1: wait until only the latter remain
+#ifndef EK_ABL_NOSYNC
+        if (step + 1 < nsteps) wait_vmcnt<LOADS>();
+        else wait_vmcnt<0>();
+        block_barrier();   // tile of `step` visible to all waves; stage of step-1 is free again
+#endif
+#ifndef EK_ABL_NODMA
+        if (step + 2 < nsteps) EK_ISSUE(step + 2);
+#endif
+
+        const uint8_t *stage = lds + (step % kTileStages) * G::STAGE;
+        const uint8_t *wreg = stage + w_off;
+        u32x4 aq[2][CB];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) aq[tt][cb] = *(const u32x4 *)(wreg + aoff[cb] + tt * 512);
+
+        // A operands of k-group grp: int8 -> half (grp & 1) of read grp >> 1, dequantised;
+        // 16-bit -> read grp as it is.  Software pipeline, pinned with scheduling fences:
+        // per row block 2 MFMAs, the B fragment read of the next k-group, and a quarter of
+        // the next k-group's dequantisation.
+        u32x4 af[2][CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            if constexpr (W8) {
+                const u32x2 lo = dequant_u8x4<T>(aq[0][cb][0], as[cb], ac[cb]);
+                const u32x2 hi = dequant_u8x4<T>(aq[0][cb][1], as[cb], ac[cb]);
+                af[0][cb] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+            } else {
+                af[0][cb] = aq[0][cb];
+            }
+        }
+        V8 bf[2][RBn];
+#pragma unroll
+        for (int rb = 0; rb < RBn; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
+#pragma unroll
+        for (int grp = 0; grp < NGRP; ++grp) {
+            const int cur = grp & 1, nxt = cur ^ 1;
+#pragma unroll
+            for (int rb = 0; rb < RBn; ++rb) {
+                if (grp + 1 < NGRP) bf[nxt][rb] = *(const V8 *)(stage + boff[grp + 1] + rb * kRowBlockBytes);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+#ifdef EK_ABL_NOMFMA
+                    acc[rb][cb][0] += (float)bf[cur][rb][0] * (float)__builtin_bit_cast(V8, af[cur][cb])[0];
+#else
+                    acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cur][cb]), bf[cur][rb], acc[rb][cb]);
+#endif
+                if (grp + 1 < NGRP) {
+                    if constexpr (W8) {
+                        // next group's A operands: 4 dwords (2 per column block), spread over the row blocks
+                        constexpr int DW = 4 / RBn;
+#pragma unroll
+                        for (int d = 0; d < DW; ++d) {
+                            const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
+                            const int g1 = grp + 1;
+                            const uint32_t w = aq[g1 >> 1][cb][(g1 & 1) * 2 + part];
+                            const u32x2 v = dequant_u8x4<T>(w, as[cb], ac[cb]);
+                            af[nxt][cb][part * 2] = v[0];
+                            af[nxt][cb][part * 2 + 1] = v[1];
+                        }
+                    } else {
+                        if (rb == 0) {
+#pragma unroll
+                            for (int cb = 0; cb < CB; ++cb) af[nxt][cb] = aq[grp + 1][cb];
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+#undef EK_ISSUE
+
+    // ---- epilogue: lane holds, for row rb*32 + l%32, channels q*8 + kg*4 + (0..3), q = 0..3,
+    //      of each column block ----
     typedef T T4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int mr = 0; mr < MR; ++mr) {
-        const int r_in = mr * 16 + j;
+    for (int rb = 0; rb < RBn; ++rb) {
+        const int r_in = rb * 32 + l32;
         if (r_in >= nrows) continue;
         T *orow = (T *)a.out + (int64_t)(row0 + r_in) * a.out_stride;
+        if constexpr (NMAT == 2) {
+            const int cbase = (nb * kTileWaves + wave) * 32;     // 32 channels of up and gate
+            if (cbase >= a.N) continue;
 #pragma unroll
-        for (int nr = 0; nr < NR; ++nr) {
-            if (ct[nr] >= NT) continue;
-            T4 o;
+            for (int q = 0; q < 4; ++q) {
+                T4 o;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if constexpr (NMAT == 2) o[r] = swiglu_rounded<T>(acc[mr][nr][0][r], acc[mr][nr][1][r]);
-                else o[r] = (T)acc[mr][nr][0][r];
+                for (int r = 0; r < 4; ++r) o[r] = swiglu_rounded<T>(acc[rb][0][q * 4 + r], acc[rb][1][q * 4 + r]);
+                *(uint2 *)(orow + cbase + q * 8 + kg * 4) = __builtin_bit_cast(uint2, o);
             }
-            *(uint2 *)(orow + ct[nr] * 16 + 4 * g) = __builtin_bit_cast(uint2, o);
+        } else {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                const int cbase = (nb * kTileWaves + wave) * 64 + cb * 32;
+                if (cbase >= a.N) continue;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    T4 o;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[r] = (T)acc[rb][cb][q * 4 + r];
+                    *(uint2 *)(orow + cbase + q * 8 + kg * 4) = __builtin_bit_cast(uint2, o);
+                }
+            }
         }
     }
 }
 
-#undef EK_LOAD_W
-#undef EK_LOAD_X
-#undef EK_STORE_X
-
 // One launch covers the three tile lists.  Workgroup b runs on XCD b % 8
 // (round-robin dispatch), so each XCD is given a contiguous eighth of every
 // list: first its 128-row items, then its 64-row, then its 32-row ones, each
-// times nb_count channel blocks.  Neighbouring workgroups of an XCD then share
-// the activation tile (same item) and mostly the expert's weights in its L2,
-// and every XCD gets the same mix of long and short items.
+// times nb_count channel blocks.
 template <typename T, bool W8, int NMAT>
-__global__ __launch_bounds__(256, 2) void ffn_tile_kernel(FfnArgs a, int nb_count)
+__global__ __launch_bounds__(kTileThreads, 1) void ffn_tile_kernel(FfnArgs a, int nb_count)
 {
-    __shared__ __attribute__((aligned(16))) T smem[2 * 128 * (64 + 8)];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kTileStages * TileGeom<W8>::STAGE];
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)lds;
     const int x = blockIdx.x & 7;
     int i = blockIdx.x >> 3;
     const int n128 = a.lists.count[kListT128], n64 = a.lists.count[kListT64], n32 = a.lists.count[kListT32];
@@ -193,17 +315,17 @@ __global__ __launch_bounds__(256, 2) void ffn_tile_kernel(FfnArgs a, int nb_coun
     const int lo64 = x * n64 / 8, s64 = (x + 1) * n64 / 8 - lo64;
     const int lo32 = x * n32 / 8, s32 = (x + 1) * n32 / 8 - lo32;
     if (i < s128 * nb_count) {
-        tile_body<T, W8, NMAT, 8>(a, a.lists.items[kListT128][lo128 + i / nb_count], i % nb_count, smem);
+        tile_body<T, W8, NMAT, 8>(a, a.lists.items[kListT128][lo128 + i / nb_count], i % nb_count, lds, lds_base);
         return;
     }
     i -= s128 * nb_count;
     if (i < s64 * nb_count) {
-        tile_body<T, W8, NMAT, 4>(a, a.lists.items[kListT64][lo64 + i / nb_count], i % nb_count, smem);
+        tile_body<T, W8, NMAT, 4>(a, a.lists.items[kListT64][lo64 + i / nb_count], i % nb_count, lds, lds_base);
         return;
     }
     i -= s64 * nb_count;
     if (i < s32 * nb_count)
-        tile_body<T, W8, NMAT, 2>(a, a.lists.items[kListT32][lo32 + i / nb_count], i % nb_count, smem);
+        tile_body<T, W8, NMAT, 2>(a, a.lists.items[kListT32][lo32 + i / nb_count], i % nb_count, lds, lds_base);
 }
 
 template <typename T, bool W8, int NMAT>
@@ -211,12 +333,13 @@ static hipError_t launch_t(const FfnArgs &a, const int64_t max_items[kNumLists],
 {
     constexpr int NR = NMAT == 2 ? 2 : 4;
     const int NT = a.N / 16;
-    const int nb_count = (NT + 4 * NR - 1) / (4 * NR);
+    const int nb_count = (NT + kTileWaves * NR - 1) / (kTileWaves * NR);
     const int64_t per_xcd = (max_items[kListT128] + 7) / 8 + (max_items[kListT64] + 7) / 8 +
                             (max_items[kListT32] + 7) / 8;
     const int64_t blocks = per_xcd * nb_count * 8;
     if (blocks <= 0) return hipSuccess;
-    hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT>), dim3((unsigned)blocks), dim3(256), 0, s, a, nb_count);
+    hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT>), dim3((unsigned)blocks), dim3(kTileThreads), 0, s, a,
+                       nb_count);
     return hipGetLastError();
 }
 

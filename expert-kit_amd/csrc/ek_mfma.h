@@ -8,6 +8,7 @@ namespace ek {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 template <typename T> struct Act;
 template <> struct Act<__bf16> {
@@ -16,12 +17,20 @@ template <> struct Act<__bf16> {
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
 };
 template <> struct Act<_Float16> {
     using V8 = f16x8;
     static __device__ __forceinline__ f32x4 mfma(V8 a, V8 b, f32x4 c)
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x16 mfma32(V8 a, V8 b, f32x16 c)
+    {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
 };
 
@@ -54,6 +63,17 @@ template <> __device__ __forceinline__ uint32_t pack2<_Float16>(float lo, float 
     typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
     const f32x2 v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
+// 4 offset-binary bytes (one dword) of one output channel -> 4 dequantised weights
+// rne_T((u - 128) * s) as two packed dwords; c = -128 * s
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+template <typename T> __device__ __forceinline__ u32x2 dequant_u8x4(uint32_t w, float s, float c)
+{
+    u32x2 r;
+    r[0] = pack2<T>(__builtin_fmaf((float)(w & 0xffu), s, c), __builtin_fmaf((float)((w >> 8) & 0xffu), s, c));
+    r[1] = pack2<T>(__builtin_fmaf((float)((w >> 16) & 0xffu), s, c), __builtin_fmaf((float)(w >> 24), s, c));
+    return r;
 }
 
 // 8 offset-binary bytes (two dwords) of one output channel -> 8 dequantised
