@@ -14,7 +14,9 @@
 //     16-byte load per lane straight from the chunked HBM layout (no LDS);
 //   - the <= 16 activation rows of the segment are the "B" operand (32 k x 16
 //     rows), re-read from L2 by every wave;
-//   - D loads deep software prefetch keeps >= D KiB per wave in flight.
+//   - D loads deep software prefetch keeps >= D KiB per wave in flight
+//     (measured best on MI355X: one channel tile of up+gate per wave, 8 deep,
+//     for stage 1; two channel tiles, 8 deep, for stage 2).
 // int8 weights are dequantised in registers to exactly the tensor a CPU backend
 // would hold, W[n,k] = rne_16bit(f32(q[n,k]) * f32(scale[n])): they are stored
 // offset-binary (u = q + 128) so v_cvt_f32_ubyteN converts them, one
@@ -155,29 +157,44 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(FfnArgs a)
     }
 }
 
-template <typename T, bool W8, int NMAT, int NG>
+// Tuned on MI355X at the DeepSeek-V3 shape (see the profiles): channel tiles per wave (NG)
+// and prefetch depth in k steps (D) per stage.
+#ifndef EK_TUNE_S1_NG
+#define EK_TUNE_S1_NG 1
+#endif
+#ifndef EK_TUNE_S1_D
+#define EK_TUNE_S1_D 8
+#endif
+#ifndef EK_TUNE_S2_NG
+#define EK_TUNE_S2_NG 2
+#endif
+#ifndef EK_TUNE_S2_D
+#define EK_TUNE_S2_D 8
+#endif
+
+template <typename T, bool W8, int NMAT, int NG, int D>
 static hipError_t launch_d(const FfnArgs &a, int32_t nseg, hipStream_t s)
 {
     constexpr int KE = W8 ? 64 : 32;
     const int KT = a.Kdim / KE;
     const int NT = a.N / 16;
+    if constexpr (D > 1) {
+        if (KT % D != 0) return launch_d<T, W8, NMAT, NG, D / 2>(a, nseg, s);
+    }
     dim3 grid((NT + 4 * NG - 1) / (4 * NG), nseg);
-    if (KT % 4 == 0)
-        hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, 4>), grid, dim3(256), 0, s, a);
-    else if (KT % 2 == 0)
-        hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, 2>), grid, dim3(256), 0, s, a);
-    else
-        hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, 1>), grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, D>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
 template <typename T, bool W8, int NMAT>
 static hipError_t launch_g(const FfnArgs &a, int32_t nseg, hipStream_t s)
 {
+    constexpr int NG = NMAT == 2 ? EK_TUNE_S1_NG : EK_TUNE_S2_NG;
+    constexpr int D = NMAT == 2 ? EK_TUNE_S1_D : EK_TUNE_S2_D;
     const int NT = a.N / 16;
-    if (NMAT == 1 && NT % 4 == 0) return launch_d<T, W8, NMAT, 4>(a, nseg, s);
-    if (NT % 2 == 0) return launch_d<T, W8, NMAT, 2>(a, nseg, s);
-    return launch_d<T, W8, NMAT, 1>(a, nseg, s);
+    if (NT % NG == 0) return launch_d<T, W8, NMAT, NG, D>(a, nseg, s);
+    if (NT % 2 == 0) return launch_d<T, W8, NMAT, 2, D>(a, nseg, s);
+    return launch_d<T, W8, NMAT, 1, D>(a, nseg, s);
 }
 
 hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items,
