@@ -175,8 +175,10 @@ ek_status validate_cfg(const ek_cfg *c)
     if (c->w_dtype != c->act_dtype && c->w_dtype != EK_I8)
         return fail(EK_INVALID_INPUT, "w_dtype must equal act_dtype or be EK_I8 (got %d)", c->w_dtype);
     const int64_t ke = 64;   // contraction step of the tile kernel; int8 chunk width
-    if (c->hidden <= 0 || c->inter <= 0 || c->hidden % ke || c->inter % ke)
-        return fail(EK_INVALID_INPUT, "hidden (%lld) and inter (%lld) must be positive multiples of %lld",
+    // the tile kernel's pipeline needs two contraction steps (64 wide for int8, 32 for 16-bit)
+    const int64_t kmin = c->w_dtype == EK_I8 ? 128 : 64;
+    if (c->hidden < kmin || c->inter < kmin || c->hidden % ke || c->inter % ke)
+        return fail(EK_INVALID_INPUT, "hidden (%lld) and inter (%lld) must be multiples of %lld (at least 128 for int8)",
                     (long long)c->hidden, (long long)c->inter, (long long)ke);
     if (c->n_experts < 1 || c->n_experts > ek::kMaxExperts)
         return fail(EK_INVALID_INPUT, "n_experts must be in [1, %d] (got %d)", ek::kMaxExperts,

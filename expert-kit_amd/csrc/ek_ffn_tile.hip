@@ -54,6 +54,7 @@ __device__ __forceinline__ void block_barrier()
 constexpr int kTileThreads = 512;
 constexpr int kTileWaves = 8;
 constexpr int kTileStages = 3;
+constexpr int kCusPerXcd = 32;   // MI355X: 8 XCDs x 32 CUs
 
 template <bool W8> struct TileGeom {
     static constexpr int BK = W8 ? 64 : 32;          // contraction elements per step = per weight chunk
@@ -71,8 +72,22 @@ template <int PPR> __device__ __forceinline__ int swizzle_key(int row)
     else return ((row >> 1) & 3) ^ ((row >> 3) & 1);
 }
 
+// What one wavefront needs to know about one tile (work item x channel block).
+template <typename T, int NR, int LX> struct TileCtx {
+    const uint8_t *wp[NR];   // this lane's 16 bytes of the wave's weight chunks at step 0
+    const T *xsrc[LX];       // this lane's 16-byte pieces of the activation tile at step 0
+    float as[2], ac[2];      // dequantisation constants of the lane's channel, per column block
+    int row0, nrows;         // the item's packed rows
+    int chan0;               // first output channel of the wave's block
+};
+
+// All tiles of one class (MR*16-row items) that fall to this workgroup: tiles first,
+// first + stride, ... of `ntiles`, tile = (item, channel block).  The LDS-DMA pipeline
+// runs across tile boundaries: the first two steps of the next tile are issued during the
+// last two steps of the current one, so only the epilogue separates two tiles.
 template <typename T, bool W8, int NMAT, int MR>
-__device__ __forceinline__ void tile_body(const FfnArgs &a, const WorkItem item, const int nb,
+__device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *items, const int ntiles,
+                                          const int nb_count, const int first, const int stride,
                                           uint8_t *lds, const uint32_t lds_base)
 {
     using V8 = typename Act<T>::V8;
@@ -84,248 +99,261 @@ __device__ __forceinline__ void tile_body(const FfnArgs &a, const WorkItem item,
     constexpr int XINSTR = BM * PPR / 64;      // DMA instructions per activation stage
     constexpr int LX = (XINSTR + kTileWaves - 1) / kTileWaves;   // ... per wave
     constexpr int LOADS = NWC + LX;            // DMAs per wave and stage
+    constexpr int CB = 2;                      // column blocks of 32 channels per wave
+    constexpr int RB = MR / 2;                 // 32-row blocks
+    constexpr int NGRP = BK / 16;              // MFMA k-groups per step (4 int8, 2 16-bit)
+    constexpr int kRowBlockBytes = 32 * PPR * 16;
     static_assert(NWC == 4, "wave-private weight region holds 4 chunks");
+    static_assert(RB >= 1, "items have at least 32 rows");
+    typedef TileCtx<T, NR, LX> Ctx;
 
-    const int e = item.expert, row0 = item.row0, nrows = item.nrows;
-    const ExpertSlab slab = a.slabs[e];
-    const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
-    if (wmat == nullptr) return;                // expert not loaded: pack has flagged the call
-
+    if (first >= ntiles) return;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int j = lane & 15;
+    const int j = lane & 15, l32 = lane & 31, kg = lane >> 5, hh = l32 >> 4;
     const int NT = a.N >> 4;
-    const int KT = a.Kdim / BK;                 // chunks along k = steps
-    const int nsteps = KT;
+    const int nsteps = a.Kdim / BK;             // >= 2 (hidden, inter >= 128)
 
-    // ---- activation tile: which 16 bytes this lane brings in ------------------
-    const T *xsrc[LX];
+    // ---- tile-independent lane constants ---------------------------------------
+    // activation tile: DMA instruction q brings pieces q*64 .. q*64+63 (row-major, PPR per
+    // row, piece index XOR-swizzled by the row's key)
+    int xrow[LX], xcol[LX];
     uint32_t xdst[LX];
 #pragma unroll
     for (int i = 0; i < LX; ++i) {
         const int q = (wave + i * kTileWaves) % XINSTR;    // surplus waves repeat an instruction
         const int sidx = q * 64 + lane;
-        const int r = sidx / PPR, ps = sidx % PPR;
-        const int c = ps ^ swizzle_key<PPR>(r);
-        const int rr = min(r, nrows - 1);                   // rows past the item re-read its last row
-        const int64_t row = a.rows ? (int64_t)a.rows[row0 + rr] : (int64_t)(row0 + rr);
-        xsrc[i] = (const T *)a.x + row * a.x_stride + c * 8;
+        xrow[i] = sidx / PPR;
+        xcol[i] = ((sidx % PPR) ^ swizzle_key<PPR>(xrow[i])) * 8;
         xdst[i] = q * 1024;
     }
-
-    // ---- weights: this wave's channel tiles -------------------------------------
-    const uint8_t *wp[NR];
-    float ws[NR][NMAT], wc[NR][NMAT];
-    int ct[NR];
-#pragma unroll
-    for (int nr = 0; nr < NR; ++nr) {
-        ct[nr] = (nb * kTileWaves + wave) * NR + nr;
-        const int ctc = min(ct[nr], NT - 1);    // channel tiles past N recompute the last one
-        wp[nr] = wmat + (int64_t)ctc * KT * (NMAT * kChunkBytes) + lane * 16;
-#pragma unroll
-        for (int m = 0; m < NMAT; ++m) {
-            float sv = 1.f;
-            if constexpr (W8) {
-                const int ch = ctc * 16 + j;
-                sv = NMAT == 2 ? (m == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
-            }
-            ws[nr][m] = sv;
-            wc[nr][m] = -128.f * sv;
-        }
-    }
     const uint32_t w_off = G::XS + wave * (NWC * kChunkBytes);   // wave-private weight region
-
-#define EK_ISSUE(step)                                                                          \
-    {                                                                                           \
-        const uint32_t st_ = lds_base + ((step) % kTileStages) * G::STAGE;                      \
-        _Pragma("unroll") for (int nr = 0; nr < NR; ++nr)                                       \
-        _Pragma("unroll") for (int m = 0; m < NMAT; ++m)                                        \
-            dma16(wp[nr] + (int64_t)((step) * NMAT + m) * kChunkBytes,                          \
-                  st_ + w_off + (nr * NMAT + m) * kChunkBytes);                                 \
-        _Pragma("unroll") for (int i = 0; i < LX; ++i) dma16(xsrc[i] + (step) * BK, st_ + xdst[i]); \
-    }
-
-    // ---- MFMA 32x32x16 geometry ----------------------------------------------------
-    // The wave's 4 weight chunks (16 channels each) form CB = 2 column blocks of 32
-    // channels: {up, gate} of the same 32 channels (stage 1) or 64 consecutive channels
-    // (stage 2).  Lane l feeds channel l%32 and k-half kg = l/32 of the A operand, and row
-    // l%32 of a 32-row block of the B operand.  A 16-byte LDS read of weight slot
-    // (2*tt + kg) gives the lane the A operands of two MFMAs (int8) or one (16-bit); the
-    // matching B operand is the 16-byte piece with the same k.
-    constexpr int CB = 2;
-    constexpr int RB = MR / 2;                 // 32-row blocks
-    constexpr int NGRP = BK / 16;              // MFMA k-groups per step (4 int8, 2 16-bit)
-    const int l32 = lane & 31, kg = lane >> 5, hh = l32 >> 4;
-    f32x16 acc[RB < 1 ? 1 : RB][CB];
-    constexpr int RBn = RB < 1 ? 1 : RB;
-#pragma unroll
-    for (int rb = 0; rb < RBn; ++rb)
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.f;
-
+    // MFMA 32x32x16 operands.  The wave's 4 weight chunks (16 channels each) form CB = 2
+    // column blocks of 32 channels: {up, gate} of the same 32 channels (stage 1) or 64
+    // consecutive channels (stage 2).  Lane l feeds channel l%32 and k-half kg = l/32 of the
+    // A operand, and row l%32 of a 32-row block of the B operand.  A 16-byte LDS read of
+    // weight slot (2*tt + kg) gives the lane the A operands of two MFMAs (int8) or one
+    // (16-bit); the matching B operand is the 16-byte piece with the same k.
     int aoff[CB];
-    float as[CB], ac[CB];
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
-        // chunk (nr, m) sits at index nr*NMAT + m of the wave's region
         const int nr = NMAT == 2 ? hh : cb * 2 + hh, m = NMAT == 2 ? cb : 0;
         aoff[cb] = (nr * NMAT + m) * kChunkBytes + kg * 256 + j * 16;
-        // per-lane dequantisation constants of that channel
-        as[cb] = hh ? ws[NMAT == 2 ? 1 : cb * 2 + 1][m] : ws[NMAT == 2 ? 0 : cb * 2][m];
-        ac[cb] = -128.f * as[cb];
     }
-    // B fragment offsets of the step's k-groups for row block 0 (bytes inside a stage)
     int boff[NGRP];
 #pragma unroll
     for (int grp = 0; grp < NGRP; ++grp) {
         const int c = W8 ? ((grp >> 1) * 2 + kg) * 2 + (grp & 1) : grp * 2 + kg;
         boff[grp] = (l32 * PPR + (c ^ swizzle_key<PPR>(j))) * 16;
     }
-    constexpr int kRowBlockBytes = 32 * PPR * 16;
 
-    EK_ISSUE(0);
-    if (nsteps > 1) EK_ISSUE(1);
-
-    for (int step = 0; step < nsteps; ++step) {
-        // the DMAs of this step are older than those of step+1: wait until only the latter remain
-#ifndef EK_ABL_NOSYNC
-        if (step + 1 < nsteps) wait_vmcnt<LOADS>();
-        else wait_vmcnt<0>();
-        block_barrier();   // tile of `step` visible to all waves; stage of step-1 is free again
-#endif
-#ifndef EK_ABL_NODMA
-        if (step + 2 < nsteps) EK_ISSUE(step + 2);
-#endif
-
-        const uint8_t *stage = lds + (step % kTileStages) * G::STAGE;
-        const uint8_t *wreg = stage + w_off;
-        u32x4 aq[2][CB];
+    // Fills `c` for the first tile at or after index t (stepping by stride) whose expert is
+    // loaded; returns its index or -1.
+    auto fetch = [&](int t, Ctx &c) -> int {
+        for (; t < ntiles; t += stride) {
+            const WorkItem item = items[t / nb_count];
+            const int nb = t % nb_count;
+            const ExpertSlab slab = a.slabs[item.expert];
+            const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
+            if (wmat == nullptr) continue;       // not loaded: pack has flagged the call
+            c.row0 = item.row0;
+            c.nrows = item.nrows;
+            const int cblock = nb * kTileWaves + wave;
+            c.chan0 = cblock * NR * 16;
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) aq[tt][cb] = *(const u32x4 *)(wreg + aoff[cb] + tt * 512);
-
-        // A operands of k-group grp: int8 -> half (grp & 1) of read grp >> 1, dequantised;
-        // 16-bit -> read grp as it is.  Software pipeline, pinned with scheduling fences:
-        // per row block 2 MFMAs, the B fragment read of the next k-group, and a quarter of
-        // the next k-group's dequantisation.
-        u32x4 af[2][CB];
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            if constexpr (W8) {
-                const u32x2 lo = dequant_u8x4<T>(aq[0][cb][0], as[cb], ac[cb]);
-                const u32x2 hi = dequant_u8x4<T>(aq[0][cb][1], as[cb], ac[cb]);
-                af[0][cb] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
-            } else {
-                af[0][cb] = aq[0][cb];
+            for (int nr = 0; nr < NR; ++nr) {
+                const int ctc = min(cblock * NR + nr, NT - 1);   // tiles past N recompute the last one
+                c.wp[nr] = wmat + (int64_t)ctc * nsteps * (NMAT * kChunkBytes) + lane * 16;
             }
-        }
-        V8 bf[2][RBn];
-#pragma unroll
-        for (int rb = 0; rb < RBn; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
-#pragma unroll
-        for (int grp = 0; grp < NGRP; ++grp) {
-            const int cur = grp & 1, nxt = cur ^ 1;
-#pragma unroll
-            for (int rb = 0; rb < RBn; ++rb) {
-                if (grp + 1 < NGRP) bf[nxt][rb] = *(const V8 *)(stage + boff[grp + 1] + rb * kRowBlockBytes);
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb)
-#ifdef EK_ABL_NOMFMA
-                    acc[rb][cb][0] += (float)bf[cur][rb][0] * (float)__builtin_bit_cast(V8, af[cur][cb])[0];
-#else
-                    acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cur][cb]), bf[cur][rb], acc[rb][cb]);
-#endif
-                if (grp + 1 < NGRP) {
-                    if constexpr (W8) {
-                        // next group's A operands: 4 dwords (2 per column block), spread over the row blocks
-                        constexpr int DW = 4 / RBn;
-#pragma unroll
-                        for (int d = 0; d < DW; ++d) {
-                            const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
-                            const int g1 = grp + 1;
-                            const uint32_t w = aq[g1 >> 1][cb][(g1 & 1) * 2 + part];
-                            const u32x2 v = dequant_u8x4<T>(w, as[cb], ac[cb]);
-                            af[nxt][cb][part * 2] = v[0];
-                            af[nxt][cb][part * 2 + 1] = v[1];
-                        }
-                    } else {
-                        if (rb == 0) {
-#pragma unroll
-                            for (int cb = 0; cb < CB; ++cb) af[nxt][cb] = aq[grp + 1][cb];
-                        }
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    }
-#undef EK_ISSUE
-
-    // ---- epilogue: lane holds, for row rb*32 + l%32, channels q*8 + kg*4 + (0..3), q = 0..3,
-    //      of each column block ----
-    typedef T T4 __attribute__((ext_vector_type(4)));
-#pragma unroll
-    for (int rb = 0; rb < RBn; ++rb) {
-        const int r_in = rb * 32 + l32;
-        if (r_in >= nrows) continue;
-        T *orow = (T *)a.out + (int64_t)(row0 + r_in) * a.out_stride;
-        if constexpr (NMAT == 2) {
-            const int cbase = (nb * kTileWaves + wave) * 32;     // 32 channels of up and gate
-            if (cbase >= a.N) continue;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                T4 o;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) o[r] = swiglu_rounded<T>(acc[rb][0][q * 4 + r], acc[rb][1][q * 4 + r]);
-                *(uint2 *)(orow + cbase + q * 8 + kg * 4) = __builtin_bit_cast(uint2, o);
-            }
-        } else {
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
-                const int cbase = (nb * kTileWaves + wave) * 64 + cb * 32;
-                if (cbase >= a.N) continue;
+                float sv = 1.f;
+                if constexpr (W8) {
+                    const int nr = NMAT == 2 ? hh : cb * 2 + hh;
+                    const int ch = min(cblock * NR + nr, NT - 1) * 16 + j;
+                    sv = NMAT == 2 ? (cb == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
+                }
+                c.as[cb] = sv;
+                c.ac[cb] = -128.f * sv;
+            }
+#pragma unroll
+            for (int i = 0; i < LX; ++i) {
+                const int rr = min(xrow[i], item.nrows - 1);     // rows past the item re-read its last row
+                const int64_t row = a.rows ? (int64_t)a.rows[item.row0 + rr] : (int64_t)(item.row0 + rr);
+                c.xsrc[i] = (const T *)a.x + row * a.x_stride + xcol[i];
+            }
+            return t;
+        }
+        return -1;
+    };
+
+#define EK_ISSUE(ctx, step, ring)                                                               \
+    {                                                                                           \
+        const uint32_t st_ = lds_base + (ring) * G::STAGE;                                      \
+        _Pragma("unroll") for (int nr = 0; nr < NR; ++nr)                                       \
+        _Pragma("unroll") for (int m = 0; m < NMAT; ++m)                                        \
+            dma16((ctx).wp[nr] + (int64_t)((step) * NMAT + m) * kChunkBytes,                    \
+                  st_ + w_off + (nr * NMAT + m) * kChunkBytes);                                 \
+        _Pragma("unroll") for (int i = 0; i < LX; ++i) dma16((ctx).xsrc[i] + (step) * BK, st_ + xdst[i]); \
+    }
+
+    Ctx cur, nxt;
+    int tc = fetch(first, cur);
+    if (tc < 0) return;
+    int ring = 0;                                // stage of the current step
+    block_barrier();                             // every wave has left the previous class's stages
+    EK_ISSUE(cur, 0, 0);
+    EK_ISSUE(cur, 1, 1);
+
+    while (true) {
+        // the next tile's addresses are needed two steps before this one ends; fetching
+        // them here costs one drain of the (two-stage deep) DMA queue per tile
+        const int tn = fetch(tc + stride, nxt);
+
+        f32x16 acc[RB][CB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.f;
+
+        for (int step = 0; step < nsteps; ++step) {
+            // the DMAs of this step are older than those of the next one (of this tile or of
+            // the next tile): wait until only the latter remain
+            if (step + 1 < nsteps || tn >= 0) wait_vmcnt<LOADS>();
+            else wait_vmcnt<0>();
+            block_barrier();   // this step's tile is visible to all waves; the stage of the
+                               // previous step is free again
+            const int ring2 = ring == 0 ? 2 : ring - 1;          // (ring + 2) % 3
+            if (step + 2 < nsteps) {
+                EK_ISSUE(cur, step + 2, ring2);
+            } else if (tn >= 0) {
+                EK_ISSUE(nxt, step + 2 - nsteps, ring2);
+            }
+
+            const uint8_t *stage = lds + ring * G::STAGE;
+            const uint8_t *wreg = stage + w_off;
+            u32x4 aq[2][CB];
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) aq[tt][cb] = *(const u32x4 *)(wreg + aoff[cb] + tt * 512);
+
+            // A operands of k-group grp: int8 -> half (grp & 1) of read grp >> 1, dequantised;
+            // 16-bit -> read grp as it is.  Software pipeline, pinned with scheduling fences:
+            // per row block 2 MFMAs, the B fragment read of the next k-group, and a share of
+            // the next k-group's dequantisation.
+            u32x4 af[2][CB];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                if constexpr (W8) {
+                    const u32x2 lo = dequant_u8x4<T>(aq[0][cb][0], cur.as[cb], cur.ac[cb]);
+                    const u32x2 hi = dequant_u8x4<T>(aq[0][cb][1], cur.as[cb], cur.ac[cb]);
+                    af[0][cb] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+                } else {
+                    af[0][cb] = aq[0][cb];
+                }
+            }
+            V8 bf[2][RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
+#pragma unroll
+            for (int grp = 0; grp < NGRP; ++grp) {
+                const int cg = grp & 1, ng = cg ^ 1;
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    if (grp + 1 < NGRP)
+                        bf[ng][rb] = *(const V8 *)(stage + boff[(grp + 1) % NGRP] + rb * kRowBlockBytes);
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb)
+                        acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cg][cb]), bf[cg][rb], acc[rb][cb]);
+                    if (grp + 1 < NGRP) {
+                        if constexpr (W8) {
+                            // next group's A operands: 4 dwords (2 per column block) spread over the row blocks
+                            constexpr int DW = 4 / RB;
+#pragma unroll
+                            for (int d = 0; d < DW; ++d) {
+                                const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
+                                const int g1 = grp + 1;
+                                const u32x2 v = dequant_u8x4<T>(aq[g1 >> 1][cb][(g1 & 1) * 2 + part], cur.as[cb], cur.ac[cb]);
+                                af[ng][cb][part * 2] = v[0];
+                                af[ng][cb][part * 2 + 1] = v[1];
+                            }
+                        } else {
+                            if (rb == 0) {
+#pragma unroll
+                                for (int cb = 0; cb < CB; ++cb) af[ng][cb] = aq[(grp + 1) % 2][cb];
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            ring = ring == 2 ? 0 : ring + 1;
+        }
+
+        // ---- epilogue: lane holds, for row rb*32 + l%32, channels q*8 + kg*4 + (0..3), q = 0..3,
+        //      of each column block ----
+        typedef T T4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int r_in = rb * 32 + l32;
+            if (r_in >= cur.nrows) continue;
+            T *orow = (T *)a.out + (int64_t)(cur.row0 + r_in) * a.out_stride;
+            if constexpr (NMAT == 2) {
+                if (cur.chan0 >= a.N) continue;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     T4 o;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) o[r] = (T)acc[rb][cb][q * 4 + r];
-                    *(uint2 *)(orow + cbase + q * 8 + kg * 4) = __builtin_bit_cast(uint2, o);
+                    for (int r = 0; r < 4; ++r) o[r] = swiglu_rounded<T>(acc[rb][0][q * 4 + r], acc[rb][1][q * 4 + r]);
+                    *(uint2 *)(orow + cur.chan0 + q * 8 + kg * 4) = __builtin_bit_cast(uint2, o);
+                }
+            } else {
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const int cbase = cur.chan0 + cb * 32;
+                    if (cbase >= a.N) continue;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        T4 o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[r] = (T)acc[rb][cb][q * 4 + r];
+                        *(uint2 *)(orow + cbase + q * 8 + kg * 4) = __builtin_bit_cast(uint2, o);
+                    }
                 }
             }
         }
+        if (tn < 0) break;
+        cur = nxt;
+        tc = tn;
     }
+#undef EK_ISSUE
 }
 
-// One launch covers the three tile lists.  Workgroup b runs on XCD b % 8
-// (round-robin dispatch), so each XCD is given a contiguous eighth of every
-// list: first its 128-row items, then its 64-row, then its 32-row ones, each
-// times nb_count channel blocks.
+// Persistent launch: one workgroup per CU (the LDS stages fill it), numbered so that
+// workgroup b runs on XCD b % 8 (round-robin dispatch).  Each XCD is given a contiguous
+// eighth of every work list, and its workgroups walk that eighth's tiles side by side:
+// neighbouring CUs share the activation tile (same item) and mostly the expert's weights
+// in the XCD's L2.  Every workgroup's tile sequence is fixed by its index: no queues, no
+// spinning, and it ends when its indices run out.
 template <typename T, bool W8, int NMAT>
 __global__ __launch_bounds__(kTileThreads, 1) void ffn_tile_kernel(FfnArgs a, int nb_count)
 {
     __shared__ __attribute__((aligned(1024))) uint8_t lds[kTileStages * TileGeom<W8>::STAGE];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)lds;
-    const int x = blockIdx.x & 7;
-    int i = blockIdx.x >> 3;
+    const int x = blockIdx.x & 7, slot = blockIdx.x >> 3, nslots = gridDim.x >> 3;
     const int n128 = a.lists.count[kListT128], n64 = a.lists.count[kListT64], n32 = a.lists.count[kListT32];
     const int lo128 = x * n128 / 8, s128 = (x + 1) * n128 / 8 - lo128;
     const int lo64 = x * n64 / 8, s64 = (x + 1) * n64 / 8 - lo64;
     const int lo32 = x * n32 / 8, s32 = (x + 1) * n32 / 8 - lo32;
-    if (i < s128 * nb_count) {
-        tile_body<T, W8, NMAT, 8>(a, a.lists.items[kListT128][lo128 + i / nb_count], i % nb_count, lds, lds_base);
-        return;
-    }
-    i -= s128 * nb_count;
-    if (i < s64 * nb_count) {
-        tile_body<T, W8, NMAT, 4>(a, a.lists.items[kListT64][lo64 + i / nb_count], i % nb_count, lds, lds_base);
-        return;
-    }
-    i -= s64 * nb_count;
-    if (i < s32 * nb_count)
-        tile_body<T, W8, NMAT, 2>(a, a.lists.items[kListT32][lo32 + i / nb_count], i % nb_count, lds, lds_base);
+    run_tiles<T, W8, NMAT, 8>(a, a.lists.items[kListT128] + lo128, s128 * nb_count, nb_count, slot, nslots, lds, lds_base);
+    // the shorter classes start where the long one left the CUs least loaded
+    const int r64 = (slot + nslots - (s128 * nb_count) % nslots) % nslots;
+    run_tiles<T, W8, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds, lds_base);
+    const int r32 = (r64 + nslots - (s64 * nb_count) % nslots) % nslots;
+    run_tiles<T, W8, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32, nslots, lds, lds_base);
 }
 
 template <typename T, bool W8, int NMAT>
@@ -336,9 +364,10 @@ static hipError_t launch_t(const FfnArgs &a, const int64_t max_items[kNumLists],
     const int nb_count = (NT + kTileWaves * NR - 1) / (kTileWaves * NR);
     const int64_t per_xcd = (max_items[kListT128] + 7) / 8 + (max_items[kListT64] + 7) / 8 +
                             (max_items[kListT32] + 7) / 8;
-    const int64_t blocks = per_xcd * nb_count * 8;
-    if (blocks <= 0) return hipSuccess;
-    hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT>), dim3((unsigned)blocks), dim3(kTileThreads), 0, s, a,
+    int64_t slots = per_xcd * nb_count;          // tiles an XCD can get at most
+    if (slots <= 0) return hipSuccess;
+    if (slots > kCusPerXcd) slots = kCusPerXcd;
+    hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT>), dim3((unsigned)(slots * 8)), dim3(kTileThreads), 0, s, a,
                        nb_count);
     return hipGetLastError();
 }
