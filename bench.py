@@ -33,14 +33,15 @@ def measured_traffic(workload: str, stage: int, decode: bool):
     if not os.path.exists(path):
         return None
     table = json.load(open(path)).get(workload, {})
-    want = "ffn_stream_kernel" if decode else "ffn_tile_kernel"
-    nmat = ", 2" if stage == 1 else ", 1"
+    # kernel names in the profile end in <..., E, NMAT, ...>: NMAT = 2 is stage 1, 1 is stage 2;
+    # the stage's time covers both kernel families, so does its traffic
+    tag = "E, 2" if stage == 1 else "E, 1"
+    total, seen = 0.0, False
     for name, t in table.items():
-        if want in name and name.split("E" + nmat)[0] != name and ("E" + nmat + ",") in name + ",":
-            return t["fetch_bytes"] + t["write_bytes"]
-        if want in name and ("E" + nmat + ">") in name:
-            return t["fetch_bytes"] + t["write_bytes"]
-    return None
+        if ("ffn_stream_kernel" in name or "ffn_tile_kernel" in name) and (tag + ",") in name.replace(">", ","):
+            total += t["fetch_bytes"] + t["write_bytes"]
+            seen = True
+    return total if seen else None
 
 
 def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
@@ -214,7 +215,8 @@ def main():
     hbm_frac = b_layer / step_s / HBM_PEAK
     mfma_frac = f_layer / step_s / MFMA_PEAK_16
     dom = 1 if k_us[1] >= k_us[2] else 2
-    dom_name = "ffn_stream_kernel(stage 1: up/gate + SwiGLU)" if dom == 1 else "ffn_stream_kernel(stage 2: down)"
+    fam = "ffn_stream_kernel" if hbm_frac >= mfma_frac else "ffn_tile_kernel (+ ffn_stream_kernel for items of <= 16 rows)"
+    dom_name = fam + (", stage 1: up/gate + SwiGLU" if dom == 1 else ", stage 2: down")
     dom_bytes = b_ffn1 if dom == 1 else b_ffn2
     dom_flops = w.pairs * (4 if dom == 1 else 2) * w.hidden * w.inter
     dom_s = k_us[dom] * 1e-6

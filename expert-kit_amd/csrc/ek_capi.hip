@@ -66,7 +66,7 @@ int64_t elem_size(int dt)
     switch (dt) {
     case EK_BF16: case EK_F16: return 2;
     case EK_F32: return 4;
-    case EK_I8: return 1;
+    case EK_I8: case EK_F8E4M3: return 1;
     default: return 0;
     }
 }
@@ -268,14 +268,31 @@ ek_status check_desc(const ek_weight_desc *d, const char *name, int64_t rows, in
         if (!d->scale) return fail(EK_WEIGHT_NOT_FOUND, "%s scale is missing", name);
         if (d->scale_dtype != EK_BF16 && d->scale_dtype != EK_F32 && d->scale_dtype != EK_F16)
             return fail(EK_INVALID_INPUT, "%s scale: bad dtype %d", name, d->scale_dtype);
+    } else if (d->scale_kind == EK_SCALE_BLOCK128) {
+        // block-scaled checkpoint tensors are dequantised to the 16-bit type at load
+        if (d->dtype != EK_I8 && d->dtype != EK_F8E4M3 && d->dtype != EK_BF16 && d->dtype != EK_F16 &&
+            d->dtype != EK_F32)
+            return fail(EK_INVALID_INPUT, "%s weight: bad dtype %d", name, d->dtype);
+        if (!d->scale) return fail(EK_WEIGHT_NOT_FOUND, "%s block scale is missing", name);
+        if (d->scale_dtype != EK_BF16 && d->scale_dtype != EK_F32 && d->scale_dtype != EK_F16)
+            return fail(EK_INVALID_INPUT, "%s scale: bad dtype %d", name, d->scale_dtype);
     } else {
         if (d->dtype != EK_BF16 && d->dtype != EK_F16 && d->dtype != EK_F32)
-            return fail(EK_INVALID_INPUT, "%s weight: dtype %d cannot be cast to the layer's 16-bit type",
-                        name, d->dtype);
+            return fail(EK_INVALID_INPUT, "%s weight: dtype %d cannot be cast to the layer's 16-bit type "
+                        "without block scales", name, d->dtype);
         if (d->scale_kind != EK_SCALE_NONE)
-            return fail(EK_INVALID_INPUT, "%s weight: scales are only valid with EK_I8", name);
+            return fail(EK_INVALID_INPUT, "%s weight: per-channel scales need an EK_I8 layer", name);
     }
     return EK_OK;
+}
+
+// bytes of a descriptor's scale tensor (0 if it has none)
+size_t scale_bytes(const ek_weight_desc *d)
+{
+    if (d->scale_kind == EK_SCALE_PER_CHANNEL) return (size_t)d->rows * elem_size(d->scale_dtype);
+    if (d->scale_kind == EK_SCALE_BLOCK128)
+        return (size_t)((d->rows + 127) / 128) * ((d->cols + 127) / 128) * elem_size(d->scale_dtype);
+    return 0;
 }
 
 // Brings `bytes` of (host or device) source to a device address usable by the
@@ -309,7 +326,7 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
         if (d->mem == EK_HOST) {
             need += (size_t)d->rows * d->cols * elem_size(d->dtype);
             need = (need + 255) & ~(size_t)255;
-            if (L->w8) need += ((size_t)d->rows * elem_size(d->scale_dtype) + 255) & ~(size_t)255;
+            need += (scale_bytes(d) + 255) & ~(size_t)255;
         }
     }
     if (need > L->st_raw_bytes) {
@@ -348,16 +365,17 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
         st = stage_raw(L, d->ptr, d->mem, bytes, off, &src);
         if (d->mem == EK_HOST) off = (off + bytes + 255) & ~(size_t)255;
         if (st != EK_OK) break;
-        ek::launch_tile_weights(src, d->dtype, d->rows, d->cols, wdst[i], dst_dt, mi[i], nmat[i],
-                                L->load_stream);
-        if (L->w8) {
-            const void *ssrc = nullptr;
-            const size_t sbytes = (size_t)d->rows * elem_size(d->scale_dtype);
+        const void *ssrc = nullptr;
+        const size_t sbytes = scale_bytes(d);
+        if (sbytes) {
             st = stage_raw(L, d->scale, d->mem, sbytes, off, &ssrc);
             if (d->mem == EK_HOST) off = (off + sbytes + 255) & ~(size_t)255;
             if (st != EK_OK) break;
-            ek::launch_scales_to_f32(ssrc, d->scale_dtype, d->rows, sdst[i], L->load_stream);
         }
+        ek::launch_tile_weights(src, d->dtype, d->rows, d->cols, wdst[i], dst_dt, mi[i], nmat[i],
+                                d->scale_kind == EK_SCALE_BLOCK128 ? ssrc : nullptr, d->scale_dtype,
+                                L->load_stream);
+        if (L->w8) ek::launch_scales_to_f32(ssrc, d->scale_dtype, d->rows, sdst[i], L->load_stream);
     }
     if (st == EK_OK) {
         hipError_t e = hipGetLastError();

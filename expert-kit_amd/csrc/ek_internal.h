@@ -121,9 +121,11 @@ void launch_combine(const CombineArgs &a, hipStream_t s);
 
 // ---- weight ingestion -------------------------------------------------------
 // src [N, K] row-major of src_dtype (ek_dtype numbering) -> chunked layout at
-// dst, matrix m of an nmat-group.  dst_dtype: 0 bf16, 1 f16, 3 int8.
+// dst, matrix m of an nmat-group.  dst_dtype: 0 bf16, 1 f16, 3 int8.  block_scale (16-bit
+// destinations only, may be nullptr): [ceil(N/128), ceil(K/128)] factors of scale_dtype.
 void launch_tile_weights(const void *src, int src_dtype, int64_t N, int64_t K, uint8_t *dst,
-                         int dst_dtype, int m, int nmat, hipStream_t s);
+                         int dst_dtype, int m, int nmat, const void *block_scale, int scale_dtype,
+                         hipStream_t s);
 void launch_scales_to_f32(const void *src, int src_dtype, int64_t n, float *dst, hipStream_t s);
 
 }  // namespace ek

@@ -56,19 +56,36 @@ void launch_combine(const CombineArgs &a, hipStream_t s)
 
 // ---- weight ingestion ---------------------------------------------------------
 
+// OCP fp8 e4m3fn -> fp32 (no infinities; 0x7f / 0xff are NaN)
+__device__ __forceinline__ float f8e4m3_to_f32(uint8_t b)
+{
+    const uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+    const uint32_t exp = (b >> 3) & 0xfu, man = b & 0x7u;
+    float v;
+    if (exp == 0) v = (float)man * 0.001953125f;                          // subnormal: man * 2^-9
+    else if (exp == 15 && man == 7) v = __builtin_nanf("");
+    else v = __builtin_bit_cast(float, ((exp + 120u) << 23) | (man << 20));
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) | sign);
+}
+
 __device__ __forceinline__ float load_src(const void *src, int dt, int64_t i)
 {
     switch (dt) {
     case 0: return (float)((const __bf16 *)src)[i];
     case 1: return (float)((const _Float16 *)src)[i];
+    case 3: return (float)((const int8_t *)src)[i];
+    case 4: return f8e4m3_to_f32(((const uint8_t *)src)[i]);
     default: return ((const float *)src)[i];
     }
 }
 
 // One thread writes one lane's 16 bytes of one chunk.
+// scale (optional): one factor per 128x128 block, [ceil(N/128), ceil(K/128)]; the product is
+// formed in fp32 and rounded once, as w8a16_activate does (ffn/expert_torch.rs:45-52).
 template <typename T>
 __global__ __launch_bounds__(256) void tile_weights16_kernel(const void *src, int src_dt, int64_t N,
-                                                            int64_t K, uint8_t *dst, int m, int nmat)
+                                                            int64_t K, uint8_t *dst, int m, int nmat,
+                                                            const void *scale, int scale_dt)
 {
     typedef T V8 __attribute__((ext_vector_type(8)));
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -79,7 +96,11 @@ __global__ __launch_bounds__(256) void tile_weights16_kernel(const void *src, in
     const int64_t row = nt * 16 + (l & 15), col = kt * 32 + (l >> 4) * 8;
     V8 v;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = (T)load_src(src, src_dt, row * K + col + i);
+    for (int i = 0; i < 8; ++i) {
+        float f = load_src(src, src_dt, row * K + col + i);
+        if (scale) f = f * load_src(scale, scale_dt, (row >> 7) * ((K + 127) >> 7) + ((col + i) >> 7));
+        v[i] = (T)f;
+    }
     *(V8 *)(dst + (chunk * nmat + m) * kChunkBytes + l * 16) = v;
 }
 
@@ -98,7 +119,8 @@ __global__ __launch_bounds__(256) void tile_weights8_kernel(const uint8_t *src, 
 }
 
 void launch_tile_weights(const void *src, int src_dtype, int64_t N, int64_t K, uint8_t *dst,
-                         int dst_dtype, int m, int nmat, hipStream_t s)
+                         int dst_dtype, int m, int nmat, const void *block_scale, int scale_dtype,
+                         hipStream_t s)
 {
     if (dst_dtype == 3) {
         const int64_t total = (N / 16) * (K / 64) * 64;
@@ -108,10 +130,10 @@ void launch_tile_weights(const void *src, int src_dtype, int64_t N, int64_t K, u
         const int64_t total = (N / 16) * (K / 32) * 64;
         if (dst_dtype == 0)
             hipLaunchKernelGGL(tile_weights16_kernel<__bf16>, dim3((total + 255) / 256), dim3(256), 0,
-                               s, src, src_dtype, N, K, dst, m, nmat);
+                               s, src, src_dtype, N, K, dst, m, nmat, block_scale, scale_dtype);
         else
             hipLaunchKernelGGL(tile_weights16_kernel<_Float16>, dim3((total + 255) / 256), dim3(256),
-                               0, s, src, src_dtype, N, K, dst, m, nmat);
+                               0, s, src, src_dtype, N, K, dst, m, nmat, block_scale, scale_dtype);
     }
 }
 

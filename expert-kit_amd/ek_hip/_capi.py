@@ -14,9 +14,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("EK_HIP_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libek_hip.so")
 
 EK_OK, EK_INVALID_INPUT, EK_EXPERT_NOT_FOUND, EK_WEIGHT_NOT_FOUND, EK_OOM, EK_HIP_ERROR, EK_INTERNAL = range(7)
-EK_BF16, EK_F16, EK_F32, EK_I8 = range(4)
+EK_BF16, EK_F16, EK_F32, EK_I8, EK_F8E4M3 = range(5)
 EK_HOST, EK_DEVICE = 0, 1
-EK_SCALE_NONE, EK_SCALE_PER_CHANNEL = 0, 1
+EK_SCALE_NONE, EK_SCALE_PER_CHANNEL, EK_SCALE_BLOCK128 = 0, 1, 2
 
 STATUS_NAMES = ["EK_OK", "EK_INVALID_INPUT", "EK_EXPERT_NOT_FOUND", "EK_WEIGHT_NOT_FOUND", "EK_OOM",
                 "EK_HIP_ERROR", "EK_INTERNAL"]

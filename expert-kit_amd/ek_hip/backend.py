@@ -24,7 +24,8 @@ import torch
 
 from . import _capi as C
 
-_DT = {torch.bfloat16: C.EK_BF16, torch.float16: C.EK_F16, torch.float32: C.EK_F32, torch.int8: C.EK_I8}
+_DT = {torch.bfloat16: C.EK_BF16, torch.float16: C.EK_F16, torch.float32: C.EK_F32, torch.int8: C.EK_I8,
+       torch.float8_e4m3fn: C.EK_F8E4M3}
 
 
 def _mem(t: torch.Tensor) -> int:
@@ -78,9 +79,12 @@ class ExpertWeight:
         if gate is None:
             raise C.EKError(C.EK_WEIGHT_NOT_FOUND, "w3/gate_w")
         return cls(up_w=up, gate_w=gate, down_w=down,
-                   up_scale=cls._lookup_suffix(tensors, ["w1.weight_scale", "up_proj.weight_scale"]),
-                   gate_scale=cls._lookup_suffix(tensors, ["w3.weight_scale", "gate_proj.weight_scale"]),
-                   down_scale=cls._lookup_suffix(tensors, ["w2.weight_scale", "down_proj.weight_scale"]))
+                   up_scale=cls._lookup_suffix(tensors, ["w1.weight_scale", "up_proj.weight_scale",
+                                                         "w1.weight_scale_inv", "up_proj.weight_scale_inv"]),
+                   gate_scale=cls._lookup_suffix(tensors, ["w3.weight_scale", "gate_proj.weight_scale",
+                                                           "w3.weight_scale_inv", "gate_proj.weight_scale_inv"]),
+                   down_scale=cls._lookup_suffix(tensors, ["w2.weight_scale", "down_proj.weight_scale",
+                                                           "w2.weight_scale_inv", "down_proj.weight_scale_inv"]))
 
     @classmethod
     def from_rand_linear(cls, hidden: int, intermediate: int, dtype=torch.bfloat16, device="cpu"):
@@ -107,7 +111,8 @@ def _desc(w: Optional[torch.Tensor], scale: Optional[torch.Tensor]):
             scale = scale.to(w.device)
         d.scale = scale.data_ptr()
         d.scale_dtype = _DT[scale.dtype]
-        d.scale_kind = C.EK_SCALE_PER_CHANNEL
+        # [rows] = per output channel; [rows/128, cols/128] = the checkpoint's weight_scale_inv blocks
+        d.scale_kind = C.EK_SCALE_PER_CHANNEL if scale.dim() == 1 else C.EK_SCALE_BLOCK128
         keep.append(scale)
     else:
         d.scale = None
@@ -266,7 +271,9 @@ class HipFFN:
     def construct(cls, x: EKInstance, weight: ExpertWeight, act_dtype=torch.bfloat16, max_rows: int = 4096,
                   device_id: int = 0) -> "HipFFN":
         lib = C.load()
-        w_dtype = torch.int8 if weight.up_w is not None and weight.up_w.dtype == torch.int8 else act_dtype
+        per_channel_i8 = (weight.up_w is not None and weight.up_w.dtype == torch.int8
+                          and weight.up_scale is not None and weight.up_scale.dim() == 1)
+        w_dtype = torch.int8 if per_channel_i8 else act_dtype
         cfg = C.ek_cfg(hidden=x.hidden, inter=x.intermediate, n_experts=1, top_k=1, act_dtype=_DT[act_dtype],
                        w_dtype=_DT[w_dtype], max_tokens=max_rows, device_id=device_id, flags=0)
         up, k1 = _desc(weight.up_w, weight.up_scale)

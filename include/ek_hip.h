@@ -47,13 +47,25 @@ typedef enum ek_status {
 
 /* Element types (ek-computation/src/backend/mod.rs:7-16 and
  * backend/torch/tch_safetensors.rs:12-46 list the reference's). */
-typedef enum ek_dtype { EK_BF16 = 0, EK_F16 = 1, EK_F32 = 2, EK_I8 = 3 } ek_dtype;
+typedef enum ek_dtype {
+    EK_BF16 = 0,
+    EK_F16 = 1,
+    EK_F32 = 2,
+    EK_I8 = 3,
+    EK_F8E4M3 = 4 /* OCP e4m3fn, DType::Float8e4m3fn (backend/mod.rs:13); load-time source type only */
+} ek_dtype;
 
 typedef enum ek_mem { EK_HOST = 0, EK_DEVICE = 1 } ek_mem;
 
 typedef enum ek_scale_kind {
     EK_SCALE_NONE = 0,
-    EK_SCALE_PER_CHANNEL = 1 /* one scale per output row: W[n,:] = q[n,:] * scale[n] */
+    EK_SCALE_PER_CHANNEL = 1, /* one scale per output row: W[n,:] = q[n,:] * scale[n] */
+    /* one scale per 128x128 block, scale [ceil(rows/128), ceil(cols/128)] (the
+     * `weight_scale_inv` tensors of DeepSeek Block-INT8 / FP8 checkpoints).  The weights are
+     * dequantised once at load to the layer's 16-bit type, exactly as w8a16_activate does
+     * (ffn/expert_torch.rs:24-53): W[r,c] = rne(f32(q[r,c]) * s[r/128, c/128]); the layer's
+     * w_dtype must be its act_dtype. */
+    EK_SCALE_BLOCK128 = 2
 } ek_scale_kind;
 
 /* Stands for EKInstance{hidden, intermediate, backend} (ek-computation/src/x.rs:27-32)
@@ -78,10 +90,11 @@ typedef struct ek_weight_desc {
     int64_t rows;
     int64_t cols;
     int32_t dtype;       /* EK_BF16 / EK_F16 / EK_F32 (cast on load, as
-                            TorchFFN::load_module does, ffn/expert_torch.rs:61-78) or EK_I8 */
+                            TorchFFN::load_module does, ffn/expert_torch.rs:61-78), EK_I8, or
+                            EK_F8E4M3 (block-scaled only) */
     int32_t mem;         /* ek_mem of ptr and scale */
     const void *scale;   /* NULL unless scale_kind != EK_SCALE_NONE */
-    int32_t scale_dtype; /* EK_BF16 or EK_F32 */
+    int32_t scale_dtype; /* EK_BF16, EK_F16 or EK_F32 */
     int32_t scale_kind;  /* ek_scale_kind */
 } ek_weight_desc;
 

@@ -315,3 +315,43 @@ def test_error_paths(ek, cuda):
     assert layer.forward(x[:0], ok_ids[:0], gw[:0]).shape == (0, 128)   # T = 0
     layer.close()
     layer.close()                                               # idempotent
+
+
+# ------------------------------------------- block-scaled checkpoint weights
+
+@pytest.mark.parametrize("src", ["int8", "fp8"])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_block128_scaled_weights(ek, oracle, cuda, src, dt):
+    """DeepSeek Block-INT8 / FP8 tensors with 128x128 `weight_scale_inv` blocks are
+    dequantised at load exactly as w8a16_activate does (ffn/expert_torch.rs:24-53)."""
+    H, I, n = 384, 256, 40
+    g = torch.Generator().manual_seed(77)
+
+    def q(r, c):
+        if src == "int8":
+            return torch.randint(-127, 128, (r, c), generator=g, dtype=torch.int8)
+        return (torch.randn(r, c, generator=g) * 40).to(torch.float8_e4m3fn)
+
+    def s(r, c):
+        return torch.rand((r + 127) // 128, (c + 127) // 128, generator=g) * 2e-3 + 5e-4
+
+    ew = ek.ExpertWeight(up_w=q(I, H), gate_w=q(I, H), down_w=q(H, I), up_scale=s(I, H), gate_scale=s(I, H),
+                         down_scale=s(H, I))
+    ffn = ek.HipFFN.construct(ek.EKInstance(H, I), ew, act_dtype=dt, max_rows=64)
+    wu, wg, wd = (oracle.dequant_block(w.float(), sc) for w, sc in
+                  ((ew.up_w, ew.up_scale), (ew.gate_w, ew.gate_scale), (ew.down_w, ew.down_scale)))
+    if dt == torch.float16:      # the fp16 layer rounds the fp32 product to fp16 instead
+        wu, wg, wd = ((w.float() * sc.repeat_interleave(128, 0)[:w.shape[0]].repeat_interleave(128, 1)[:, :w.shape[1]]).to(dt)
+                      for w, sc in ((ew.up_w, ew.up_scale), (ew.gate_w, ew.gate_scale), (ew.down_w, ew.down_scale)))
+    x = torch.randn(n, H, generator=g).to(dt)
+    ref = oracle.ffn(x, wu, wg, wd, mode=2)
+    got = ffn.forward(x.to(cuda))
+    ffn_gate(got, ref, f"block128 {src} {dt}")
+    assert check_vs_rounded(got, ref, f"block128 {src} {dt}") > 0.9
+    # the same tensors through the checkpoint's names (ExpertWeight::from_safetensor suffixes)
+    named = {"m.experts.3.up_proj.weight": ew.up_w, "m.experts.3.up_proj.weight_scale_inv": ew.up_scale,
+             "m.experts.3.gate_proj.weight": ew.gate_w, "m.experts.3.gate_proj.weight_scale_inv": ew.gate_scale,
+             "m.experts.3.down_proj.weight": ew.down_w, "m.experts.3.down_proj.weight_scale_inv": ew.down_scale}
+    be = ek.ExpertBackend.build(ek.EKInstance(H, I), named, act_dtype=dt, max_rows=64)
+    assert torch.equal(be.forward(x.to(cuda)).cpu().view(torch.int16), got.cpu().view(torch.int16))
+    ffn.close()
