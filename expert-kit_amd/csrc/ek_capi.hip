@@ -15,6 +15,14 @@ namespace {
 
 thread_local std::string g_last_error;
 
+}  // namespace
+
+namespace ek {
+void set_last_error(const char *msg) { g_last_error = msg ? msg : ""; }
+}  // namespace ek
+
+namespace {
+
 ek_status fail(ek_status st, const char *fmt, ...)
 {
     char buf[512];
@@ -93,6 +101,10 @@ struct ek_layer {
     ek::WorkLists lists{};                   // device work lists (see ek_internal.h)
     int64_t list_cap[ek::kNumLists] = {0, 0, 0, 0};
     int32_t *h_err = nullptr;                // pinned
+    // host-built work lists (ek_layer_experts_forward): pinned image of the device lists,
+    // reused once ev_items says the previous copy has been consumed
+    uint8_t *h_items = nullptr;
+    hipEvent_t ev_items = nullptr;
 
     // staging for host-memory callers (allocated on first use)
     void *st_x = nullptr, *st_w = nullptr, *st_y = nullptr, *st_xp = nullptr;
@@ -159,6 +171,8 @@ void free_layer(ek_layer *L)
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
     if (L->h_err) (void)hipHostFree(L->h_err);
+    if (L->h_items) (void)hipHostFree(L->h_items);
+    if (L->ev_items) (void)hipEventDestroy(L->ev_items);
     if (L->stream) (void)hipStreamDestroy(L->stream);
     if (L->load_stream) (void)hipStreamDestroy(L->load_stream);
     if (L->side_stream) (void)hipStreamDestroy(L->side_stream);
@@ -788,6 +802,117 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
         {
             std::lock_guard<std::mutex> sl(layer->stats_mu);
             layer->stats.expert_forward_calls += 1;
+        }
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_describe(ek_layer *layer, int64_t *hidden, int64_t *inter, int32_t *n_experts,
+                            int32_t *top_k, int32_t *act_dtype)
+{
+    if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+    if (hidden) *hidden = layer->cfg.hidden;
+    if (inter) *inter = layer->cfg.inter;
+    if (n_experts) *n_experts = layer->cfg.n_experts;
+    if (top_k) *top_k = layer->cfg.top_k;
+    if (act_dtype) *act_dtype = layer->cfg.act_dtype;
+    return EK_OK;
+}
+
+ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32_t *experts,
+                                   const void *const *xs, const int64_t *rows, void *const *outs,
+                                   int32_t mem, void *stream)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        if (n_calls < 0) return fail(EK_INVALID_INPUT, "n_calls is negative");
+        if (n_calls > 0 && (!experts || !xs || !rows || !outs)) return fail(EK_INVALID_INPUT, "NULL argument");
+        if (mem != EK_HOST && mem != EK_DEVICE) return fail(EK_INVALID_INPUT, "bad mem %d", mem);
+        if (mem == EK_HOST && stream)
+            return fail(EK_INVALID_INPUT, "host-memory calls are blocking: stream must be NULL");
+        const int64_t H = layer->cfg.hidden;
+        int64_t P = 0;
+        for (int i = 0; i < n_calls; ++i) {
+            if (experts[i] < 0 || experts[i] >= layer->cfg.n_experts)
+                return fail(EK_INVALID_INPUT, "call %d: expert %d outside [0, %d)", i, experts[i],
+                            layer->cfg.n_experts);
+            if (rows[i] < 0 || rows[i] > layer->Pmax - P)
+                return fail(EK_INVALID_INPUT, "call %d: rows exceed the layer's capacity of %lld", i,
+                            (long long)layer->Pmax);
+            if (rows[i] > 0 && (!xs[i] || !outs[i])) return fail(EK_INVALID_INPUT, "call %d: NULL tensor pointer", i);
+            P += rows[i];
+        }
+        DeviceGuard dg(layer->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
+        std::lock_guard<std::mutex> lk(layer->mu);
+        for (int i = 0; i < n_calls; ++i)
+            if (!layer->expert_mem[experts[i]])
+                return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", experts[i]);
+        hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+        if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
+        if (P > 0) {
+            // Work lists cut on the host exactly as the pack kernels cut them: a call is one
+            // segment (ek_internal.h, "work lists").
+            std::vector<ek::WorkItem> items[ek::kNumLists];
+            int64_t row0 = 0;
+            for (int i = 0; i < n_calls; ++i) {
+                const int32_t n = (int32_t)rows[i], full = n >> 7, r = n & 127;
+                for (int32_t t = 0; t < full; ++t)
+                    items[ek::kListT128].push_back(ek::WorkItem{experts[i], (int32_t)row0 + t * 128, 128, 0});
+                const ek::WorkItem rem{experts[i], (int32_t)row0 + full * 128, r, 0};
+                if (r > 64) items[ek::kListT128].push_back(rem);
+                else if (r > 32) items[ek::kListT64].push_back(rem);
+                else if (r > 16) items[ek::kListT32].push_back(rem);
+                else if (r > 0) items[ek::kListStream].push_back(rem);
+                row0 += n;
+            }
+            size_t off[ek::kNumLists + 1];
+            off[0] = 16;
+            for (int l = 0; l < ek::kNumLists; ++l) {
+                if ((int64_t)items[l].size() > layer->list_cap[l])
+                    return fail(EK_INVALID_INPUT, "too many calls for one launch (work list %d holds %lld items)", l,
+                                (long long)layer->list_cap[l]);
+                off[l + 1] = off[l] + sizeof(ek::WorkItem) * (size_t)layer->list_cap[l];
+            }
+            if (!layer->h_items) {
+                EK_HIP(hipHostMalloc((void **)&layer->h_items, off[ek::kNumLists], hipHostMallocDefault));
+                EK_HIP(hipEventCreateWithFlags(&layer->ev_items, hipEventDisableTiming));
+            } else {
+                EK_HIP(hipEventSynchronize(layer->ev_items));
+            }
+            int32_t *cnt = (int32_t *)layer->h_items;
+            for (int l = 0; l < ek::kNumLists; ++l) {
+                cnt[l] = (int32_t)items[l].size();
+                if (cnt[l]) {
+                    memcpy(layer->h_items + off[l], items[l].data(), sizeof(ek::WorkItem) * items[l].size());
+                    EK_HIP(hipMemcpyAsync(layer->lists.items[l], layer->h_items + off[l],
+                                          sizeof(ek::WorkItem) * items[l].size(), hipMemcpyHostToDevice, s));
+                }
+            }
+            EK_HIP(hipMemcpyAsync(layer->lists.count, cnt, sizeof(int32_t) * ek::kNumLists, hipMemcpyHostToDevice, s));
+            EK_HIP(hipEventRecord(layer->ev_items, s));
+            EK_TRY(ensure_io_staging(layer));
+            const hipMemcpyKind in_kind = mem == EK_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice;
+            const hipMemcpyKind out_kind = mem == EK_HOST ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice;
+            row0 = 0;
+            for (int i = 0; i < n_calls; ++i) {
+                if (rows[i])
+                    EK_HIP(hipMemcpyAsync((char *)layer->st_x + row0 * H * 2, xs[i], (size_t)rows[i] * H * 2, in_kind, s));
+                row0 += rows[i];
+            }
+            EK_TRY(enqueue_ffn(layer, layer->st_x, nullptr, layer->st_y, P, n_calls, s, nullptr));
+            EK_HIP(hipGetLastError());
+            row0 = 0;
+            for (int i = 0; i < n_calls; ++i) {
+                if (rows[i])
+                    EK_HIP(hipMemcpyAsync(outs[i], (char *)layer->st_y + row0 * H * 2, (size_t)rows[i] * H * 2, out_kind, s));
+                row0 += rows[i];
+            }
+        }
+        if (!stream) EK_HIP(hipStreamSynchronize(s));
+        {
+            std::lock_guard<std::mutex> sl(layer->stats_mu);
+            layer->stats.expert_forward_calls += n_calls;
         }
         return EK_OK;
     )

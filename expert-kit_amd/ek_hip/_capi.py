@@ -45,10 +45,18 @@ class ek_stats(ctypes.Structure):
                 ("kernel_us", ctypes.c_double * 4), ("profiled_calls", ctypes.c_int64)]
 
 
+class ek_tensor_view(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("shape", ctypes.c_int64 * 4), ("rank", ctypes.c_int32),
+                ("dtype", ctypes.c_int32), ("nbytes", ctypes.c_int64)]
+
+
 _P = ctypes.c_void_p
 _PP = ctypes.POINTER(ctypes.c_void_p)
 _I32, _I64 = ctypes.c_int32, ctypes.c_int64
 _DESC = ctypes.POINTER(ek_weight_desc)
+_SZ = ctypes.c_size_t
+_VIEW = ctypes.POINTER(ek_tensor_view)
+_STRS = ctypes.POINTER(ctypes.c_char_p)
 
 # name -> (restype, argtypes); every symbol include/ek_hip.h declares
 PROTOTYPES = {
@@ -63,6 +71,20 @@ PROTOTYPES = {
     "ek_layer_forward": (_I32, [_P, _P, _P, _P, _I32, _I64, _P, ctypes.POINTER(ek_route_out), _I32, _P]),
     "ek_layer_pack": (_I32, [_P, _P, _I64, ctypes.POINTER(ek_route_out), _P, _P, _I32, _P]),
     "ek_layer_expert_forward": (_I32, [_P, _I32, _P, _I64, _P, _I32, _P]),
+    "ek_layer_describe": (_I32, [_P, ctypes.POINTER(_I64), ctypes.POINTER(_I64), ctypes.POINTER(_I32),
+                                 ctypes.POINTER(_I32), ctypes.POINTER(_I32)]),
+    "ek_layer_experts_forward": (_I32, [_P, _I32, ctypes.POINTER(_I32), _PP, ctypes.POINTER(_I64), _PP, _I32, _P]),
+    "ek_expert_id_parse": (_I32, [ctypes.c_char_p, ctypes.POINTER(_I32), ctypes.POINTER(_I32)]),
+    "ek_expert_id_format": (_I32, [ctypes.c_char_p, _I32, _I32, ctypes.c_char_p, _SZ]),
+    "ek_safetensors_find": (_I32, [_P, _SZ, ctypes.c_char_p, _VIEW]),
+    "ek_safetensors_find_suffix": (_I32, [_P, _SZ, _STRS, _I32, _VIEW]),
+    "ek_safetensors_size": (_SZ, [ctypes.c_char_p, _I32, _I32, ctypes.POINTER(_I64)]),
+    "ek_safetensors_emit": (_I32, [ctypes.c_char_p, _I32, _I32, ctypes.POINTER(_I64), _P, _P, _SZ,
+                                   ctypes.POINTER(_SZ)]),
+    "ek_layer_set_expert_safetensors": (_I32, [_P, _I32, _P, _SZ]),
+    "ek_worker_forward": (_I32, [_P, ctypes.c_char_p, _P, _SZ, _P, _SZ, ctypes.POINTER(_SZ)]),
+    "ek_worker_forward_batch": (_I32, [_P, _I32, _STRS, _PP, ctypes.POINTER(_SZ), _PP, ctypes.POINTER(_SZ),
+                                       ctypes.POINTER(_SZ)]),
     "ek_layer_profile": (_I32, [_P, _I32]),
     "ek_layer_get_stats": (_I32, [_P, ctypes.POINTER(ek_stats)]),
     "ek_chain_create": (_I32, [_PP, _I32, _PP]),

@@ -206,6 +206,44 @@ class HipLayer:
                                                   _stream_ptr(stream)))
         return out
 
+    def experts_forward(self, experts: Sequence[int], xs: Sequence[torch.Tensor], stream=None):
+        """Several per-expert calls as one grouped launch; xs[i] is [n_i, H]."""
+        n = len(experts)
+        assert n == len(xs)
+        xs = [x.contiguous() for x in xs]
+        outs = [torch.empty_like(x) for x in xs]
+        mem = _mem(xs[0]) if n else C.EK_HOST
+        assert all(_mem(x) == mem for x in xs)
+        ex = (ctypes.c_int32 * n)(*experts)
+        rows = (ctypes.c_int64 * n)(*[x.shape[0] for x in xs])
+        xp = (ctypes.c_void_p * n)(*[x.data_ptr() for x in xs])
+        op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+        C.check(self._lib.ek_layer_experts_forward(self._h, n, ex, xp, rows, op, mem, _stream_ptr(stream)))
+        return outs
+
+    def set_expert_safetensors(self, e: int, blob: bytes) -> None:
+        """ExpertBackend::build from the bytes ek-db serves for one expert (ffn/mod.rs:27-34)."""
+        C.check(self._lib.ek_layer_set_expert_safetensors(self._h, e, blob, len(blob)))
+
+    def worker_forward(self, expert_id: str, req: bytes) -> bytes:
+        """EKInstanceGate::forward on wire bytes (worker/core.rs:47-74)."""
+        return self.worker_forward_batch([expert_id], [req])[0]
+
+    def worker_forward_batch(self, expert_ids: Sequence[str], reqs: Sequence[bytes]):
+        n = len(expert_ids)
+        assert n == len(reqs)
+        # a response is never larger than its request: same tensor name, dtype and shape
+        caps = [len(r) + 64 for r in reqs]
+        bufs = [ctypes.create_string_buffer(c) for c in caps]
+        ids = (ctypes.c_char_p * n)(*[i.encode() for i in expert_ids])
+        rp = (ctypes.c_void_p * n)(*[ctypes.cast(ctypes.c_char_p(r), ctypes.c_void_p).value for r in reqs])
+        rl = (ctypes.c_size_t * n)(*[len(r) for r in reqs])
+        op = (ctypes.c_void_p * n)(*[ctypes.addressof(b) for b in bufs])
+        oc = (ctypes.c_size_t * n)(*caps)
+        ol = (ctypes.c_size_t * n)()
+        C.check(self._lib.ek_worker_forward_batch(self._h, n, ids, rp, rl, op, oc, ol))
+        return [bufs[i].raw[:ol[i]] for i in range(n)]
+
     def profile(self, enable: bool) -> None:
         C.check(self._lib.ek_layer_profile(self._h, int(enable)))
 

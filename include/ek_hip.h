@@ -27,6 +27,7 @@
 #ifndef EK_HIP_H
 #define EK_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -182,6 +183,74 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
  * exceed cfg.max_tokens * top_k only if it still fits the workspace. */
 ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x, int64_t n,
                                   void *out, int32_t mem, void *stream);
+
+/* Geometry of a layer handle (what EKInstance carries: x.rs:27-32). Any out pointer may be NULL. */
+ek_status ek_layer_describe(ek_layer *layer, int64_t *hidden, int64_t *inter, int32_t *n_experts,
+                            int32_t *top_k, int32_t *act_dtype);
+
+/* Several per-expert calls as ONE grouped launch.  The controller fires one
+ * ForwardReq per expert concurrently (controller/executor.rs:141-195) and the
+ * worker answers each with Expert::forward (worker/core.rs:55-59); a worker
+ * that collects the concurrent requests hands them over together:
+ *   call i: xs[i] [rows[i], H] -> outs[i] [rows[i], H], expert experts[i].
+ * Results are bit-identical to n_calls separate ek_layer_expert_forward calls.
+ * The same expert may appear more than once; sum(rows) is bounded like n of
+ * ek_layer_expert_forward.  All pointers of one call share `mem`. */
+ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32_t *experts,
+                                   const void *const *xs, const int64_t *rows, void *const *outs,
+                                   int32_t mem, void *stream);
+
+/* ---- wire format of the worker contract ---------------------------------------
+ * Expert ids are "{model}/l{layer}-e{expert}": ExpertKey::from_expert_id and
+ * as_object_key (ek-db/src/safetensor/mod.rs:57-90).  Tensors travel as
+ * safetensors blobs: 8-byte little-endian header length, a JSON header
+ * {name: {dtype, shape, data_offsets}}, raw data. */
+ek_status ek_expert_id_parse(const char *id, int32_t *layer, int32_t *expert);
+ek_status ek_expert_id_format(const char *model, int32_t layer, int32_t expert, char *out, size_t cap);
+
+typedef struct ek_tensor_view {
+    const void *data;  /* points into the blob */
+    int64_t shape[4];  /* unused dimensions are 1 */
+    int32_t rank;
+    int32_t dtype;     /* ek_dtype */
+    int64_t nbytes;
+} ek_tensor_view;
+
+/* SafeTensors::deserialize + tensor(name) (worker/core.rs:52-53).  A name that is
+ * absent gives EK_WEIGHT_NOT_FOUND, a malformed blob or a dtype outside ek_dtype
+ * EK_INVALID_INPUT. */
+ek_status ek_safetensors_find(const void *blob, size_t len, const char *name, ek_tensor_view *out);
+/* First tensor (header order) whose name ends with one of the suffixes:
+ * FromSafeTensor::lookup_suffix (backend/torch/mod.rs:138-152). */
+ek_status ek_safetensors_find_suffix(const void *blob, size_t len, const char *const *suffixes,
+                                     int32_t n_suffixes, ek_tensor_view *out);
+/* Size and bytes of a one-tensor blob: TchTensor::serialize
+ * (backend/torch/mod.rs:115-117).  ek_safetensors_size returns 0 for a bad description. */
+size_t ek_safetensors_size(const char *name, int32_t dtype, int32_t rank, const int64_t *shape);
+ek_status ek_safetensors_emit(const char *name, int32_t dtype, int32_t rank, const int64_t *shape,
+                              const void *data, void *out, size_t cap, size_t *written);
+
+/* Loads one expert from the blob ek-db serves for it (transformer.rs:248-300):
+ * ExpertWeight::from_safetensor (ffn/meta.rs:56-75) picks up / down / gate by
+ * the suffixes w1|up_proj, w2|down_proj, w3|gate_proj ".weight"; a tensor named
+ * "<weight>_scale_inv" (or "<weight>_scale") beside a weight is taken as its
+ * scale: [rows] per channel, [rows/128, cols/128] per block.  Then as
+ * ek_layer_set_expert. */
+ek_status ek_layer_set_expert_safetensors(ek_layer *layer, int32_t expert, const void *blob, size_t len);
+
+/* EKInstanceGate::forward (worker/core.rs:47-74) on wire bytes: req is a
+ * safetensors blob with tensor "data" [n, H] of the layer's act dtype,
+ * expert_id the request's sequences[0].experts[0]; resp receives the blob of
+ * the result [n, H] (resp_len bytes; ek_safetensors_size gives the capacity
+ * to provide).  The layer part of the id is not checked: the handle is the
+ * layer. */
+ek_status ek_worker_forward(ek_layer *layer, const char *expert_id, const void *req, size_t req_len,
+                            void *resp, size_t resp_cap, size_t *resp_len);
+/* The same for n_calls requests collected by the worker, as one grouped launch
+ * (ek_layer_experts_forward). */
+ek_status ek_worker_forward_batch(ek_layer *layer, int32_t n_calls, const char *const *expert_ids,
+                                  const void *const *reqs, const size_t *req_lens, void *const *resps,
+                                  const size_t *resp_caps, size_t *resp_lens);
 
 /* Turns per-phase HIP-event timing of ek_layer_forward on (1) or off (0) and
  * clears the accumulated kernel_us.  Stands for the PerfTimer checkpoints of

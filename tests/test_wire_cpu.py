@@ -1,0 +1,145 @@
+"""Wire format of the worker contract, host side only (no GPU needed).
+
+The checker for the safetensors codec is the `safetensors` Python package (the
+Rust implementation the reference links, behind its Python binding): blobs
+written by it must parse, and blobs written here must be byte-identical to its
+output and load back through it.  The id codec is checked against the cases
+ExpertKey::from_expert_id accepts and rejects (ek-db/src/safetensor/mod.rs:57-73).
+"""
+import ctypes
+import json
+import struct
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import load as st_load
+from safetensors.torch import save as st_save
+
+from ek_hip import _capi as C
+from ek_hip import wire
+
+
+@pytest.mark.parametrize("text,layer,expert", [
+    ("ds-tiny/l0-e0", 0, 0),
+    ("qwen3-30b/l47-e127", 47, 127),
+    ("org/model/l3-e255", 3, 255),       # only "/l" splits; other slashes belong to the model name
+    ("m-e1/l2-e9", 2, 9),                # "-e" before "/l" belongs to the model name
+    ("m/l+4-e+5", 4, 5),                 # usize::from_str takes a leading plus
+])
+def test_expert_id_parse(text, layer, expert):
+    key = wire.ExpertKey.from_expert_id(text)
+    assert (key.layer, key.expert) == (layer, expert)
+
+
+@pytest.mark.parametrize("text", ["", "model", "m/l1", "m/l1-e", "m/l-e1", "m/lx-e1", "m/l1-ey", "m/l1-e2-e3",
+                                  "a/l1-e2/l3-e4", "m/l-1-e2", "m/l1 -e2", "m/l1-e2 "])
+def test_expert_id_rejects(text):
+    with pytest.raises(C.EKError) as ei:
+        wire.ExpertKey.from_expert_id(text)
+    assert ei.value.status == C.EK_INVALID_INPUT
+
+
+def test_expert_id_round_trip():
+    for model, layer, expert in [("ds-tiny", 0, 0), ("deepseek-v3", 60, 255), ("a/b", 7, 1023)]:
+        text = wire.ExpertKey(model, layer, expert).as_object_key()
+        assert text == f"{model}/l{layer}-e{expert}"
+        back = wire.ExpertKey.from_expert_id(text)
+        assert (back.model, back.layer, back.expert) == (model, layer, expert)
+    buf = ctypes.create_string_buffer(4)
+    assert C.load().ek_expert_id_format(b"model", 1, 2, buf, 4) == C.EK_INVALID_INPUT
+
+
+def _rand(shape, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    if dtype == torch.int8:
+        return torch.randint(-128, 128, shape, generator=g, dtype=torch.int8)
+    if dtype == torch.float8_e4m3fn:
+        return torch.randint(0, 256, shape, generator=g, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    return torch.randn(shape, generator=g).to(dtype)
+
+
+def _same(a, b):
+    return a.dtype == b.dtype and a.shape == b.shape and \
+        torch.equal(a.contiguous().view(torch.uint8), b.contiguous().view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.int8, torch.float8_e4m3fn])
+@pytest.mark.parametrize("shape", [(1, 64), (17, 128), (0, 64), (5,), (2, 3, 4)])
+def test_emit_matches_safetensors(dtype, shape):
+    t = _rand(shape, dtype, 1)
+    mine = wire.emit("data", t)
+    theirs = st_save({"data": t})
+    assert mine == theirs                       # byte for byte, header padding included
+    assert _same(st_load(mine)["data"], t)
+    assert _same(wire.find(theirs, "data"), t)
+
+
+def test_find_in_multi_tensor_blob():
+    tensors = {
+        "model.layers.3.mlp.experts.7.up_proj.weight": _rand((128, 64), torch.bfloat16, 2),
+        "model.layers.3.mlp.experts.7.gate_proj.weight": _rand((128, 64), torch.bfloat16, 3),
+        "model.layers.3.mlp.experts.7.down_proj.weight": _rand((64, 128), torch.bfloat16, 4),
+        "model.layers.3.mlp.experts.7.down_proj.weight_scale_inv": _rand((1, 1), torch.float32, 5),
+    }
+    blob = st_save(tensors, metadata={"format": "pt", "note": "a {nested} \"quoted\" [value]"})
+    for name, t in tensors.items():
+        assert _same(wire.find(blob, name), t)
+    # lookup_suffix: "…down_proj.weight_scale_inv" does not end with "down_proj.weight"
+    assert _same(wire.find_suffix(blob, ["w2.weight", "down_proj.weight"]),
+                 tensors["model.layers.3.mlp.experts.7.down_proj.weight"])
+    assert _same(wire.find_suffix(blob, ["w1.weight", "up_proj.weight"]),
+                 tensors["model.layers.3.mlp.experts.7.up_proj.weight"])
+    with pytest.raises(C.EKError) as ei:
+        wire.find(blob, "data")
+    assert ei.value.status == C.EK_WEIGHT_NOT_FOUND
+    with pytest.raises(C.EKError) as ei:
+        wire.find_suffix(blob, ["w9.weight"])
+    assert ei.value.status == C.EK_WEIGHT_NOT_FOUND
+
+
+def _blob(header: dict, data: bytes = b"", pad=True) -> bytes:
+    h = json.dumps(header, separators=(",", ":")).encode()
+    if pad:
+        h += b" " * ((8 - len(h) % 8) % 8)
+    return struct.pack("<Q", len(h)) + h + data
+
+
+@pytest.mark.parametrize("blob", [
+    b"",
+    b"\x01\x02\x03",
+    struct.pack("<Q", 1 << 40) + b"{}",                                                        # header longer than blob
+    struct.pack("<Q", 2) + b"[]",                                                              # not an object
+    _blob({"data": {"dtype": "BF16", "shape": [2, 4], "data_offsets": [0, 16]}}, b"\0" * 8),   # data truncated
+    _blob({"data": {"dtype": "BF16", "shape": [2, 4], "data_offsets": [0, 12]}}, b"\0" * 16),  # size mismatch
+    _blob({"data": {"dtype": "BF16", "shape": [2, 4], "data_offsets": [8, 4]}}, b"\0" * 16),   # end < begin
+    _blob({"data": {"dtype": "BF16", "shape": [2, -4], "data_offsets": [0, 16]}}, b"\0" * 16),
+    _blob({"data": {"dtype": "U64", "shape": [2], "data_offsets": [0, 16]}}, b"\0" * 16),      # dtype outside ek_dtype
+    _blob({"data": {"dtype": "BF16", "shape": [1, 1, 1, 1, 8], "data_offsets": [0, 16]}}, b"\0" * 16),
+    _blob({"data": {"dtype": "BF16", "shape": [1 << 40, 1 << 40], "data_offsets": [0, 16]}}, b"\0" * 16),
+    struct.pack("<Q", 24) + b'{"data":{"dtype":"BF16",',                                       # cut mid-object
+])
+def test_malformed_blobs_are_rejected(blob):
+    view = C.ek_tensor_view()
+    st = C.load().ek_safetensors_find(blob, len(blob), b"data", ctypes.byref(view))
+    assert st == C.EK_INVALID_INPUT, C.load().ek_last_error()
+
+
+def test_unpadded_header_and_key_order_are_accepted():
+    data = np.arange(8, dtype=np.float32).tobytes()
+    blob = _blob({"__metadata__": {"k": "v"},
+                  "data": {"data_offsets": [0, 32], "shape": [2, 4], "dtype": "F32"}}, data, pad=False)
+    t = wire.find(blob, "data")
+    assert t.dtype == torch.float32 and t.tolist() == [[0, 1, 2, 3], [4, 5, 6, 7]]
+
+
+def test_emit_rejects_small_buffer_and_bad_description():
+    lib = C.load()
+    shape = (ctypes.c_int64 * 2)(2, 4)
+    assert lib.ek_safetensors_size(b"data", 99, 2, shape) == 0
+    assert lib.ek_safetensors_size(b"data", C.EK_BF16, 5, shape) == 0
+    need = lib.ek_safetensors_size(b"data", C.EK_BF16, 2, shape)
+    src = ctypes.create_string_buffer(16)
+    out = ctypes.create_string_buffer(need)
+    assert lib.ek_safetensors_emit(b"data", C.EK_BF16, 2, shape, src, out, need - 1, None) == C.EK_INVALID_INPUT
+    assert lib.ek_safetensors_emit(b"data", C.EK_BF16, 2, shape, src, out, need, None) == C.EK_OK
