@@ -109,6 +109,10 @@ struct ek_layer {
     // staging for host-memory callers (allocated on first use)
     void *st_x = nullptr, *st_w = nullptr, *st_y = nullptr, *st_xp = nullptr;
     int32_t *st_ids = nullptr;
+    // router outputs and staging (allocated on first use)
+    int32_t *rt_ids = nullptr;
+    void *rt_w = nullptr, *st_logits = nullptr;
+    float *st_bias = nullptr;
     void *st_raw = nullptr;                  // raw weight bytes during ingestion
     size_t st_raw_bytes = 0;
     hipStream_t load_stream = nullptr;
@@ -166,7 +170,7 @@ void free_layer(ek_layer *L)
     for (void *p : L->expert_mem) if (p) (void)hipFree(p);
     void *bufs[] = {L->d_slabs, L->counts, L->offsets, L->perm, L->inv_perm, L->row_token,
                     L->block_hist, L->err, L->h, L->yp, L->st_x, L->st_w, L->st_y, L->st_xp,
-                    L->st_ids, L->st_raw, L->lists.count, L->lists.items[0], L->lists.items[1],
+                    L->st_ids, L->st_raw, L->rt_ids, L->rt_w, L->st_logits, L->st_bias, L->lists.count, L->lists.items[0], L->lists.items[1],
                     L->lists.items[2], L->lists.items[3]};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
@@ -1172,6 +1176,145 @@ ek_status ek_expert_destroy(ek_expert *expert)
         delete expert;
         return st;
     )
+}
+
+}  // extern "C"
+
+namespace {
+
+ek_status check_router(ek_layer *L, const ek_router_cfg *r)
+{
+    if (!r) return fail(EK_INVALID_INPUT, "router cfg is NULL");
+    const int E = L->cfg.n_experts, K = L->cfg.top_k;
+    if (r->kind < EK_ROUTER_SOFTMAX_TOPK || r->kind > EK_ROUTER_SIGMOID_GROUP)
+        return fail(EK_INVALID_INPUT, "unknown router kind %d", r->kind);
+    if (r->logits_dtype != EK_BF16 && r->logits_dtype != EK_F16 && r->logits_dtype != EK_F32)
+        return fail(EK_INVALID_INPUT, "logits_dtype must be EK_BF16, EK_F16 or EK_F32 (got %d)", r->logits_dtype);
+    if (r->w_dtype != L->cfg.act_dtype && r->w_dtype != EK_F32)
+        return fail(EK_INVALID_INPUT, "router w_dtype must be the activation dtype or EK_F32 (got %d)", r->w_dtype);
+    if (K > 64) return fail(EK_INVALID_INPUT, "the router kernel takes top_k <= 64 (layer has %d)", K);
+    if (r->kind == EK_ROUTER_SIGMOID_GROUP) {
+        if (r->n_group < 1 || r->n_group > 64 || E % r->n_group)
+            return fail(EK_INVALID_INPUT, "n_group = %d must divide n_experts = %d and be in [1, 64]", r->n_group, E);
+        const int G = E / r->n_group;
+        if (G < 2) return fail(EK_INVALID_INPUT, "groups of %d expert(s): the group score needs two", G);
+        if (r->topk_group < 1 || r->topk_group > r->n_group || (int64_t)r->topk_group * G < K)
+            return fail(EK_INVALID_INPUT, "topk_group = %d must be in [1, n_group] and keep at least top_k experts",
+                        r->topk_group);
+        if (!(r->routed_scaling == r->routed_scaling)) return fail(EK_INVALID_INPUT, "routed_scaling is NaN");
+    } else if (r->bias) {
+        return fail(EK_INVALID_INPUT, "a correction bias belongs to EK_ROUTER_SIGMOID_GROUP only");
+    }
+    return EK_OK;
+}
+
+ek_status ensure_router_ws(ek_layer *L, bool host)
+{
+    const int64_t T = L->cfg.max_tokens, K = L->cfg.top_k, E = L->cfg.n_experts;
+    if (!L->rt_ids) {
+        EK_TRY(dev_alloc((void **)&L->rt_ids, (size_t)T * K * 4, "router ids"));
+        EK_TRY(dev_alloc(&L->rt_w, (size_t)T * K * 4, "router weights"));
+    }
+    if (host && !L->st_logits) {
+        EK_TRY(dev_alloc(&L->st_logits, (size_t)T * E * 4, "logits staging"));
+        EK_TRY(dev_alloc((void **)&L->st_bias, (size_t)E * 4, "bias staging"));
+    }
+    return EK_OK;
+}
+
+// router on stream s; logits / bias are device addresses
+ek_status enqueue_router(ek_layer *L, const ek_router_cfg *r, const void *logits, const float *bias, int64_t T,
+                         int32_t *ids, void *w, hipStream_t s)
+{
+    ek::RouterArgs a;
+    a.logits = logits; a.logits_dt = r->logits_dtype; a.bias = bias; a.T = T;
+    a.E = L->cfg.n_experts; a.K = L->cfg.top_k; a.kind = r->kind; a.renorm = r->renorm;
+    a.n_group = r->n_group; a.topk_group = r->topk_group;
+    a.mask_neg_inf = (r->flags & EK_ROUTER_MASK_NEG_INF) != 0;
+    a.routed_scaling = r->routed_scaling; a.ids = ids; a.w = w; a.w_dt = r->w_dtype;
+    EK_HIP(ek::launch_router(a, s));
+    return EK_OK;
+}
+
+// shared body of ek_layer_route (x == y == nullptr) and ek_layer_forward_logits
+ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, const ek_router_cfg *rcfg,
+                            int64_t T, void *y, int32_t *ids_out, void *w_out, const ek_route_out *route,
+                            int32_t mem, void *stream, bool forward)
+{
+    if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+    EK_TRY(check_router(layer, rcfg));
+    if (T < 0 || T > layer->cfg.max_tokens)
+        return fail(EK_INVALID_INPUT, "T = %lld outside [0, max_tokens = %lld]", (long long)T,
+                    (long long)layer->cfg.max_tokens);
+    if (mem != EK_HOST && mem != EK_DEVICE) return fail(EK_INVALID_INPUT, "bad mem %d", mem);
+    if (T > 0 && (!logits || (forward && (!x || !y)) || (!forward && (!ids_out || !w_out))))
+        return fail(EK_INVALID_INPUT, "NULL tensor pointer");
+    if (mem == EK_HOST && stream)
+        return fail(EK_INVALID_INPUT, "host-memory calls are blocking: stream must be NULL");
+    DeviceGuard dg(layer->cfg.device_id);
+    if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
+    Timer tm;
+    const int64_t H = layer->cfg.hidden, K = layer->cfg.top_k, E = layer->cfg.n_experts, P = T * K;
+    const int w_f32 = rcfg->w_dtype == EK_F32;
+    const size_t w_bytes = (size_t)P * (w_f32 ? 4 : 2);
+    const size_t l_bytes = (size_t)T * E * (rcfg->logits_dtype == EK_F32 ? 4 : 2);
+    std::lock_guard<std::mutex> lk(layer->mu);
+    hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+    if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
+    EK_TRY(ensure_router_ws(layer, mem == EK_HOST));
+    const void *d_logits = logits, *d_x = x;
+    const float *d_bias = (const float *)rcfg->bias;
+    void *d_y = y;
+    const hipMemcpyKind back = mem == EK_HOST ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice;
+    if (mem == EK_HOST) {
+        if (forward) EK_TRY(ensure_io_staging(layer));
+        if (T > 0) {
+            EK_HIP(hipMemcpyAsync(layer->st_logits, logits, l_bytes, hipMemcpyHostToDevice, s));
+            if (forward) EK_HIP(hipMemcpyAsync(layer->st_x, x, (size_t)T * H * 2, hipMemcpyHostToDevice, s));
+        }
+        if (rcfg->bias) {
+            EK_HIP(hipMemcpyAsync(layer->st_bias, rcfg->bias, (size_t)E * 4, hipMemcpyHostToDevice, s));
+            d_bias = layer->st_bias;
+        }
+        d_logits = layer->st_logits;
+        d_x = layer->st_x;
+        d_y = layer->st_y;
+    }
+    EK_TRY(enqueue_router(layer, rcfg, d_logits, d_bias, T, layer->rt_ids, layer->rt_w, s));
+    if (P > 0 && ids_out) EK_HIP(hipMemcpyAsync(ids_out, layer->rt_ids, (size_t)P * 4, back, s));
+    if (P > 0 && w_out) EK_HIP(hipMemcpyAsync(w_out, layer->rt_w, w_bytes, back, s));
+    ek_status st = EK_OK;
+    if (forward) {
+        EK_TRY(enqueue_forward(layer, d_x, layer->rt_ids, layer->rt_w, w_f32, T, d_y, s));
+        if (mem == EK_HOST && T > 0) EK_HIP(hipMemcpyAsync(y, layer->st_y, (size_t)T * H * 2, hipMemcpyDeviceToHost, s));
+        EK_TRY(copy_route_out(layer, route, P, mem, s));
+        if (!stream) st = finish_blocking(layer, s);
+        std::lock_guard<std::mutex> sl(layer->stats_mu);
+        layer->stats.forward_calls += 1;
+        layer->stats.tokens += T;
+        layer->stats.pairs += P;
+        if (!stream) layer->stats.last_forward_us = tm.us();
+    } else if (!stream) {
+        EK_HIP(hipStreamSynchronize(s));
+    }
+    return st;
+}
+
+}  // namespace
+
+extern "C" {
+
+ek_status ek_layer_route(ek_layer *layer, const void *logits, const ek_router_cfg *router, int64_t T,
+                         int32_t *ids, void *w, int32_t mem, void *stream)
+{
+    EK_GUARDED(return route_and_forward(layer, nullptr, logits, router, T, nullptr, ids, w, nullptr, mem, stream, false);)
+}
+
+ek_status ek_layer_forward_logits(ek_layer *layer, const void *x, const void *logits, const ek_router_cfg *router,
+                                  int64_t T, void *y, int32_t *ids, void *w, const ek_route_out *route,
+                                  int32_t mem, void *stream)
+{
+    EK_GUARDED(return route_and_forward(layer, x, logits, router, T, y, ids, w, route, mem, stream, true);)
 }
 
 }  // extern "C"

@@ -55,6 +55,25 @@ inline int64_t list_capacity(int list, int64_t P, int64_t E)
     return by_rows < E ? by_rows : E;
 }
 
+// ---- router (logits -> ids, gate weights) -------------------------------------
+struct RouterArgs {
+    const void *logits;       // [T, E]
+    int32_t logits_dt;        // 0 bf16, 1 f16, 2 f32
+    const float *bias;        // [E] or nullptr (kind 4: added to the scores for the choice only)
+    int64_t T;
+    int32_t E, K;
+    int32_t kind;             // ek_router_kind
+    int32_t renorm;
+    int32_t n_group, topk_group;
+    int32_t mask_neg_inf;     // kind 4: experts outside the kept groups compete with -inf instead of 0
+    float routed_scaling;
+    int32_t *ids;             // [T, K]
+    void *w;                  // [T, K]
+    int32_t w_dt;             // 0 bf16, 1 f16, 2 f32
+};
+// needs E <= 1024, K <= 64, n_group <= 64 (checked by the caller)
+hipError_t launch_router(const RouterArgs &a, hipStream_t s);
+
 // ---- routing (pack) ---------------------------------------------------------
 struct PackArgs {
     const int32_t *ids;       // [P]

@@ -50,6 +50,16 @@ class ek_tensor_view(ctypes.Structure):
                 ("dtype", ctypes.c_int32), ("nbytes", ctypes.c_int64)]
 
 
+class ek_router_cfg(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int32), ("renorm", ctypes.c_int32), ("n_group", ctypes.c_int32),
+                ("topk_group", ctypes.c_int32), ("routed_scaling", ctypes.c_float), ("flags", ctypes.c_int32),
+                ("logits_dtype", ctypes.c_int32), ("w_dtype", ctypes.c_int32), ("bias", ctypes.c_void_p)]
+
+
+(EK_ROUTER_SOFTMAX_TOPK, EK_ROUTER_TOPK_RAW, EK_ROUTER_TOPK_SOFTMAX, EK_ROUTER_TOPK_SIGMOID,
+ EK_ROUTER_SIGMOID_GROUP) = range(5)
+EK_ROUTER_MASK_NEG_INF = 1
+
 _P = ctypes.c_void_p
 _PP = ctypes.POINTER(ctypes.c_void_p)
 _I32, _I64 = ctypes.c_int32, ctypes.c_int64
@@ -85,6 +95,9 @@ PROTOTYPES = {
     "ek_worker_forward": (_I32, [_P, ctypes.c_char_p, _P, _SZ, _P, _SZ, ctypes.POINTER(_SZ)]),
     "ek_worker_forward_batch": (_I32, [_P, _I32, _STRS, _PP, ctypes.POINTER(_SZ), _PP, ctypes.POINTER(_SZ),
                                        ctypes.POINTER(_SZ)]),
+    "ek_layer_route": (_I32, [_P, _P, ctypes.POINTER(ek_router_cfg), _I64, _P, _P, _I32, _P]),
+    "ek_layer_forward_logits": (_I32, [_P, _P, _P, ctypes.POINTER(ek_router_cfg), _I64, _P, _P, _P,
+                                       ctypes.POINTER(ek_route_out), _I32, _P]),
     "ek_layer_profile": (_I32, [_P, _I32]),
     "ek_layer_get_stats": (_I32, [_P, ctypes.POINTER(ek_stats)]),
     "ek_chain_create": (_I32, [_PP, _I32, _PP]),

@@ -122,6 +122,19 @@ def _desc(w: Optional[torch.Tensor], scale: Optional[torch.Tensor]):
 
 
 @dataclass
+class RouterConfig:
+    """Which of the reference shims' routers to run in front of pack (ek_router_cfg)."""
+    kind: int = C.EK_ROUTER_SOFTMAX_TOPK
+    renorm: bool = True              # norm_topk_prob
+    n_group: int = 1
+    topk_group: int = 1
+    routed_scaling: float = 1.0
+    mask_neg_inf: bool = False
+    w_dtype: Optional[torch.dtype] = None    # None: the layer's activation dtype
+    bias: Optional[torch.Tensor] = None      # e_score_correction_bias [E] fp32
+
+
+@dataclass
 class RouteTables:
     counts: torch.Tensor
     offsets: torch.Tensor
@@ -205,6 +218,43 @@ class HipLayer:
         C.check(self._lib.ek_layer_expert_forward(self._h, e, _ptr(x), x.shape[0], _ptr(out), _mem(x),
                                                   _stream_ptr(stream)))
         return out
+
+    def _router_cfg(self, r: RouterConfig, logits: torch.Tensor):
+        cfg = C.ek_router_cfg(kind=r.kind, renorm=int(r.renorm), n_group=r.n_group, topk_group=r.topk_group,
+                              routed_scaling=r.routed_scaling,
+                              flags=C.EK_ROUTER_MASK_NEG_INF if r.mask_neg_inf else 0,
+                              logits_dtype=_DT[logits.dtype], w_dtype=_DT[r.w_dtype or self.act_dtype])
+        bias = None
+        if r.bias is not None:
+            bias = r.bias.to(device=logits.device, dtype=torch.float32).contiguous()
+            cfg.bias = bias.data_ptr()
+        return cfg, bias
+
+    def route(self, logits: torch.Tensor, router: RouterConfig, stream=None):
+        """logits [T,E] -> (ids [T,K] int32, w [T,K])."""
+        logits = logits.contiguous()
+        T, K = logits.shape[0], self.cfg.top_k
+        cfg, keep = self._router_cfg(router, logits)
+        ids = torch.empty(T, K, dtype=torch.int32, device=logits.device)
+        w = torch.empty(T, K, dtype=router.w_dtype or self.act_dtype, device=logits.device)
+        C.check(self._lib.ek_layer_route(self._h, _ptr(logits), ctypes.byref(cfg), T, _ptr(ids), _ptr(w),
+                                         _mem(logits), _stream_ptr(stream)))
+        del keep
+        return ids, w
+
+    def forward_logits(self, x: torch.Tensor, logits: torch.Tensor, router: RouterConfig, stream=None):
+        """Router + layer in one call; returns (y, ids, w)."""
+        x, logits = x.contiguous(), logits.contiguous()
+        T, K = x.shape[0], self.cfg.top_k
+        assert logits.shape[0] == T and _mem(x) == _mem(logits)
+        cfg, keep = self._router_cfg(router, logits)
+        y = torch.empty_like(x)
+        ids = torch.empty(T, K, dtype=torch.int32, device=x.device)
+        w = torch.empty(T, K, dtype=router.w_dtype or self.act_dtype, device=x.device)
+        C.check(self._lib.ek_layer_forward_logits(self._h, _ptr(x), _ptr(logits), ctypes.byref(cfg), T, _ptr(y),
+                                                  _ptr(ids), _ptr(w), None, _mem(x), _stream_ptr(stream)))
+        del keep
+        return y, ids, w
 
     def experts_forward(self, experts: Sequence[int], xs: Sequence[torch.Tensor], stream=None):
         """Several per-expert calls as one grouped launch; xs[i] is [n_i, H]."""

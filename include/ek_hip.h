@@ -261,6 +261,52 @@ ek_status ek_layer_profile(ek_layer *layer, int32_t enable);
 /* Snapshot of the layer's counters (waits for recorded events to complete). */
 ek_status ek_layer_get_stats(ek_layer *layer, ek_stats *out);
 
+/* ---- routers: logits -> (ids, gate weights), fused in front of pack ----------
+ * Every choice is "larger value first, lower expert index on equal values"
+ * (torch.topk leaves the order of equal values open). */
+typedef enum ek_router_kind {
+    EK_ROUTER_SOFTMAX_TOPK = 0,  /* softmax_fp32 over E, top-K, w /= sum(w) if renorm, cast:
+                                    expertkit_torch/models/qwen3_moe.py:161-169 */
+    EK_ROUTER_TOPK_RAW = 1,      /* top-K of the logits, w = the logits:
+                                    expertkit_vllm/experts/grpc_expert.py:120-121 */
+    EK_ROUTER_TOPK_SOFTMAX = 2,  /* top-K of the logits, softmax over the K:
+                                    expertkit_vllm/models/deepseek_v2.py:123-128 */
+    EK_ROUTER_TOPK_SIGMOID = 3,  /* top-K of the logits, sigmoid of the K: deepseek_v2.py:123-130 */
+    EK_ROUTER_SIGMOID_GROUP = 4  /* DeepSeek-V3 group-limited routing, called by the reference at
+                                    expertkit_torch/models/deepseek_v3/model.py:142 (the routine
+                                    itself is transformers' DeepseekV3TopkRouter; parameters in
+                                    ek-db/resources/ds-tiny/config.json:26-48): s = sigmoid(logits);
+                                    c = s + bias; group score = sum of the group's two largest c;
+                                    keep the topk_group best groups; top-K of c inside them;
+                                    w = s[ids]; if renorm w /= sum(w) + 1e-20; w *= routed_scaling */
+} ek_router_kind;
+
+/* experts outside the kept groups compete with -inf (newer transformers) instead of 0.0 */
+#define EK_ROUTER_MASK_NEG_INF 1
+
+typedef struct ek_router_cfg {
+    int32_t kind;         /* ek_router_kind */
+    int32_t renorm;       /* norm_topk_prob (kinds 0 and 4) */
+    int32_t n_group;      /* kind 4 */
+    int32_t topk_group;   /* kind 4 */
+    float routed_scaling; /* kind 4 */
+    int32_t flags;        /* EK_ROUTER_* */
+    int32_t logits_dtype; /* EK_F32, EK_BF16 or EK_F16 */
+    int32_t w_dtype;      /* type of the gate weights produced: the layer's act dtype or EK_F32 */
+    const void *bias;     /* kind 4: e_score_correction_bias [E] fp32 (same memory kind as the
+                             call's tensors) or NULL */
+} ek_router_cfg;
+
+/* Router only: logits [T,E] -> ids [T,K] int32, w [T,K] of router->w_dtype. */
+ek_status ek_layer_route(ek_layer *layer, const void *logits, const ek_router_cfg *router, int64_t T,
+                         int32_t *ids, void *w, int32_t mem, void *stream);
+/* ek_layer_forward that takes logits instead of (ids, w): router, pack, FFN and
+ * combine are enqueued back to back.  ids / w (optional) receive what the router chose.
+ * The result is bit-identical to ek_layer_route followed by ek_layer_forward. */
+ek_status ek_layer_forward_logits(ek_layer *layer, const void *x, const void *logits,
+                                  const ek_router_cfg *router, int64_t T, void *y, int32_t *ids, void *w,
+                                  const ek_route_out *route, int32_t mem, void *stream);
+
 /* ---- chain of layers: consecutive MoE layers launched as one HIP graph ------
  * The reference issues one ForwardReq per MoE layer from the attention side
  * (qwen3_moe.py:89-104 is entered once per decoder layer); a chain runs L

@@ -157,6 +157,139 @@ int eko_router_softmax_topk(const float *logits, int64_t T, int E, int K, int re
     return 0;
 }
 
+/*
+ * exp(x) built from IEEE-754 single operations only (fused multiply-add,
+ * multiply, add, round-to-nearest-even), so that any conforming machine gives
+ * the same bits: Cody-Waite reduction by ln 2, the degree-5 polynomial of
+ * Cephes' expf, scaling by an exponent-field constant.  The argument is
+ * clamped to [-87, 88], where the result is a normal number.  Within 2 ulp of
+ * the exact value (pinned against libm in tests/test_oracle_router.py).
+ * Compile with -ffp-contract=off: the unfused operations must stay unfused.
+ */
+float eko_expf(float x)
+{
+    x = x < -87.0f ? -87.0f : (x > 88.0f ? 88.0f : x);
+    const float n = rintf(x * 1.44269504088896341f);
+    float r = fmaf(n, -0.693359375f, x);
+    r = fmaf(n, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = fmaf(p, r, 1.3981999507e-3f);
+    p = fmaf(p, r, 8.3334519073e-3f);
+    p = fmaf(p, r, 4.1665795894e-2f);
+    p = fmaf(p, r, 1.6666665459e-1f);
+    p = fmaf(p, r, 5.0000001201e-1f);
+    const float y = fmaf(r * r, p, r) + 1.0f;
+    return y * bits_f32((uint32_t)((int32_t)n + 127) << 23);
+}
+float eko_sigmoidf(float x) { return 1.0f / (1.0f + eko_expf(-x)); }
+
+/* larger value first, lower index on equal values */
+static int pick_best(const float *v, const char *used, int n)
+{
+    int best = -1;
+    for (int e = 0; e < n; ++e)
+        if (!used[e] && (best < 0 || v[e] > v[best])) best = e;
+    return best;
+}
+
+/*
+ * The routers of the reference's model shims, one token at a time.
+ *   kind 0  softmax_fp32 over E, top-K, optional renormalisation, cast
+ *           (expertkit_torch/models/qwen3_moe.py:161-169).  The choice is made on
+ *           the logits: softmax is monotone, so this is the choice torch.topk
+ *           makes on the probabilities wherever those are distinct.
+ *   kind 1  top-K of the raw logits, weights = the logits
+ *           (expertkit_vllm/experts/grpc_expert.py:120-121)
+ *   kind 2  top-K of the logits, softmax over the K (expertkit_vllm/models/deepseek_v2.py:123-128)
+ *   kind 3  top-K of the logits, sigmoid of the K   (deepseek_v2.py:123-130)
+ *   kind 4  DeepSeek-V3 group-limited routing.  The reference calls it at
+ *           expertkit_torch/models/deepseek_v3/model.py:142; the routine is
+ *           transformers' DeepseekV3TopkRouter.forward (third party, pinned by the
+ *           reference at transformers==4.51.3, not part of the reference tree):
+ *             s = sigmoid(logits); c = s + bias;
+ *             group score = sum of the two largest c of the group;
+ *             keep the topk_group best groups; c of every other expert := 0
+ *             (-inf in newer transformers: mask_neg_inf); ids = top-K of c;
+ *             w = s[ids]; if renorm: w /= sum(w) + 1e-20; w *= routed_scaling.
+ * exp and sigmoid are eko_expf / eko_sigmoidf.  Sums run over k (or e) ascending.
+ * logits [T,E] of logits_dt; bias [E] f32 or NULL; ids [T,K] int32; w [T,K] of w_dt.
+ */
+int eko_route(int kind, const void *logits, int logits_dt, const float *bias, int64_t T, int E, int K,
+              int renorm, int n_group, int topk_group, int mask_neg_inf, float routed_scaling,
+              int32_t *ids, void *w, int w_dt)
+{
+    if (K > E || K <= 0 || kind < 0 || kind > 4) return -1;
+    if (kind == 4 && (n_group < 1 || E % n_group || E / n_group < 2 || topk_group < 1 || topk_group > n_group ||
+                      (int64_t)topk_group * (E / n_group) < K))
+        return -1;
+    float *v = (float *)malloc(sizeof(float) * (size_t)E);      /* the value the choice is made on */
+    float *sc = (float *)malloc(sizeof(float) * (size_t)E);     /* kind 4: unbiased scores */
+    float *wk = (float *)malloc(sizeof(float) * (size_t)K);
+    float *gs = (float *)malloc(sizeof(float) * (size_t)(n_group > 0 ? n_group : 1));
+    char *used = (char *)malloc((size_t)E);
+    char *gkeep = (char *)malloc((size_t)(n_group > 0 ? n_group : 1));
+    if (!v || !sc || !wk || !gs || !used || !gkeep) { free(v); free(sc); free(wk); free(gs); free(used); free(gkeep); return -2; }
+    for (int64_t t = 0; t < T; ++t) {
+        for (int e = 0; e < E; ++e) v[e] = load_act(logits, t * E + e, logits_dt);
+        float m = 0.f, s = 1.f;
+        if (kind == 0) {
+            m = v[0];
+            for (int e = 1; e < E; ++e) if (v[e] > m) m = v[e];
+            s = 0.f;
+            for (int e = 0; e < E; ++e) s += eko_expf(v[e] - m);
+        } else if (kind == 4) {
+            const int G = E / n_group;
+            for (int e = 0; e < E; ++e) {
+                sc[e] = eko_sigmoidf(v[e]);
+                v[e] = bias ? sc[e] + bias[e] : sc[e];
+            }
+            for (int g = 0; g < n_group; ++g) {
+                float b0 = -INFINITY, b1 = -INFINITY;
+                for (int i = 0; i < G; ++i) {
+                    const float c = v[g * G + i];
+                    if (c > b0) { b1 = b0; b0 = c; }
+                    else if (c > b1) b1 = c;
+                }
+                gs[g] = b0 + b1;
+            }
+            memset(used, 0, (size_t)n_group);
+            memset(gkeep, 0, (size_t)n_group);
+            for (int k = 0; k < topk_group; ++k) {
+                const int g = pick_best(gs, used, n_group);
+                used[g] = 1;
+                gkeep[g] = 1;
+            }
+            for (int e = 0; e < E; ++e)
+                if (!gkeep[e / G]) v[e] = mask_neg_inf ? -INFINITY : 0.f;
+        }
+        memset(used, 0, (size_t)E);
+        for (int k = 0; k < K; ++k) {
+            const int best = pick_best(v, used, E);
+            used[best] = 1;
+            ids[t * K + k] = best;
+        }
+        for (int k = 0; k < K; ++k) {
+            const float l = v[ids[t * K + k]];
+            switch (kind) {
+            case 0: wk[k] = eko_expf(l - m) / s; break;
+            case 1: wk[k] = l; break;
+            case 2: wk[k] = eko_expf(l - v[ids[t * K]]); break;
+            case 3: wk[k] = eko_sigmoidf(l); break;
+            default: wk[k] = sc[ids[t * K + k]]; break;
+            }
+        }
+        if (kind == 2 || ((kind == 0 || kind == 4) && renorm)) {
+            float tot = 0.f;
+            for (int k = 0; k < K; ++k) tot += wk[k];
+            if (kind == 4) tot += 1e-20f;
+            for (int k = 0; k < K; ++k) wk[k] = wk[k] / tot;
+        }
+        for (int k = 0; k < K; ++k) store_act(w, t * K + k, kind == 4 ? wk[k] * routed_scaling : wk[k], w_dt);
+    }
+    free(v); free(sc); free(wk); free(gs); free(used); free(gkeep);
+    return 0;
+}
+
 /* ------------------------------------------------------------------ pack */
 
 /*

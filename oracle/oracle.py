@@ -87,6 +87,31 @@ def router(logits: torch.Tensor, k: int, renorm: bool = True, w_dtype=torch.floa
     return ids, w
 
 
+def expf(x: torch.Tensor) -> torch.Tensor:
+    """eko_expf element by element (the IEEE-operations-only exp the routers use)."""
+    L = lib()
+    L.eko_expf.restype = ctypes.c_float
+    L.eko_expf.argtypes = [ctypes.c_float]
+    return torch.tensor([L.eko_expf(float(v)) for v in x.flatten().tolist()], dtype=torch.float32).reshape(x.shape)
+
+
+def route(kind: int, logits: torch.Tensor, k: int, renorm: bool = True, w_dtype=torch.float32, bias=None,
+          n_group: int = 1, topk_group: int = 1, mask_neg_inf: bool = False, routed_scaling: float = 1.0):
+    """The reference shims' routers (see eko_route): kind 0 Qwen3, 1-3 the vLLM shims, 4 DeepSeek-V3."""
+    logits = logits.contiguous()
+    T, E = logits.shape
+    ids = torch.empty(T, k, dtype=torch.int32)
+    w = torch.empty(T, k, dtype=w_dtype)
+    if bias is not None:
+        bias = bias.contiguous().float()
+    rc = lib().eko_route(kind, _p(logits), _DT[logits.dtype], _p(bias), _i64(T), E, k, int(renorm), n_group,
+                         topk_group, int(mask_neg_inf), ctypes.c_float(routed_scaling), _p(ids), _p(w),
+                         _DT[w_dtype])
+    if rc:
+        raise ValueError(f"eko_route rc={rc}")
+    return ids, w
+
+
 def pack(ids: torch.Tensor, n_experts: int):
     """Group (token, slot) pairs by expert (controller/executor.rs:283-304).
 
@@ -237,6 +262,39 @@ def torch_router(logits: torch.Tensor, k: int, renorm: bool = True, w_dtype=torc
     if renorm:
         rw = rw / rw.sum(dim=-1, keepdim=True)
     return sel.to(torch.int32), rw.to(w_dtype)
+
+
+def torch_route(kind: int, logits: torch.Tensor, k: int, renorm: bool = True, w_dtype=torch.float32, bias=None,
+                n_group: int = 1, topk_group: int = 1, mask_neg_inf: bool = False, routed_scaling: float = 1.0):
+    """The same routers in torch primitives, written after the reference's lines (kinds 0-3) and
+    after the published DeepseekV3TopkRouter.forward (kind 4)."""
+    if kind == 0:      # qwen3_moe.py:161-169
+        p = torch.softmax(logits, dim=1, dtype=torch.float)
+        w, ids = torch.topk(p, k, dim=-1)
+        if renorm:
+            w = w / w.sum(dim=-1, keepdim=True)
+        return ids.to(torch.int32), w.to(w_dtype)
+    if kind in (1, 2, 3):   # grpc_expert.py:120-121, deepseek_v2.py:123-130
+        w, ids = torch.topk(logits, k, dim=-1)
+        if kind == 2:
+            w = torch.softmax(w, dim=-1)
+        elif kind == 3:
+            w = torch.sigmoid(w)
+        return ids.to(torch.int32), w.to(w_dtype)
+    T, E = logits.shape
+    scores = logits.float().sigmoid()
+    choice = scores + bias if bias is not None else scores.clone()
+    group_scores = choice.view(T, n_group, E // n_group).topk(2, dim=-1)[0].sum(dim=-1)
+    group_idx = torch.topk(group_scores, k=topk_group, dim=-1, sorted=False)[1]
+    group_mask = torch.zeros_like(group_scores)
+    group_mask.scatter_(1, group_idx, 1)
+    score_mask = group_mask.unsqueeze(-1).expand(T, n_group, E // n_group).reshape(T, E)
+    choice = choice.masked_fill(~score_mask.bool(), float("-inf") if mask_neg_inf else 0.0)
+    ids = torch.topk(choice, k=k, dim=-1, sorted=True)[1]
+    w = scores.gather(1, ids)
+    if renorm:
+        w = w / (w.sum(dim=-1, keepdim=True) + 1e-20)
+    return ids.to(torch.int32), (w * routed_scaling).to(w_dtype)
 
 
 def torch_dequant_channel(q: torch.Tensor, scale: torch.Tensor, dtype=torch.bfloat16) -> torch.Tensor:
