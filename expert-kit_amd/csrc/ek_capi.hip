@@ -122,6 +122,11 @@ struct ek_layer {
 
     ek_stats stats{};
     std::mutex stats_mu;
+    // worker_expert_activation: pairs per expert, summed by the pack kernel on the device
+    // (fused calls) and on the host (per-expert calls)
+    uint64_t *d_activation = nullptr;
+    std::vector<int64_t> h_activation;
+    ek_histogram forward_hist{};             // worker_forward: blocking compute calls, microseconds
 
     // per-phase event timing (ek_layer_profile)
     bool profiling = false;
@@ -170,7 +175,7 @@ void free_layer(ek_layer *L)
     for (void *p : L->expert_mem) if (p) (void)hipFree(p);
     void *bufs[] = {L->d_slabs, L->counts, L->offsets, L->perm, L->inv_perm, L->row_token,
                     L->block_hist, L->err, L->h, L->yp, L->st_x, L->st_w, L->st_y, L->st_xp,
-                    L->st_ids, L->st_raw, L->rt_ids, L->rt_w, L->st_logits, L->st_bias, L->lists.count, L->lists.items[0], L->lists.items[1],
+                    L->d_activation, L->st_ids, L->st_raw, L->rt_ids, L->rt_w, L->st_logits, L->st_bias, L->lists.count, L->lists.items[0], L->lists.items[1],
                     L->lists.items[2], L->lists.items[3]};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
@@ -238,6 +243,9 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     A((void **)&L->row_token, sizeof(int32_t) * pmax, "row_token");
     A((void **)&L->block_hist, sizeof(int32_t) * nblocks * E, "block_hist");
     A((void **)&L->err, sizeof(int32_t) * 4, "err");
+    A((void **)&L->d_activation, sizeof(uint64_t) * E, "activation counters");
+    L->h_activation.assign(E, 0);
+    for (int i = 0; i < 10; ++i) L->forward_hist.le[i] = 4000.0 * i;   // the reference's buckets (metrics.rs:51)
     A(&L->h, (size_t)pmax * cfg->inter * 2, "h");
     A(&L->yp, (size_t)pmax * cfg->hidden * 2, "yp");
     A((void **)&L->lists.count, sizeof(int32_t) * ek::kNumLists, "work list counts");
@@ -250,6 +258,7 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     if (st == EK_OK) {
         hipError_t e = hipMemset(L->d_slabs, 0, sizeof(ek::ExpertSlab) * E);
         if (e == hipSuccess) e = hipMemset(L->err, 0, sizeof(int32_t) * 4);
+        if (e == hipSuccess) e = hipMemset(L->d_activation, 0, sizeof(uint64_t) * E);
         if (e == hipSuccess) e = hipMemset(L->lists.count, 0, sizeof(int32_t) * ek::kNumLists);
         if (e == hipSuccess) e = hipHostMalloc((void **)&L->h_err, sizeof(int32_t) * 4, hipHostMallocDefault);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
@@ -425,6 +434,16 @@ struct Timer {
     }
 };
 
+// one observation of the worker_forward histogram; the caller holds stats_mu
+void observe_forward(ek_layer *L, double us)
+{
+    ek_histogram &h = L->forward_hist;
+    for (int i = 0; i < 10; ++i) if (us <= h.le[i]) h.cumulative[i] += 1;
+    h.cumulative[10] += 1;
+    h.count += 1;
+    h.sum += us;
+}
+
 ek_status ensure_io_staging(ek_layer *L)
 {
     if (L->st_x) return EK_OK;
@@ -473,6 +492,7 @@ ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_lo
     a.inv_perm = L->inv_perm;
     a.row_token = L->row_token;
     a.err = L->err;
+    a.activation = check_loaded ? L->d_activation : nullptr;
     if (check_loaded) a.lists = L->lists;
     else a.lists = ek::WorkLists{{nullptr, nullptr, nullptr, nullptr}, nullptr};
     return a;
@@ -717,7 +737,7 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
             layer->stats.forward_calls += 1;
             layer->stats.tokens += T;
             layer->stats.pairs += P;
-            if (!stream) layer->stats.last_forward_us = tm.us();
+            if (!stream) { layer->stats.last_forward_us = tm.us(); observe_forward(layer, layer->stats.last_forward_us); }
         }
         return st;
     )
@@ -783,6 +803,7 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
         DeviceGuard dg(layer->cfg.device_id);
         if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
         const int64_t H = layer->cfg.hidden;
+        Timer tm;
         std::lock_guard<std::mutex> lk(layer->mu);
         if (!layer->expert_mem[expert])
             return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", expert);
@@ -806,6 +827,8 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
         {
             std::lock_guard<std::mutex> sl(layer->stats_mu);
             layer->stats.expert_forward_calls += 1;
+            layer->h_activation[expert] += n;
+            if (!stream) observe_forward(layer, tm.us());
         }
         return EK_OK;
     )
@@ -848,6 +871,7 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
         }
         DeviceGuard dg(layer->cfg.device_id);
         if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
+        Timer tm;
         std::lock_guard<std::mutex> lk(layer->mu);
         for (int i = 0; i < n_calls; ++i)
             if (!layer->expert_mem[experts[i]])
@@ -917,7 +941,37 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
         {
             std::lock_guard<std::mutex> sl(layer->stats_mu);
             layer->stats.expert_forward_calls += n_calls;
+            for (int i = 0; i < n_calls; ++i) layer->h_activation[experts[i]] += rows[i];
+            // the reference observes one duration per request; the requests of a batch share this one
+            if (!stream) { const double us = tm.us(); for (int i = 0; i < n_calls; ++i) observe_forward(layer, us); }
         }
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_get_activation(ek_layer *layer, int64_t *counts)
+{
+    EK_GUARDED(
+        if (!layer || !counts) return fail(EK_INVALID_INPUT, "NULL argument");
+        DeviceGuard dg(layer->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
+        const int E = layer->cfg.n_experts;
+        std::lock_guard<std::mutex> lk(layer->mu);
+        EK_HIP(hipDeviceSynchronize());   // calls enqueued on caller streams count once they have run
+        std::vector<uint64_t> dev(E);
+        EK_HIP(hipMemcpy(dev.data(), layer->d_activation, sizeof(uint64_t) * E, hipMemcpyDeviceToHost));
+        std::lock_guard<std::mutex> sl(layer->stats_mu);
+        for (int e = 0; e < E; ++e) counts[e] = (int64_t)dev[e] + layer->h_activation[e];
+        return EK_OK;
+    )
+}
+
+ek_status ek_layer_get_forward_histogram(ek_layer *layer, ek_histogram *out)
+{
+    EK_GUARDED(
+        if (!layer || !out) return fail(EK_INVALID_INPUT, "NULL argument");
+        std::lock_guard<std::mutex> sl(layer->stats_mu);
+        *out = layer->forward_hist;
         return EK_OK;
     )
 }
@@ -1293,7 +1347,7 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
         layer->stats.forward_calls += 1;
         layer->stats.tokens += T;
         layer->stats.pairs += P;
-        if (!stream) layer->stats.last_forward_us = tm.us();
+        if (!stream) { layer->stats.last_forward_us = tm.us(); observe_forward(layer, layer->stats.last_forward_us); }
     } else if (!stream) {
         EK_HIP(hipStreamSynchronize(s));
     }

@@ -102,6 +102,7 @@ __global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
             total += t;
         }
         a.counts[e] = total;
+        if (a.activation) a.activation[e] += (uint64_t)total;
         if (total > 0 && a.slabs != nullptr && a.slabs[e].upgate == nullptr) atomicOr(a.err, 2);
     }
     int32_t sum;
@@ -229,6 +230,7 @@ __global__ __launch_bounds__(1024) void pack_fused_kernel(PackArgs a, int nbits)
     if (e < a.E) {
         for (int w = 0; w < 16; ++w) total += lds[w * a.E + e];
         a.counts[e] = total;
+        if (a.activation) a.activation[e] += (uint64_t)total;
         if (total > 0 && a.slabs != nullptr && a.slabs[e].upgate == nullptr) atomicOr(lerr, 2);
     }
     int32_t sum;

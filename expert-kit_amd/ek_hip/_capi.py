@@ -50,6 +50,11 @@ class ek_tensor_view(ctypes.Structure):
                 ("dtype", ctypes.c_int32), ("nbytes", ctypes.c_int64)]
 
 
+class ek_histogram(ctypes.Structure):
+    _fields_ = [("le", ctypes.c_double * 10), ("cumulative", ctypes.c_int64 * 11), ("sum", ctypes.c_double),
+                ("count", ctypes.c_int64)]
+
+
 class ek_router_cfg(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int32), ("renorm", ctypes.c_int32), ("n_group", ctypes.c_int32),
                 ("topk_group", ctypes.c_int32), ("routed_scaling", ctypes.c_float), ("flags", ctypes.c_int32),
@@ -98,6 +103,8 @@ PROTOTYPES = {
     "ek_layer_route": (_I32, [_P, _P, ctypes.POINTER(ek_router_cfg), _I64, _P, _P, _I32, _P]),
     "ek_layer_forward_logits": (_I32, [_P, _P, _P, ctypes.POINTER(ek_router_cfg), _I64, _P, _P, _P,
                                        ctypes.POINTER(ek_route_out), _I32, _P]),
+    "ek_layer_get_activation": (_I32, [_P, ctypes.POINTER(_I64)]),
+    "ek_layer_get_forward_histogram": (_I32, [_P, ctypes.POINTER(ek_histogram)]),
     "ek_layer_profile": (_I32, [_P, _I32]),
     "ek_layer_get_stats": (_I32, [_P, ctypes.POINTER(ek_stats)]),
     "ek_chain_create": (_I32, [_PP, _I32, _PP]),

@@ -294,6 +294,18 @@ class HipLayer:
         C.check(self._lib.ek_worker_forward_batch(self._h, n, ids, rp, rl, op, oc, ol))
         return [bufs[i].raw[:ol[i]] for i in range(n)]
 
+    def activation(self) -> torch.Tensor:
+        """worker_expert_activation: rows given to each expert so far (metrics.rs:56-62)."""
+        out = (ctypes.c_int64 * self.cfg.n_experts)()
+        C.check(self._lib.ek_layer_get_activation(self._h, out))
+        return torch.tensor(list(out), dtype=torch.int64)
+
+    def forward_histogram(self) -> dict:
+        """worker_forward: durations of blocking compute calls in the reference's buckets."""
+        h = C.ek_histogram()
+        C.check(self._lib.ek_layer_get_forward_histogram(self._h, ctypes.byref(h)))
+        return {"le": list(h.le), "cumulative": list(h.cumulative), "sum": h.sum, "count": h.count}
+
     def profile(self, enable: bool) -> None:
         C.check(self._lib.ek_layer_profile(self._h, int(enable)))
 

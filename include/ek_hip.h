@@ -258,6 +258,24 @@ ek_status ek_worker_forward_batch(ek_layer *layer, int32_t n_calls, const char *
  * At most 1024 calls are recorded between two ek_layer_get_stats calls. */
 ek_status ek_layer_profile(ek_layer *layer, int32_t enable);
 
+/* worker_expert_activation (metrics.rs:56-62; incremented by the number of
+ * sequences of each request, worker/server.rs:39-45): counts[e] = rows expert e
+ * has been given since the layer was created, over all compute entry points.
+ * The fused calls add the pack step's counts[] on the device.  counts: [E], host. */
+ek_status ek_layer_get_activation(ek_layer *layer, int64_t *counts);
+
+/* worker_forward (metrics.rs:46-54; observed in microseconds per request,
+ * worker/server.rs:55-63): durations of the blocking compute calls, in the
+ * reference's buckets le = 0, 4000, ..., 36000 us.  cumulative[i] counts
+ * observations <= le[i], cumulative[10] all of them (+Inf), as Prometheus does. */
+typedef struct ek_histogram {
+    double le[10];
+    int64_t cumulative[11];
+    double sum;
+    int64_t count;
+} ek_histogram;
+ek_status ek_layer_get_forward_histogram(ek_layer *layer, ek_histogram *out);
+
 /* Snapshot of the layer's counters (waits for recorded events to complete). */
 ek_status ek_layer_get_stats(ek_layer *layer, ek_stats *out);
 
