@@ -151,6 +151,7 @@ struct ek_chain {
     void *k_y = nullptr;
     int64_t k_T = -1;
     int32_t k_wdt = -1;
+    std::vector<uint8_t> k_shared;           // which layers had a shared expert when captured
     std::mutex mu;
 };
 
@@ -228,35 +229,38 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     L->w8 = cfg->w_dtype == EK_I8;
     L->Pmax = pmax;
     const int E = cfg->n_experts;
-    L->expert_mem.assign(E, nullptr);
-    L->h_slabs.assign(E, ek::ExpertSlab{nullptr, nullptr, nullptr, nullptr, nullptr});
+    // slot E of the tables is the shared expert; its segment (one row per token) follows the
+    // P routed rows in the packed buffers
+    const int64_t rows_max = pmax + cfg->max_tokens;
+    L->expert_mem.assign(E + 1, nullptr);
+    L->h_slabs.assign(E + 1, ek::ExpertSlab{nullptr, nullptr, nullptr, nullptr, nullptr});
     const int64_t nblocks = (pmax + ek::kPackChunk - 1) / ek::kPackChunk;
     ek_status st = EK_OK;
     auto A = [&](void **p, size_t bytes, const char *what) {
         if (st == EK_OK) st = dev_alloc(p, bytes, what);
     };
-    A((void **)&L->d_slabs, sizeof(ek::ExpertSlab) * E, "slab table");
+    A((void **)&L->d_slabs, sizeof(ek::ExpertSlab) * (E + 1), "slab table");
     A((void **)&L->counts, sizeof(int32_t) * E, "counts");
     A((void **)&L->offsets, sizeof(int32_t) * (E + 1), "offsets");
     A((void **)&L->perm, sizeof(int32_t) * pmax, "perm");
     A((void **)&L->inv_perm, sizeof(int32_t) * pmax, "inv_perm");
-    A((void **)&L->row_token, sizeof(int32_t) * pmax, "row_token");
+    A((void **)&L->row_token, sizeof(int32_t) * rows_max, "row_token");
     A((void **)&L->block_hist, sizeof(int32_t) * nblocks * E, "block_hist");
     A((void **)&L->err, sizeof(int32_t) * 4, "err");
     A((void **)&L->d_activation, sizeof(uint64_t) * E, "activation counters");
     L->h_activation.assign(E, 0);
     for (int i = 0; i < 10; ++i) L->forward_hist.le[i] = 4000.0 * i;   // the reference's buckets (metrics.rs:51)
-    A(&L->h, (size_t)pmax * cfg->inter * 2, "h");
-    A(&L->yp, (size_t)pmax * cfg->hidden * 2, "yp");
+    A(&L->h, (size_t)rows_max * cfg->inter * 2, "h");
+    A(&L->yp, (size_t)rows_max * cfg->hidden * 2, "yp");
     A((void **)&L->lists.count, sizeof(int32_t) * ek::kNumLists, "work list counts");
     for (int l = 0; l < ek::kNumLists; ++l) {
         // the per-expert entry point cuts one segment of up to pmax rows: capacity for E = 1 too
-        const int64_t cap = ek::list_capacity(l, pmax, E) + 1;
+        const int64_t cap = ek::list_capacity(l, rows_max, E + 1) + 1;
         L->list_cap[l] = cap;
         A((void **)&L->lists.items[l], sizeof(ek::WorkItem) * cap, "work list");
     }
     if (st == EK_OK) {
-        hipError_t e = hipMemset(L->d_slabs, 0, sizeof(ek::ExpertSlab) * E);
+        hipError_t e = hipMemset(L->d_slabs, 0, sizeof(ek::ExpertSlab) * (E + 1));
         if (e == hipSuccess) e = hipMemset(L->err, 0, sizeof(int32_t) * 4);
         if (e == hipSuccess) e = hipMemset(L->d_activation, 0, sizeof(uint64_t) * E);
         if (e == hipSuccess) e = hipMemset(L->lists.count, 0, sizeof(int32_t) * ek::kNumLists);
@@ -275,6 +279,16 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         return st;
     }
     *out = L;
+    return EK_OK;
+}
+
+// table slot of a public expert index; EK_SHARED_EXPERT names the shared expert
+ek_status expert_slot(ek_layer *L, int32_t expert, int32_t *slot)
+{
+    if (expert == EK_SHARED_EXPERT) { *slot = L->cfg.n_experts; return EK_OK; }
+    if (expert < 0 || expert >= L->cfg.n_experts)
+        return fail(EK_INVALID_INPUT, "expert %d outside [0, %d)", expert, L->cfg.n_experts);
+    *slot = expert;
     return EK_OK;
 }
 
@@ -561,13 +575,17 @@ ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const 
     }
     if (ev) EK_HIP(hipEventRecord(ev[0], s));
     ek::launch_pack(pack_args(L, ids, P, true), s);
+    // the shared expert is one more segment: every token once, rows P .. P+T-1 of the packed buffers
+    const bool shared = L->expert_mem[E] != nullptr && T > 0;
+    if (shared) ek::launch_append_segment(L->lists, E, (int32_t)P, (int32_t)T, L->row_token, s);
     if (ev) EK_HIP(hipEventRecord(ev[1], s));
     if (P > 0) {
-        EK_TRY(enqueue_ffn(L, x, L->row_token, L->yp, P, E, s, ev));
+        EK_TRY(enqueue_ffn(L, x, L->row_token, L->yp, shared ? P + T : P, shared ? E + 1 : E, s, ev));
         if (ev) EK_HIP(hipEventRecord(ev[3], s));
         ek::CombineArgs c;
         c.yp = L->yp; c.inv_perm = L->inv_perm; c.w = w; c.y = y; c.T = T; c.K = K; c.H = H;
         c.act = L->act; c.w_f32 = w_f32;
+        c.shared = shared ? (const char *)L->yp + (size_t)P * H * 2 : nullptr;
         ek::launch_combine(c, s);
     } else if (ev) {
         EK_HIP(hipEventRecord(ev[2], s));
@@ -645,8 +663,7 @@ ek_status ek_layer_set_expert(ek_layer *layer, int32_t expert, const ek_weight_d
 {
     EK_GUARDED(
         if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
-        if (expert < 0 || expert >= layer->cfg.n_experts)
-            return fail(EK_INVALID_INPUT, "expert %d outside [0, %d)", expert, layer->cfg.n_experts);
+        EK_TRY(expert_slot(layer, expert, &expert));
         DeviceGuard dg(layer->cfg.device_id);
         std::lock_guard<std::mutex> lk(layer->load_mu);
         return set_expert_locked(layer, expert, up, gate, down);
@@ -657,8 +674,7 @@ ek_status ek_layer_remove_expert(ek_layer *layer, int32_t expert)
 {
     EK_GUARDED(
         if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
-        if (expert < 0 || expert >= layer->cfg.n_experts)
-            return fail(EK_INVALID_INPUT, "expert %d outside [0, %d)", expert, layer->cfg.n_experts);
+        EK_TRY(expert_slot(layer, expert, &expert));
         DeviceGuard dg(layer->cfg.device_id);
         std::lock_guard<std::mutex> lk0(layer->load_mu);
         void *old = nullptr;
@@ -681,8 +697,7 @@ ek_status ek_layer_has_expert(ek_layer *layer, int32_t expert, int32_t *loaded)
 {
     EK_GUARDED(
         if (!layer || !loaded) return fail(EK_INVALID_INPUT, "NULL argument");
-        if (expert < 0 || expert >= layer->cfg.n_experts)
-            return fail(EK_INVALID_INPUT, "expert %d outside [0, %d)", expert, layer->cfg.n_experts);
+        EK_TRY(expert_slot(layer, expert, &expert));
         std::lock_guard<std::mutex> lk(layer->mu);
         *loaded = layer->expert_mem[expert] != nullptr;
         return EK_OK;
@@ -1125,8 +1140,13 @@ ek_status ek_chain_forward(ek_chain *chain, const void *x, const int32_t *ids, c
         if (!use_graph) {
             EK_TRY(enqueue_chain(chain, x, ids, w, w_f32, T, y, s));
         } else {
+            // a shared expert adds launches to its layer: part of the key
+            std::vector<uint8_t> shared(L);
+            for (int l = 0; l < L; ++l)
+                shared[l] = chain->layers[l]->expert_mem[chain->layers[l]->cfg.n_experts] != nullptr;
             const bool same = chain->exec && chain->k_x == x && chain->k_ids == ids && chain->k_w == w &&
-                              chain->k_y == y && chain->k_T == T && chain->k_wdt == w_dtype;
+                              chain->k_y == y && chain->k_T == T && chain->k_wdt == w_dtype &&
+                              chain->k_shared == shared;
             if (!same) {
                 if (chain->exec) { (void)hipGraphExecDestroy(chain->exec); chain->exec = nullptr; }
                 if (chain->graph) { (void)hipGraphDestroy(chain->graph); chain->graph = nullptr; }
@@ -1140,7 +1160,7 @@ ek_status ek_chain_forward(ek_chain *chain, const void *x, const int32_t *ids, c
                 chain->graph = g;
                 EK_HIP(hipGraphInstantiate(&chain->exec, g, nullptr, nullptr, 0));
                 chain->k_x = x; chain->k_ids = ids; chain->k_w = w; chain->k_y = y;
-                chain->k_T = T; chain->k_wdt = w_dtype;
+                chain->k_T = T; chain->k_wdt = w_dtype; chain->k_shared = shared;
             }
             EK_HIP(hipGraphLaunch(chain->exec, s));
         }

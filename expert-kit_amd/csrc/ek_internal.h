@@ -100,6 +100,10 @@ constexpr int kMaxExperts = 1024;
 void launch_pack(const PackArgs &a, hipStream_t s);
 // work lists for one segment [0, n) of expert e (per-expert forward)
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, hipStream_t s);
+// appends the segment (expert, rows row0 .. row0+n-1) to the lists pack has built and maps
+// its rows to tokens 0 .. n-1
+void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token,
+                           hipStream_t s);
 void launch_gather(const void *x, const int32_t *row_token, int64_t P, int64_t row_bytes, void *xp,
                    hipStream_t s);
 
@@ -136,6 +140,7 @@ struct CombineArgs {
     int64_t H;
     int32_t act;              // 0 bf16, 1 f16
     int32_t w_f32;            // gate weights are fp32 (DeepSeek shim) instead of act dtype
+    const void *shared;       // [T, H] shared-expert output added to the rounded sum, or nullptr
 };
 void launch_combine(const CombineArgs &a, hipStream_t s);
 

@@ -38,6 +38,13 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a)
     V8 o;
 #pragma unroll
     for (int i = 0; i < 8; ++i) o[i] = (T)acc[i];
+    if (a.shared) {
+        // hidden_states + shared_experts(residuals), both in the activation dtype
+        // (deepseek_v3/model.py:152)
+        const V8 sh = *(const V8 *)((const T *)a.shared + t * a.H + c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (T)((float)o[i] + (float)sh[i]);
+    }
     *(V8 *)((T *)a.y + t * a.H + c) = o;
 }
 

@@ -135,6 +135,35 @@ __global__ void single_lists_kernel(WorkLists l, int32_t e, int32_t n)
     l.count[kListStream] = c.ns;
 }
 
+__global__ __launch_bounds__(256) void append_segment_kernel(WorkLists l, int32_t e, int32_t row0, int32_t n,
+                                                             int32_t *row_token)
+{
+    const int32_t p128 = l.count[kListT128], p64 = l.count[kListT64], p32 = l.count[kListT32],
+                  ps = l.count[kListStream];
+    __syncthreads();   // every thread has read the old lengths before thread 0 replaces them
+    const SegmentCut c = cut_segment(n);
+    const int32_t full = n >> 7, r = n & 127;
+    for (int32_t t = threadIdx.x; t < full; t += 256) l.items[kListT128][p128 + t] = WorkItem{e, row0 + t * 128, 128, 0};
+    for (int32_t t = threadIdx.x; t < n; t += 256) row_token[row0 + t] = t;
+    if (threadIdx.x == 0) {
+        const WorkItem rem{e, row0 + full * 128, r, 0};
+        if (r > 64) l.items[kListT128][p128 + full] = rem;
+        else if (r > 32) l.items[kListT64][p64] = rem;
+        else if (r > 16) l.items[kListT32][p32] = rem;
+        else if (r > 0) l.items[kListStream][ps] = rem;
+        l.count[kListT128] = p128 + c.n128;
+        l.count[kListT64] = p64 + c.n64;
+        l.count[kListT32] = p32 + c.n32;
+        l.count[kListStream] = ps + c.ns;
+    }
+}
+
+void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token,
+                           hipStream_t s)
+{
+    hipLaunchKernelGGL(append_segment_kernel, dim3(1), dim3(256), 0, s, lists, expert, row0, n, row_token);
+}
+
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, hipStream_t s)
 {
     hipLaunchKernelGGL(single_lists_kernel, dim3(1), dim3(1), 0, s, lists, expert, n);

@@ -164,6 +164,10 @@ class HipLayer:
         C.check(self._lib.ek_layer_set_expert(self._h, e, ref(up), ref(gate), ref(down)))
         del k1, k2, k3
 
+    def set_shared_expert(self, weight: ExpertWeight) -> None:
+        """DeepSeek's always-on shared expert (deepseek_v3/model.py:57-61,152) as one more segment."""
+        self.set_expert(C.EK_SHARED_EXPERT, weight)
+
     def remove_expert(self, e: int) -> None:
         C.check(self._lib.ek_layer_remove_expert(self._h, e))
 

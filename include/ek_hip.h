@@ -142,6 +142,16 @@ int32_t ek_device_count(void);
 ek_status ek_layer_create(const ek_cfg *cfg, ek_layer **out);
 ek_status ek_layer_destroy(ek_layer *layer);
 
+/* Expert index that names the layer's shared expert in ek_layer_set_expert /
+ * remove_expert / has_expert / set_expert_safetensors.  DeepSeek-V3 adds
+ * shared_experts(x) to the routed result for every token
+ * (expertkit_torch/models/deepseek_v3/model.py:57-61,152); the reference runs
+ * it on the attention side.  Once loaded here it is one more segment of the
+ * grouped launch (all T tokens, gate weight 1) and ek_layer_forward returns
+ * round(routed + shared) in the activation dtype.  Its shape must be the
+ * routed experts' (moe_intermediate_size * n_shared_experts == cfg.inter). */
+#define EK_SHARED_EXPERT (-1)
+
 /* ExpertDB::insert after ExpertBackend::build (ffn/mod.rs:23-36;
  * worker/x.rs:13-34): copies the three matrices to HBM in the kernels' tiled
  * layout, casting to cfg.w_dtype.  Shapes must be up,gate [I,H], down [H,I].

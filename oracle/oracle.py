@@ -232,6 +232,16 @@ def layer_forward(x, ids, w, w_up, w_gate, w_down, mode: int = 0, return_y3: boo
     return (y, counts, offsets, perm, inv, y3) if return_y3 else (y, counts, offsets, perm, inv)
 
 
+def add_shared(y_routed: torch.Tensor, x: torch.Tensor, w_up, w_gate, w_down, rounded: bool = True):
+    """hidden_states + shared_experts(residuals) (deepseek_v3/model.py:57-61,152): the routed result
+    and the shared MLP's output are both tensors of the activation dtype; their sum is formed in
+    fp32 and (rounded=True) stored in the activation dtype."""
+    assert y_routed.dtype == x.dtype
+    y_shared = ffn(x, w_up, w_gate, w_down, mode=0)
+    total = y_routed.float() + y_shared.float()
+    return total.to(x.dtype) if rounded else total
+
+
 def layer_loop_form(x, ids, w, w_up, w_gate, w_down):
     """Whole layer, stock per-expert loop + index_add_ (qwen3_moe.py:115-151)."""
     x = x.contiguous()

@@ -1,0 +1,119 @@
+"""DeepSeek's shared expert as an always-on segment of the grouped launch.
+
+Bars: (1) composition, bit-exact: the fused result equals round(y_routed + y_shared) where
+y_routed is the same layer's result without the shared expert and y_shared the same weights'
+output through the per-expert entry point (same kernels, same cut of the T rows);
+(2) against the oracle: 2e-2 * rms of the reference plus the storage quanta of the two
+16-bit summands and of the result.
+"""
+import pytest
+import torch
+
+from ek_hip import _capi as C
+from ek_hip import workloads as wl
+from test_gpu_parity import TOL, oracle_weights, ulp_of
+
+pytestmark = pytest.mark.gpu
+
+H, I, E, K = 256, 192, 8, 2
+
+
+def build(ek, dt, w8, max_tokens=512):
+    work = wl.Workload("shared", H, I, E + 1, K, 1, dt, w8=w8)
+    ws = {e: wl.make_expert(work, e, std=0.05) for e in range(E + 1)}      # index E: the shared one
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=torch.int8 if w8 else dt, max_tokens=max_tokens)
+    for e in range(E):
+        layer.set_expert(e, ws[e])
+    return layer, ws
+
+
+def routing(T, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, H, generator=g)
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32).reshape(T, K)
+    w = torch.rand(T, K, generator=g) + 0.1
+    return x, ids, w / w.sum(-1, keepdim=True)
+
+
+@pytest.mark.parametrize("dt,w8", [(torch.bfloat16, False), (torch.float16, False), (torch.bfloat16, True)])
+def test_shared_expert_segment(ek, oracle, cuda, dt, w8):
+    layer, ws = build(ek, dt, w8)
+    single = ek.HipLayer(H, I, 1, 1, act_dtype=dt, w_dtype=torch.int8 if w8 else dt, max_tokens=512)
+    single.set_expert(0, ws[E])
+    wu, wg, wd = oracle_weights(oracle, ws, E + 1, dt)
+    for T in (1, 16, 17, 33, 100, 130, 300):
+        x, ids, w = routing(T, 40 + T)
+        x, w = x.to(dt), w.to(dt)
+        assert not layer.has_expert(C.EK_SHARED_EXPERT)
+        y_plain = layer.forward(x.to(cuda), ids.to(cuda), w.to(cuda))
+        layer.set_shared_expert(ws[E])
+        assert layer.has_expert(C.EK_SHARED_EXPERT)
+        y = layer.forward(x.to(cuda), ids.to(cuda), w.to(cuda))
+        # (1) composition
+        y_sh = single.expert_forward(0, x.to(cuda))
+        want = (y_plain.float() + y_sh.float()).to(dt)
+        assert torch.equal(y.view(torch.int16), want.view(torch.int16)), T
+        assert not torch.equal(y, y_plain)
+        # host-memory call takes the same path
+        assert torch.equal(layer.forward(x, ids, w).view(torch.int16), y.cpu().view(torch.int16))
+        # (2) oracle
+        y_r = oracle.layer_forward(x, ids, w, wu[:E], wg[:E], wd[:E], mode=0)[0]
+        ref32 = oracle.add_shared(y_r, x, wu[E], wg[E], wd[E], rounded=False)
+        y_s = ref32 - y_r.float()
+        rms = float(ref32.pow(2).mean().sqrt())
+        err = (y.float().cpu() - ref32).abs()
+        quanta = 0.5 * ulp_of(ref32, dt) * 1.0001 + ulp_of(y_r.float(), dt) + ulp_of(y_s, dt)
+        worst = float(err.max()) / rms
+        over = float((err > TOL * rms).float().mean())
+        print(f"shared {dt} w8={w8} T={T}: max|err|/rms = {worst:.3e}, elements over 2e-2*rms: {over:.2e}", flush=True)
+        assert bool((err <= TOL * rms + quanta).all()), worst
+        assert over <= 1e-4 or T * H * over <= 2      # tiny outputs: allow two elements
+        layer.remove_expert(C.EK_SHARED_EXPERT)
+        again = layer.forward(x.to(cuda), ids.to(cuda), w.to(cuda))
+        assert torch.equal(again.view(torch.int16), y_plain.view(torch.int16))
+    assert layer.activation().shape == (E,)                    # the shared expert is not a routed expert
+    with pytest.raises(ek.EKError) as ei:
+        layer.remove_expert(C.EK_SHARED_EXPERT)
+    assert ei.value.status == C.EK_EXPERT_NOT_FOUND
+    layer.close()
+    single.close()
+
+
+def test_shared_expert_in_a_chain(ek, cuda):
+    dt, L, T = torch.float16, 3, 90
+    layers = []
+    for l in range(L):
+        work = wl.Workload("shared-chain", H, I, E + 1, K, 1, dt)
+        layer = ek.HipLayer(H, I, E, K, act_dtype=dt, max_tokens=128)
+        for e in range(E):
+            layer.set_expert(e, wl.make_expert(work, e, layer=l, std=0.08))
+        if l != 1:                                              # layers 0 and 2 have one, layer 1 does not
+            layer.set_shared_expert(wl.make_expert(work, E, layer=l, std=0.08))
+        layers.append(layer)
+    x, _, _ = routing(T, 7)
+    x = x.to(dt).to(cuda)
+    ids = torch.stack([routing(T, 100 + l)[1] for l in range(L)]).to(cuda)
+    w = torch.stack([routing(T, 100 + l)[2] for l in range(L)]).to(dt).to(cuda)
+    step = x
+    for l in range(L):
+        step = layers[l].forward(step, ids[l], w[l])
+    chain = ek.HipChain(layers)
+    eager = chain.forward(x, ids, w, use_graph=False)
+    assert torch.equal(eager.view(torch.int16), step.view(torch.int16))
+    for rep in range(3):
+        got = chain.forward(x, ids, w, use_graph=True)
+        assert torch.equal(got.view(torch.int16), step.view(torch.int16)), rep
+        torch.cuda.synchronize()
+    # loading a shared expert into layer 1 changes the launches: the graph must be captured again
+    work = wl.Workload("shared-chain", H, I, E + 1, K, 1, dt)
+    layers[1].set_shared_expert(wl.make_expert(work, E, layer=1, std=0.08))
+    step2 = x
+    for l in range(L):
+        step2 = layers[l].forward(step2, ids[l], w[l])
+    assert not torch.equal(step2, step)
+    for rep in range(2):
+        got = chain.forward(x, ids, w, use_graph=True)
+        assert torch.equal(got.view(torch.int16), step2.view(torch.int16)), rep
+    chain.close()
+    for layer in layers:
+        layer.close()
