@@ -46,6 +46,19 @@ template <int N> __device__ __forceinline__ void wait_vmcnt()
 {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
+// s_waitcnt vmcnt(n) for a wave-uniform run-time n: the count is an immediate, so this is a
+// jump over the possible values.  n beyond 24 waits for 24 (stricter, hence safe).
+__device__ __forceinline__ void wait_vmcnt_dyn(int n)
+{
+    switch (n) {
+#define EK_CASE(k) case k: wait_vmcnt<k>(); break;
+        EK_CASE(0) EK_CASE(1) EK_CASE(2) EK_CASE(3) EK_CASE(4) EK_CASE(5) EK_CASE(6) EK_CASE(7)
+        EK_CASE(8) EK_CASE(9) EK_CASE(10) EK_CASE(11) EK_CASE(12) EK_CASE(13) EK_CASE(14) EK_CASE(15)
+        EK_CASE(16) EK_CASE(17) EK_CASE(18) EK_CASE(19) EK_CASE(20) EK_CASE(21) EK_CASE(22) EK_CASE(23)
+#undef EK_CASE
+    default: wait_vmcnt<24>(); break;
+    }
+}
 __device__ __forceinline__ void block_barrier()
 {
     asm volatile("s_barrier" : : : "memory");
@@ -205,10 +218,15 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     EK_ISSUE(cur, 0, 0);
     EK_ISSUE(cur, 1, 1);
 
+    // The next tile's addresses are needed two steps before this one ends.  Fetching them
+    // makes the wave wait on ordinary loads, i.e. on every vector-memory operation issued
+    // before them: it is done three steps before the end, right after the barrier and before
+    // the step's DMAs are issued, when only the next step's DMAs (a step old) are in flight.
+    const int fstep = nsteps > 3 ? nsteps - 3 : 0;
+    int pend_st = 0;   // global stores of the previous tile's epilogue, issued after the DMAs of
+                       // this tile's first two steps (stores count in vmcnt like loads)
     while (true) {
-        // the next tile's addresses are needed two steps before this one ends; fetching
-        // them here costs one drain of the (two-stage deep) DMA queue per tile
-        const int tn = fetch(tc + stride, nxt);
+        int tn = -1;
 
         f32x16 acc[RB][CB];
 #pragma unroll
@@ -220,11 +238,16 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 
         for (int step = 0; step < nsteps; ++step) {
             // the DMAs of this step are older than those of the next one (of this tile or of
-            // the next tile): wait until only the latter remain
-            if (step + 1 < nsteps || tn >= 0) wait_vmcnt<LOADS>();
-            else wait_vmcnt<0>();
+            // the next tile) and than the previous epilogue's stores: wait until only those remain
+            if (step + 1 < nsteps || tn >= 0) {
+                if (step < 2 && pend_st) wait_vmcnt_dyn(LOADS + pend_st);
+                else wait_vmcnt<LOADS>();
+            } else {
+                wait_vmcnt<0>();
+            }
             block_barrier();   // this step's tile is visible to all waves; the stage of the
                                // previous step is free again
+            if (step == fstep) tn = fetch(tc + stride, nxt);
             const int ring2 = ring == 0 ? 2 : ring - 1;          // (ring + 2) % 3
             if (step + 2 < nsteps) {
                 EK_ISSUE(cur, step + 2, ring2);
@@ -293,36 +316,55 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             ring = ring == 2 ? 0 : ring + 1;
         }
 
-        // ---- epilogue: lane holds, for row rb*32 + l%32, channels q*8 + kg*4 + (0..3), q = 0..3,
-        //      of each column block ----
+        // ---- epilogue.  A lane holds, for row rb*32 + l%32, channels q*8 + kg*4 + (0..3),
+        //      q = 0..3, of each column block: written as they are, a store instruction would
+        //      touch 32 rows with 16 bytes each.  The rounded values go through LDS instead
+        //      (the stage of the last step, once every wave has left it), wave-private, one
+        //      32-row block at a time, and leave as whole rows: 16 bytes per lane, a row of the
+        //      wave's OUTC channels per 2*OUTC/16 lanes.
         typedef T T4 __attribute__((ext_vector_type(4)));
+        constexpr int OUTC = NMAT == 2 ? 32 : 64;          // output channels per wave
+        constexpr int RS = OUTC * 2 + 16;                  // scratch row stride: 16 bytes of padding
+        constexpr int PPO = OUTC * 2 / 16, RPI = 64 / PPO; // pieces per row, rows per store instruction
+        static_assert(kTileWaves * 32 * RS <= G::STAGE, "epilogue scratch fits one stage");
+        block_barrier();
+        pend_st = 0;
+        if (cur.chan0 < a.N) {
+            uint8_t *scr = lds + (ring == 0 ? 2 : ring - 1) * G::STAGE + wave * (32 * RS);
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            const int r_in = rb * 32 + l32;
-            if (r_in >= cur.nrows) continue;
-            T *orow = (T *)a.out + (int64_t)(cur.row0 + r_in) * a.out_stride;
-            if constexpr (NMAT == 2) {
-                if (cur.chan0 >= a.N) continue;
+            for (int rb = 0; rb < RB; ++rb) {
+                if (rb * 32 >= cur.nrows) break;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    T4 o;
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) o[r] = swiglu_rounded<T>(acc[rb][0][q * 4 + r], acc[rb][1][q * 4 + r]);
-                    *(uint2 *)(orow + cur.chan0 + q * 8 + kg * 4) = __builtin_bit_cast(uint2, o);
-                }
-            } else {
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    const int cbase = cur.chan0 + cb * 32;
-                    if (cbase >= a.N) continue;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
+                    if constexpr (NMAT == 2) {
                         T4 o;
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) o[r] = (T)acc[rb][cb][q * 4 + r];
-                        *(uint2 *)(orow + cbase + q * 8 + kg * 4) = __builtin_bit_cast(uint2, o);
+                        for (int r = 0; r < 4; ++r) o[r] = swiglu_rounded<T>(acc[rb][0][q * 4 + r], acc[rb][1][q * 4 + r]);
+                        *(uint2 *)(scr + l32 * RS + (q * 8 + kg * 4) * 2) = __builtin_bit_cast(uint2, o);
+                    } else {
+#pragma unroll
+                        for (int cb = 0; cb < CB; ++cb) {
+                            T4 o;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) o[r] = (T)acc[rb][cb][q * 4 + r];
+                            *(uint2 *)(scr + l32 * RS + (cb * 32 + q * 8 + kg * 4) * 2) = __builtin_bit_cast(uint2, o);
+                        }
                     }
                 }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int i = 0; i < 32 / RPI; ++i) {
+                    if (rb * 32 + i * RPI >= cur.nrows) break;    // wave-uniform: the count below is exact
+                    const int r_in = rb * 32 + i * RPI + lane / PPO;
+                    const u32x4 v = *(const u32x4 *)(scr + (i * RPI + lane / PPO) * RS + (lane % PPO) * 16);
+                    if (r_in < cur.nrows)
+                        *(u32x4 *)((T *)a.out + (int64_t)(cur.row0 + r_in) * a.out_stride + cur.chan0 + (lane % PPO) * 8) = v;
+                    pend_st += 1;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
             }
         }
         if (tn < 0) break;
