@@ -93,3 +93,42 @@ def test_weight_lookup_suffixes(ek):
         with pytest.raises(ek.EKError) as ei:
             ek.ExpertWeight.from_safetensor(d)
         assert ei.value.status == 3 and text in ei.value.message
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 on its own, and a C program linked
+    against the library must be able to call it (no GPU needed for these entry points)."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    from ek_hip import _capi as C
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include "ek_hip.h"
+#include <stdio.h>
+#include <string.h>
+int main(void) {
+    int32_t layer = -1, expert = -1;
+    char id[64];
+    ek_cfg cfg; ek_weight_desc d; ek_route_out ro; ek_stats st; ek_router_cfg rc; ek_histogram h; ek_tensor_view tv;
+    (void)cfg; (void)d; (void)ro; (void)st; (void)rc; (void)h; (void)tv;
+    if (strcmp(ek_backend_name(), "hip") != 0) return 1;
+    if (ek_expert_id_format("ds-tiny", 3, 17, id, sizeof id) != EK_OK) return 2;
+    if (ek_expert_id_parse(id, &layer, &expert) != EK_OK || layer != 3 || expert != 17) return 3;
+    if (ek_expert_id_parse("nonsense", &layer, &expert) != EK_INVALID_INPUT) return 4;
+    if (strlen(ek_last_error()) == 0) return 5;
+    if (ek_layer_forward(NULL, NULL, NULL, NULL, EK_BF16, 0, NULL, NULL, EK_HOST, NULL) != EK_INVALID_INPUT) return 6;
+    printf("%s %s\n", ek_backend_name(), id);
+    return 0;
+}
+''')
+    inc = os.path.join(ROOT, "include")
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", "-I", inc, str(src)])
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(C.LIB_PATH)
+    subprocess.check_call(["gcc", "-std=c99", "-I", inc, str(src), "-o", str(exe), "-L", libdir, "-lek_hip",
+                           "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"])
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, (out.returncode, out.stdout, out.stderr)
+    assert out.stdout.strip() == "hip ds-tiny/l3-e17"
