@@ -113,7 +113,7 @@ def bench_chain(args, w, dev):
         "metric": "token-expert pairs/s on 1 MI355X (DSv3 W8A16 layer); % HBM / MFMA roofline",
         "value": pairs / step_s, "unit": "pairs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": step_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": str(w.act_dtype).replace("torch.", "") + ", fp32 accumulate", "data": "synthetic",
+        "dtype": {"bfloat16": "bf16", "float16": "f16"}[str(w.act_dtype).replace("torch.", "")], "data": "synthetic",
         "config": {"workload": w.name, "hidden": w.hidden, "moe_intermediate": w.inter, "experts": w.n_experts,
                    "top_k": w.top_k, "tokens": w.tokens, "pairs_per_layer": w.pairs, "layers": w.n_layers,
                    "requests": len(wl.request_lengths()), "zipf_s": w.zipf_s, "launch": "one hipGraph per chain"},
@@ -234,11 +234,12 @@ def main():
         "metric": "token-expert pairs/s on 1 MI355X (DSv3 W8A16 layer); % HBM / MFMA roofline",
         "value": value, "unit": "pairs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": step_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": ("i8 weights x " if w.w8 else "") + str(w.act_dtype).replace("torch.", "") + ", fp32 accumulate",
+        # the type the MFMAs multiply in (int8 weights are dequantised to it in registers); fp32 accumulation
+        "dtype": {"bfloat16": "bf16", "float16": "f16"}[str(w.act_dtype).replace("torch.", "")],
         "data": "synthetic",
         "config": {"workload": w.name, "hidden": w.hidden, "moe_intermediate": w.inter, "experts": w.n_experts,
                    "top_k": w.top_k, "tokens": w.tokens, "pairs": w.pairs, "active_experts": active,
-                   "zipf_s": w.zipf_s},
+                   "zipf_s": w.zipf_s, "weights": "int8 per-channel" if w.w8 else "16-bit"},
         "roofline": roof,
         "layer": {"algorithmic_bytes": b_layer, "algorithmic_flops": f_layer, "hbm_frac": hbm_frac,
                   "mfma_frac": mfma_frac,
