@@ -143,3 +143,47 @@ def test_emit_rejects_small_buffer_and_bad_description():
     out = ctypes.create_string_buffer(need)
     assert lib.ek_safetensors_emit(b"data", C.EK_BF16, 2, shape, src, out, need - 1, None) == C.EK_INVALID_INPUT
     assert lib.ek_safetensors_emit(b"data", C.EK_BF16, 2, shape, src, out, need, None) == C.EK_OK
+
+
+def test_parser_survives_mutated_blobs():
+    """Blobs arrive over the wire: whatever the bytes, the parser answers with a status and a view
+    that lies inside the blob (a crash would take the test process down)."""
+    lib = C.load()
+    rng = np.random.default_rng(20240607)
+    good = [st_save({"data": _rand((5, 64), torch.bfloat16, 3)}),
+            st_save({"a.w1.weight": _rand((8, 8), torch.float32, 4), "data": _rand((3, 16), torch.int8, 5)},
+                    metadata={"k": "v"})]
+    ok = bad = 0
+    for it in range(6000):
+        blob = bytearray(good[it % 2])
+        kind = it % 6
+        if kind == 0:                                   # truncate anywhere
+            del blob[int(rng.integers(0, len(blob))):]
+        elif kind == 1:                                 # flip bytes in the header
+            hl = struct.unpack("<Q", bytes(blob[:8]))[0]
+            for _ in range(int(rng.integers(1, 6))):
+                blob[8 + int(rng.integers(0, hl))] = int(rng.integers(0, 256))
+        elif kind == 2:                                 # corrupt the length prefix
+            blob[:8] = struct.pack("<Q", int(rng.integers(0, 1 << 62)))
+        elif kind == 3:                                 # splice digits into numbers
+            hl = struct.unpack("<Q", bytes(blob[:8]))[0]
+            pos = 8 + int(rng.integers(0, hl))
+            blob[pos:pos] = b"9" * int(rng.integers(1, 30))
+        elif kind == 4:                                 # random garbage of the same length
+            blob = bytearray(rng.integers(0, 256, len(blob), dtype=np.uint8).tobytes())
+        else:                                           # drop a slice of the header
+            hl = struct.unpack("<Q", bytes(blob[:8]))[0]
+            a = 8 + int(rng.integers(0, hl))
+            del blob[a:a + int(rng.integers(1, 12))]
+        buf = (ctypes.c_char * max(len(blob), 1)).from_buffer(blob if len(blob) else bytearray(1))
+        view = C.ek_tensor_view()
+        st = lib.ek_safetensors_find(buf, len(blob), b"data", ctypes.byref(view))
+        assert st in (C.EK_OK, C.EK_INVALID_INPUT, C.EK_WEIGHT_NOT_FOUND)
+        if st == C.EK_OK:
+            ok += 1
+            base = ctypes.addressof(buf)
+            assert base <= view.data and view.data + view.nbytes <= base + len(blob)
+            assert 0 <= view.rank <= 4 and view.nbytes >= 0
+        else:
+            bad += 1
+    assert bad > 3000 and ok > 0
