@@ -2,6 +2,7 @@
 #include "../../include/ek_hip.h"
 #include "ek_internal.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
@@ -255,7 +256,9 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     A((void **)&L->lists.count, sizeof(int32_t) * ek::kNumLists, "work list counts");
     for (int l = 0; l < ek::kNumLists; ++l) {
         // the per-expert entry point cuts one segment of up to pmax rows: capacity for E = 1 too
-        const int64_t cap = ek::list_capacity(l, rows_max, E + 1) + 1;
+        // (and the wide cut, see wide_cut_pays: fewer than 128 tile items of at most 128 rows
+        // become at most two streaming items each)
+        const int64_t cap = ek::list_capacity(l, rows_max, E + 1) + (l == ek::kListStream ? 264 : 1);
         L->list_cap[l] = cap;
         A((void **)&L->lists.items[l], sizeof(ek::WorkItem) * cap, "work list");
     }
@@ -515,8 +518,11 @@ ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_lo
 // Both FFN stages over the work lists in L->lists: x [*, H] (rows picked through
 // `rows`, or packed order when nullptr) -> L->h -> out [P, H].  P and E bound the
 // list lengths (grid sizes); ev, if set, receives the stage boundary event.
+// wide_items > 0: the lists hold that many weight-streaming items of up to kWideRows rows and
+// nothing else (the per-expert entry points' cut for calls that would leave the tile kernel
+// most of the chip idle).
 ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out, int64_t P, int64_t E,
-                      hipStream_t s, hipEvent_t *ev)
+                      hipStream_t s, hipEvent_t *ev, int64_t wide_items = 0)
 {
     const int64_t H = L->cfg.hidden, I = L->cfg.inter;
     ek::FfnArgs a1;
@@ -530,6 +536,12 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
         cap[l] = ek::list_capacity(l, P, E);
         if (cap[l] > L->list_cap[l]) cap[l] = L->list_cap[l];
         if (cap[l] < 0) cap[l] = 0;
+    }
+    if (wide_items > 0) {
+        EK_HIP(ek::launch_ffn_stream(a1, 1, L->act, L->w8, wide_items, true, s));
+        if (ev) EK_HIP(hipEventRecord(ev[2], s));
+        EK_HIP(ek::launch_ffn_stream(a2, 2, L->act, L->w8, wide_items, true, s));
+        return EK_OK;
     }
     // Two independent chains: the weight-streaming kernel (items of <= 16 rows) and the
     // MFMA tile kernel (longer items) touch disjoint rows of h and out.  In the middle
@@ -550,7 +562,7 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
     }
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
-        if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->w8, cap[ek::kListStream], s_stream));
+        if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->w8, cap[ek::kListStream], false, s_stream));
         if (have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->w8, cap, s_tiles));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
     }
@@ -833,8 +845,12 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
                 d_x = layer->st_x;
                 d_out = layer->st_y;
             }
-            ek::launch_single_lists(layer->lists, expert, (int32_t)n, s);
-            EK_TRY(enqueue_ffn(layer, d_x, nullptr, d_out, n, 1, s, nullptr));
+            // the ordinary cut's tile items: full 128-row tiles and a remainder of more than 16 rows
+            const int64_t wide_items = (n + ek::kWideRows - 1) / ek::kWideRows;
+            const bool wide = ek::wide_cut_pays((n >> 7) + ((n & 127) > 16), layer->cfg.inter) &&
+                              wide_items <= layer->list_cap[ek::kListStream];
+            ek::launch_single_lists(layer->lists, expert, (int32_t)n, wide, s);
+            EK_TRY(enqueue_ffn(layer, d_x, nullptr, d_out, n, 1, s, nullptr, wide ? wide_items : 0));
             if (mem == EK_HOST)
                 EK_HIP(hipMemcpyAsync(out, layer->st_y, (size_t)n * H * 2, hipMemcpyDeviceToHost, s));
         }
@@ -897,9 +913,22 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             // Work lists cut on the host exactly as the pack kernels cut them: a call is one
             // segment (ek_internal.h, "work lists").
             std::vector<ek::WorkItem> items[ek::kNumLists];
-            int64_t row0 = 0;
+            int64_t row0 = 0, tile_items = 0, wide_items = 0;
+            for (int i = 0; i < n_calls; ++i) {
+                tile_items += (rows[i] >> 7) + ((rows[i] & 127) > 16);
+                wide_items += (rows[i] + ek::kWideRows - 1) / ek::kWideRows;
+            }
+            const bool wide = ek::wide_cut_pays(tile_items, layer->cfg.inter) &&
+                              wide_items <= layer->list_cap[ek::kListStream];
             for (int i = 0; i < n_calls; ++i) {
                 const int32_t n = (int32_t)rows[i], full = n >> 7, r = n & 127;
+                if (wide) {
+                    for (int32_t r0 = 0; r0 < n; r0 += ek::kWideRows)
+                        items[ek::kListStream].push_back(
+                            ek::WorkItem{experts[i], (int32_t)row0 + r0, std::min<int32_t>(ek::kWideRows, n - r0), 0});
+                    row0 += n;
+                    continue;
+                }
                 for (int32_t t = 0; t < full; ++t)
                     items[ek::kListT128].push_back(ek::WorkItem{experts[i], (int32_t)row0 + t * 128, 128, 0});
                 const ek::WorkItem rem{experts[i], (int32_t)row0 + full * 128, r, 0};
@@ -943,7 +972,7 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
                     EK_HIP(hipMemcpyAsync((char *)layer->st_x + row0 * H * 2, xs[i], (size_t)rows[i] * H * 2, in_kind, s));
                 row0 += rows[i];
             }
-            EK_TRY(enqueue_ffn(layer, layer->st_x, nullptr, layer->st_y, P, n_calls, s, nullptr));
+            EK_TRY(enqueue_ffn(layer, layer->st_x, nullptr, layer->st_y, P, n_calls, s, nullptr, wide ? wide_items : 0));
             EK_HIP(hipGetLastError());
             row0 = 0;
             for (int i = 0; i < n_calls; ++i) {
@@ -1131,8 +1160,13 @@ ek_status ek_chain_forward(ek_chain *chain, const void *x, const int32_t *ids, c
         DeviceGuard dg(l0->cfg.device_id);
         if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", l0->cfg.device_id);
         std::lock_guard<std::mutex> ck(chain->mu);
+        // every layer's workspace is ours for the call; locked in address order so that chains
+        // that share layers cannot deadlock each other
+        std::vector<ek_layer *> order(chain->layers);
+        std::sort(order.begin(), order.end());
+        order.erase(std::unique(order.begin(), order.end()), order.end());
         std::vector<std::unique_lock<std::mutex>> locks;
-        for (ek_layer *ly : chain->layers) locks.emplace_back(ly->mu);
+        for (ek_layer *ly : order) locks.emplace_back(ly->mu);
         hipStream_t s = stream ? (hipStream_t)stream : chain->stream;
         const int w_f32 = w_dtype == EK_F32;
         const int L = (int)chain->layers.size();

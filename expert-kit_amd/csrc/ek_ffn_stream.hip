@@ -1,4 +1,5 @@
-// Ragged grouped SwiGLU FFN, weight-streaming kernel (work items of <= 16 rows).
+// Ragged grouped SwiGLU FFN, weight-streaming kernel (work items of <= 16 rows; <= 64 rows
+// in launches the host has cut wide).
 //
 // Computes, per expert segment, the four ops of TorchFFN's closure
 // (ek-computation/src/ffn/expert_torch.rs:81-84):
@@ -23,14 +24,32 @@
 // fma(u, s, -128 s) per element gives the exact fp32 product q*s (16
 // significant bits), and v_cvt_pk_bf16_f32 rounds two of them to nearest even.
 // Each lane owns one output channel of the A operand, so s is a lane scalar.
+//
+// Accumulation order (the same bits whichever way a launch is shaped): the contraction is
+// cut into kSlices slices of whole chunks, [KT*w/8, KT*(w+1)/8); a slice is summed by the
+// MFMAs in k order into a zeroed accumulator and the slice sums are added in slice order.
+// SK = 1: one wave walks all slices.  SK = 8: eight waves of one workgroup take one slice
+// each and the first adds their sums, through LDS, in the same order -- used when a launch
+// has too few (item, channel tile) pairs to keep the chip's memory system busy (a lone
+// expert, a tiny layer), where eight times the waves mean eight times the loads in flight.
+//
+// RS = 4 (always with SK = 8): items of up to 64 rows, four 16-row B operands per weight
+// chunk.  A lone expert with a few dozen to a few hundred rows would give the tile kernel a
+// handful of workgroups; here its weights are still streamed (and dequantised) once per 64
+// rows by a full grid.  Each 16-row fragment sees the MFMA sequence it would see as an item
+// of its own, so a row's result does not depend on RS either.
 #include "ek_internal.h"
 #include "ek_mfma.h"
 
 namespace ek {
 
-template <typename T, bool W8, int NMAT, int NG, int D>
-__global__ __launch_bounds__(256) void ffn_stream_kernel(FfnArgs a)
+constexpr int kSlices = 8;
+
+template <typename T, bool W8, int NMAT, int NG, int D, int SK, int RS>
+__global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kernel(FfnArgs a)
 {
+    static_assert(SK == 1 || SK == kSlices, "one wave per launch shape or one wave per slice");
+    static_assert(RS == 1 || SK == kSlices, "wide items only in the sliced form");
     using V8 = typename Act<T>::V8;
     constexpr int KE = W8 ? 64 : 32;   // contraction elements per chunk
     constexpr int XV = W8 ? 2 : 1;     // 16-byte activation loads per chunk per lane
@@ -41,8 +60,8 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(FfnArgs a)
     const WorkItem item = a.lists.items[kListStream][blockIdx.y];
     const int e = item.expert, seg0 = item.row0, n = item.nrows;
     const int NT = a.N >> 4;
-    const int nt0 = (blockIdx.x * 4 + wave) * NG;
-    if (nt0 >= NT) return;
+    const int nt0 = SK == 1 ? (blockIdx.x * 4 + wave) * NG : blockIdx.x * NG;
+    if (nt0 >= NT) return;             // SK = 8: the same for every wave of the workgroup
     const ExpertSlab slab = a.slabs[e];
     const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
     if (wmat == nullptr) return;   // expert not loaded: pack has flagged the call
@@ -69,90 +88,139 @@ __global__ __launch_bounds__(256) void ffn_stream_kernel(FfnArgs a)
             wc[gi * NMAT + m] = -128.f * sv;
         }
 
-    {
-        constexpr int r0 = 0;   // items hold at most 16 rows
-        const int jr = min(r0 + j, n - 1);   // lanes past the segment re-read its last row
+    const int nfr = RS == 1 ? 1 : (n + 15) >> 4;   // 16-row fragments that hold rows
+    const T *xp[RS];
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs) {
+        const int jr = min(rs * 16 + j, n - 1);   // lanes past the segment re-read its last row
         const int64_t row = a.rows ? (int64_t)a.rows[seg0 + jr] : (int64_t)(seg0 + jr);
-        const T *xp = (const T *)a.x + row * a.x_stride + g * (KE / 4);
+        xp[rs] = (const T *)a.x + row * a.x_stride + g * (KE / 4);
+    }
 
-        f32x4 acc[NMAT][NG];
+    f32x4 acc[RS][NMAT][NG], tot[RS][NMAT][NG];
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs)
 #pragma unroll
         for (int m = 0; m < NMAT; ++m)
 #pragma unroll
-            for (int gi = 0; gi < NG; ++gi) acc[m][gi] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int gi = 0; gi < NG; ++gi) {
+                acc[rs][m][gi] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                tot[rs][m][gi] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            }
+    // this wave's chunks and, for SK = 1, the end of the slice it is in
+    const int kbeg = SK == 1 ? 0 : KT * wave / kSlices, kend = SK == 1 ? KT : KT * (wave + 1) / kSlices;
+    int sl = 0, kb = KT / kSlices;
+    if constexpr (SK == 1) {
+        while (kb == 0) { ++sl; kb = KT * (sl + 1) / kSlices; }   // empty leading slices (KT < 8)
+    }
 
-        uint4 wq[D][NW];
-        uint4 xq[D][XV];
+    uint4 wq[D][NW];
+    uint4 xq[D][RS][XV];
+    auto fetch = [&](int d, int kt) {
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m)
+                wq[d][gi * NMAT + m] = ldg16(wp[gi] + (int64_t)(kt * NMAT + m) * kChunkBytes);
+#pragma unroll
+        for (int rs = 0; rs < RS; ++rs)
+            if (RS == 1 || rs < nfr) {
+#pragma unroll
+                for (int v = 0; v < XV; ++v) xq[d][rs][v] = ldg16(xp[rs] + (int64_t)kt * KE + v * 8);
+            }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        if (SK == 1 || kbeg + d < kend) fetch(d, kbeg + d);
+
+    for (int kt0 = kbeg; kt0 < kend; kt0 += D) {
 #pragma unroll
         for (int d = 0; d < D; ++d) {
+            const int kt = kt0 + d;
+            if (SK != 1 && kt >= kend) break;      // SK = 1: KT is a multiple of D
+            // consume slot d
 #pragma unroll
             for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
-                for (int m = 0; m < NMAT; ++m)
-                    wq[d][gi * NMAT + m] = ldg16(wp[gi] + (int64_t)(d * NMAT + m) * kChunkBytes);
+                for (int m = 0; m < NMAT; ++m) {
+                    const uint4 q = wq[d][gi * NMAT + m];
+                    if constexpr (W8) {
+                        const float sv = ws[gi * NMAT + m], cv = wc[gi * NMAT + m];
+                        const V8 w0 = dequant_u8x8<T>(q.x, q.y, sv, cv), w1 = dequant_u8x8<T>(q.z, q.w, sv, cv);
 #pragma unroll
-            for (int v = 0; v < XV; ++v) xq[d][v] = ldg16(xp + d * KE + v * 8);
-        }
-
-        for (int kt0 = 0; kt0 < KT; kt0 += D) {
-#pragma unroll
-            for (int d = 0; d < D; ++d) {
-                const int kt = kt0 + d;
-                // consume slot d
-                if constexpr (W8) {
-                    const V8 x0 = __builtin_bit_cast(V8, xq[d][0]);
-                    const V8 x1 = __builtin_bit_cast(V8, xq[d][1]);
-#pragma unroll
-                    for (int gi = 0; gi < NG; ++gi)
-#pragma unroll
-                        for (int m = 0; m < NMAT; ++m) {
-                            const uint4 q = wq[d][gi * NMAT + m];
-                            const float sv = ws[gi * NMAT + m], cv = wc[gi * NMAT + m];
-                            acc[m][gi] = Act<T>::mfma(dequant_u8x8<T>(q.x, q.y, sv, cv), x0, acc[m][gi]);
-                            acc[m][gi] = Act<T>::mfma(dequant_u8x8<T>(q.z, q.w, sv, cv), x1, acc[m][gi]);
-                        }
-                } else {
-                    const V8 x0 = __builtin_bit_cast(V8, xq[d][0]);
-#pragma unroll
-                    for (int gi = 0; gi < NG; ++gi)
-#pragma unroll
-                        for (int m = 0; m < NMAT; ++m)
-                            acc[m][gi] = Act<T>::mfma(__builtin_bit_cast(V8, wq[d][gi * NMAT + m]),
-                                                      x0, acc[m][gi]);
-                }
-                // refill slot d with chunk kt + D
-                if (kt + D < KT) {
-#pragma unroll
-                    for (int gi = 0; gi < NG; ++gi)
-#pragma unroll
-                        for (int m = 0; m < NMAT; ++m)
-                            wq[d][gi * NMAT + m] =
-                                ldg16(wp[gi] + (int64_t)((kt + D) * NMAT + m) * kChunkBytes);
-#pragma unroll
-                    for (int v = 0; v < XV; ++v)
-                        xq[d][v] = ldg16(xp + (int64_t)(kt + D) * KE + v * 8);
-                }
-            }
-        }
-
-        // epilogue: lane (g, j) holds channels nt*16 + 4g + r (r = 0..3) of row r0 + j
-        if (r0 + j < n) {
-            T *orow = (T *)a.out + (int64_t)(seg0 + r0 + j) * a.out_stride;
-#pragma unroll
-            for (int gi = 0; gi < NG; ++gi) {
-                const int ch = (nt0 + gi) * 16 + 4 * g;
-                typedef T T4 __attribute__((ext_vector_type(4)));
-                T4 o;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if constexpr (NMAT == 2) {
-                        o[r] = swiglu_rounded<T>(acc[0][gi][r], acc[1][gi][r]);
+                        for (int rs = 0; rs < RS; ++rs)
+                            if (RS == 1 || rs < nfr) {
+                                acc[rs][m][gi] = Act<T>::mfma(w0, __builtin_bit_cast(V8, xq[d][rs][0]), acc[rs][m][gi]);
+                                acc[rs][m][gi] = Act<T>::mfma(w1, __builtin_bit_cast(V8, xq[d][rs][1]), acc[rs][m][gi]);
+                            }
                     } else {
-                        o[r] = (T)acc[0][gi][r];
+                        const V8 w0 = __builtin_bit_cast(V8, q);
+#pragma unroll
+                        for (int rs = 0; rs < RS; ++rs)
+                            if (RS == 1 || rs < nfr)
+                                acc[rs][m][gi] = Act<T>::mfma(w0, __builtin_bit_cast(V8, xq[d][rs][0]), acc[rs][m][gi]);
                     }
                 }
-                *(uint2 *)(orow + ch) = __builtin_bit_cast(uint2, o);
+            if constexpr (SK == 1) {
+                if (kt + 1 == kb) {                // a slice ends: its sum joins the total
+#pragma unroll
+                    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                        for (int gi = 0; gi < NG; ++gi) {
+                            tot[0][m][gi] += acc[0][m][gi];
+                            acc[0][m][gi] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                        }
+                    do { ++sl; kb = KT * (sl + 1) / kSlices; } while (kb == kt + 1 && sl < kSlices - 1);
+                }
             }
+            // refill slot d with chunk kt + D
+            if (kt + D < kend) fetch(d, kt + D);
+        }
+    }
+
+    if constexpr (SK != 1) {
+        // slice sums meet in LDS; the first wave adds them in slice order
+        __shared__ f32x4 red[kSlices][RS * NMAT * NG][64];
+#pragma unroll
+        for (int rs = 0; rs < RS; ++rs)
+            if (RS == 1 || rs < nfr) {
+#pragma unroll
+                for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                    for (int gi = 0; gi < NG; ++gi) red[wave][(rs * NMAT + m) * NG + gi][lane] = acc[rs][m][gi];
+            }
+        __syncthreads();
+        if (wave != 0) return;
+        for (int w = 0; w < kSlices; ++w)
+#pragma unroll
+            for (int rs = 0; rs < RS; ++rs)
+                if (RS == 1 || rs < nfr) {
+#pragma unroll
+                    for (int m = 0; m < NMAT; ++m)
+#pragma unroll
+                        for (int gi = 0; gi < NG; ++gi) tot[rs][m][gi] += red[w][(rs * NMAT + m) * NG + gi][lane];
+                }
+    }
+
+    // epilogue: lane (g, j) holds channels nt*16 + 4g + r (r = 0..3) of row rs*16 + j
+#pragma unroll
+    for (int rs = 0; rs < RS; ++rs) {
+        if (rs * 16 + j >= n) continue;
+        T *orow = (T *)a.out + (int64_t)(seg0 + rs * 16 + j) * a.out_stride;
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) {
+            const int ch = (nt0 + gi) * 16 + 4 * g;
+            typedef T T4 __attribute__((ext_vector_type(4)));
+            T4 o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if constexpr (NMAT == 2) {
+                    o[r] = swiglu_rounded<T>(tot[rs][0][gi][r], tot[rs][1][gi][r]);
+                } else {
+                    o[r] = (T)tot[rs][0][gi][r];
+                }
+            }
+            *(uint2 *)(orow + ch) = __builtin_bit_cast(uint2, o);
         }
     }
 }
@@ -182,36 +250,56 @@ static hipError_t launch_d(const FfnArgs &a, int32_t nseg, hipStream_t s)
         if (KT % D != 0) return launch_d<T, W8, NMAT, NG, D / 2>(a, nseg, s);
     }
     dim3 grid((NT + 4 * NG - 1) / (4 * NG), nseg);
-    hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, D>), grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, D, 1, 1>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
+// Below this many (item, channel group) waves a launch leaves most of the chip's memory
+// system idle: one wave per slice instead.
+constexpr int64_t kSplitBelow = 1536;
+
 template <typename T, bool W8, int NMAT>
-static hipError_t launch_g(const FfnArgs &a, int32_t nseg, hipStream_t s)
+static hipError_t launch_g(const FfnArgs &a, int32_t nseg, bool wide, hipStream_t s)
 {
     constexpr int NG = NMAT == 2 ? EK_TUNE_S1_NG : EK_TUNE_S2_NG;
     constexpr int D = NMAT == 2 ? EK_TUNE_S1_D : EK_TUNE_S2_D;
     const int NT = a.N / 16;
+    if (wide) {
+        // four activation fragments per prefetch slot: shallower, the eight slices make up for it
+        constexpr int DW = W8 ? 2 : 4;
+        if (NT % NG == 0)
+            hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, DW, kSlices, 4>), dim3(NT / NG, nseg),
+                               dim3(64 * kSlices), 0, s, a);
+        else
+            hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, 1, DW, kSlices, 4>), dim3(NT, nseg),
+                               dim3(64 * kSlices), 0, s, a);
+        return hipGetLastError();
+    }
+    if (NT % NG == 0 && (int64_t)nseg * (NT / NG) < kSplitBelow) {
+        hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, D, kSlices, 1>), dim3(NT / NG, nseg),
+                           dim3(64 * kSlices), 0, s, a);
+        return hipGetLastError();
+    }
     if (NT % NG == 0) return launch_d<T, W8, NMAT, NG, D>(a, nseg, s);
     if (NT % 2 == 0) return launch_d<T, W8, NMAT, 2, D>(a, nseg, s);
     return launch_d<T, W8, NMAT, 1, D>(a, nseg, s);
 }
 
-hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items,
+hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items, bool wide,
                              hipStream_t s)
 {
     const int32_t n_segments = (int32_t)max_items;
     if (n_segments <= 0) return hipSuccess;
     if (act == 0) {
-        if (w8) return stage == 1 ? launch_g<__bf16, true, 2>(a, n_segments, s)
-                                  : launch_g<__bf16, true, 1>(a, n_segments, s);
-        return stage == 1 ? launch_g<__bf16, false, 2>(a, n_segments, s)
-                          : launch_g<__bf16, false, 1>(a, n_segments, s);
+        if (w8) return stage == 1 ? launch_g<__bf16, true, 2>(a, n_segments, wide, s)
+                                  : launch_g<__bf16, true, 1>(a, n_segments, wide, s);
+        return stage == 1 ? launch_g<__bf16, false, 2>(a, n_segments, wide, s)
+                          : launch_g<__bf16, false, 1>(a, n_segments, wide, s);
     }
-    if (w8) return stage == 1 ? launch_g<_Float16, true, 2>(a, n_segments, s)
-                              : launch_g<_Float16, true, 1>(a, n_segments, s);
-    return stage == 1 ? launch_g<_Float16, false, 2>(a, n_segments, s)
-                      : launch_g<_Float16, false, 1>(a, n_segments, s);
+    if (w8) return stage == 1 ? launch_g<_Float16, true, 2>(a, n_segments, wide, s)
+                              : launch_g<_Float16, true, 1>(a, n_segments, wide, s);
+    return stage == 1 ? launch_g<_Float16, false, 2>(a, n_segments, wide, s)
+                      : launch_g<_Float16, false, 1>(a, n_segments, wide, s);
 }
 
 }  // namespace ek

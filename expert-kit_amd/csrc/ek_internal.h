@@ -36,6 +36,10 @@ struct ExpertSlab {           // device addresses of one expert's tensors
 // Items of one class are stored expert-ascending, rows ascending.  List sizes
 // depend on the routing, list capacities only on P, so grids are fixed on the
 // host and kernels drop items beyond the device-side count.
+//
+// Wide cut (per-expert entry points only, decided on the host): when a call's tile items
+// would occupy a small part of the chip (see wide_cut_pays), every segment is cut into
+// weight-streaming items of up to kWideRows rows instead and the tile lists stay empty.
 struct WorkItem {
     int32_t expert;
     int32_t row0;    // first packed position
@@ -47,6 +51,14 @@ struct WorkLists {
     WorkItem *items[kNumLists];
     int32_t *count;              // [kNumLists]
 };
+constexpr int kWideRows = 64;
+// tile_items: work items the ordinary cut would give the tile kernel; one of them spreads
+// over ceil(inter / 256) workgroups in stage 1.  Below half a chip of them the streaming
+// kernel, which spreads every item over inter / 16 workgroups, is faster (measured on MI355X).
+inline bool wide_cut_pays(int64_t tile_items, int64_t inter)
+{
+    return tile_items > 0 && tile_items * ((inter + 255) / 256) < 128;
+}
 inline int64_t list_capacity(int list, int64_t P, int64_t E)
 {
     const int64_t min_rows[kNumLists] = {1, 17, 33, 65};
@@ -99,7 +111,7 @@ constexpr int kMaxExperts = 1024;
 // clears *err itself (with a fill kernel, never a memset node: graph-capture safe)
 void launch_pack(const PackArgs &a, hipStream_t s);
 // work lists for one segment [0, n) of expert e (per-expert forward)
-void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, hipStream_t s);
+void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool wide, hipStream_t s);
 // appends the segment (expert, rows row0 .. row0+n-1) to the lists pack has built and maps
 // its rows to tokens 0 .. n-1
 void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token,
@@ -121,8 +133,9 @@ struct FfnArgs {
 };
 // stage = 1: up/gate + SwiGLU epilogue;  stage = 2: down projection
 // act: 0 bf16, 1 f16;  w8: int8 weights with per-channel scales
-// weight-streaming kernel over lists.items[kListStream]; max_items = grid bound
-hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items,
+// weight-streaming kernel over lists.items[kListStream]; max_items = grid bound;
+// wide: items hold up to kWideRows rows (else up to 16)
+hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items, bool wide,
                              hipStream_t s);
 // MFMA tile kernel over the three tile lists (128-row items first, then 64,
 // then 32); max_items[l] bounds list l

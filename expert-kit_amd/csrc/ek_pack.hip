@@ -125,8 +125,16 @@ __global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
     }
 }
 
-__global__ void single_lists_kernel(WorkLists l, int32_t e, int32_t n)
+__global__ void single_lists_kernel(WorkLists l, int32_t e, int32_t n, int32_t wide)
 {
+    if (wide) {
+        int32_t k = 0;
+        for (int32_t r0 = 0; r0 < n; r0 += kWideRows, ++k)
+            l.items[kListStream][k] = WorkItem{e, r0, min(kWideRows, n - r0), 0};
+        l.count[kListT128] = l.count[kListT64] = l.count[kListT32] = 0;
+        l.count[kListStream] = k;
+        return;
+    }
     const SegmentCut c = cut_segment(n);
     if (n > 0) emit_items(l, e, 0, n, 0, 0, 0, 0);
     l.count[kListT128] = c.n128;
@@ -164,9 +172,9 @@ void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0,
     hipLaunchKernelGGL(append_segment_kernel, dim3(1), dim3(256), 0, s, lists, expert, row0, n, row_token);
 }
 
-void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, hipStream_t s)
+void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool wide, hipStream_t s)
 {
-    hipLaunchKernelGGL(single_lists_kernel, dim3(1), dim3(1), 0, s, lists, expert, n);
+    hipLaunchKernelGGL(single_lists_kernel, dim3(1), dim3(1), 0, s, lists, expert, n, wide ? 1 : 0);
 }
 
 __global__ __launch_bounds__(kPackThreads) void pack_rank_kernel(PackArgs a, int nbits)

@@ -203,7 +203,12 @@ ek_status ek_layer_describe(ek_layer *layer, int64_t *hidden, int64_t *inter, in
  * worker answers each with Expert::forward (worker/core.rs:55-59); a worker
  * that collects the concurrent requests hands them over together:
  *   call i: xs[i] [rows[i], H] -> outs[i] [rows[i], H], expert experts[i].
- * Results are bit-identical to n_calls separate ek_layer_expert_forward calls.
+ * A row's result depends only on the row, the expert and the kernel family its
+ * call is cut for: calls of at most 16 rows always take the weight-streaming
+ * kernel and give the same bits alone or batched; longer calls take it too when
+ * the whole launch is small (a lone expert with up to a few hundred rows), the
+ * MFMA tile kernel otherwise, and the two differ in accumulation order (both
+ * within the parity tolerance).
  * The same expert may appear more than once; sum(rows) is bounded like n of
  * ek_layer_expert_forward.  All pointers of one call share `mem`. */
 ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32_t *experts,

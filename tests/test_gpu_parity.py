@@ -184,6 +184,52 @@ def test_expert_forward(ek, oracle, cuda, dt, w8, n):
     ffn.close()
 
 
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w8", [False, True])
+@pytest.mark.parametrize("n", [17, 32, 33, 64, 65, 128, 129, 300])
+def test_tile_route_one_expert(ek, oracle, cuda, dt, w8, n):
+    """Every token routed to one expert with gate weight 1: the layer's cut gives the MFMA tile
+    kernel one segment of n rows (a per-expert call of this size is cut for the streaming
+    kernel instead), and the combine multiplies by exactly 1."""
+    print(f"tile_route dt={dt} w8={w8} n={n}", flush=True)
+    w = wl.Workload("t", 256, 192, 2, 1, n, dt, w8=w8)
+    layer, ws = load_layer(ek, w, experts=[1])
+    g = torch.Generator().manual_seed(1000 + n)
+    x = torch.randn(n, w.hidden, generator=g).to(dt)
+    ids = torch.ones(n, 1, dtype=torch.int32)
+    gw = torch.ones(n, 1, dtype=dt)
+    wu, wg, wd = [t[1] for t in oracle_weights(oracle, ws, 2, dt)]
+    ref = oracle.ffn(x, wu, wg, wd, mode=2)
+    got = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda))
+    ffn_gate(got, ref, f"tile_route dt={dt} w8={w8} n={n}")
+    assert check_vs_rounded(got, ref) > 0.9
+    layer.close()
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w8", [False, True])
+def test_streaming_forms_agree_bitwise(ek, cuda, dt, w8):
+    """The streaming kernel has three launch forms (one wave per channel group; eight waves, one
+    per slice of the contraction; the same with 64-row items).  A row's result is the same
+    bits in all of them."""
+    E, n_items = 256, 200
+    w = wl.Workload("t", 256, 192, E, 1, 16 * n_items, dt, w8=w8)
+    layer, _ = load_layer(ek, w, experts=[0])
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(16 * n_items, w.hidden, generator=g).to(dt).to(cuda)
+    # 200 items x (12 | 8) channel groups: enough waves for the one-wave-per-group form
+    many = torch.cat(layer.experts_forward([0] * n_items, list(x.split(16))))
+    bits = lambda t: t.contiguous().view(torch.int16)
+    for lo, hi in [(0, 1), (16, 32), (5, 21), (0, 64), (32, 132), (100, 356), (7, 24), (0, 17)]:
+        got = layer.expert_forward(0, x[lo:hi].contiguous())   # sliced; 64-row items beyond 16 rows
+        assert torch.equal(bits(got), bits(many[lo:hi])), (lo, hi)
+    # a small batch of mid-sized calls is cut wide as a whole
+    outs = layer.experts_forward([0, 0, 0], [x[0:40].contiguous(), x[40:45].contiguous(), x[45:245].contiguous()])
+    assert torch.equal(bits(torch.cat(outs)), bits(many[:245]))
+    layer.close()
+
+
 def test_expert_forward_special_cases(ek, cuda):
     w = wl.Workload("t", 128, 64, 1, 1, 8, torch.bfloat16)
     ew = wl.make_expert(w, 0)

@@ -54,7 +54,8 @@ def test_worker_forward_equals_expert_forward(ek, dt, w8):
 @pytest.mark.parametrize("w8", [False, True])
 def test_batch_equals_individual_calls(ek, dt, w8):
     layer = make_layer(ek, dt, w8)
-    # every list class, empty calls, repeated experts, calls in no particular expert order
+    # every size class, empty calls, repeated experts, calls in no particular expert order (the batch is
+    # small enough that its longer calls are cut for the streaming kernel, as they are alone)
     calls = [(3, 5), (0, 0), (1, 1), (5, 16), (2, 17), (3, 32), (4, 33), (0, 64), (1, 65), (2, 128), (5, 129),
              (4, 300), (0, 7), (0, 0)]
     ids = [f"m/l3-e{e}" for e, _ in calls]
