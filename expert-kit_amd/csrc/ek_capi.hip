@@ -109,6 +109,11 @@ struct ek_layer {
 
     // staging for host-memory callers (allocated on first use)
     void *st_x = nullptr, *st_w = nullptr, *st_y = nullptr, *st_xp = nullptr;
+    // pinned bounce buffers for their small transfers (see h2d / d2h)
+    char *pin_in = nullptr, *pin_out = nullptr;
+    size_t pin_cap = 0, pin_in_used = 0, pin_out_used = 0;
+    struct PendingOut { void *dst; const char *src; size_t bytes; };
+    std::vector<PendingOut> pin_pending;
     int32_t *st_ids = nullptr;
     // router outputs and staging (allocated on first use)
     int32_t *rt_ids = nullptr;
@@ -183,6 +188,8 @@ void free_layer(ek_layer *L)
     for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
     if (L->h_err) (void)hipHostFree(L->h_err);
     if (L->h_items) (void)hipHostFree(L->h_items);
+    if (L->pin_in) (void)hipHostFree(L->pin_in);
+    if (L->pin_out) (void)hipHostFree(L->pin_out);
     if (L->ev_items) (void)hipEventDestroy(L->ev_items);
     if (L->stream) (void)hipStreamDestroy(L->stream);
     if (L->load_stream) (void)hipStreamDestroy(L->load_stream);
@@ -474,6 +481,76 @@ ek_status ensure_io_staging(ek_layer *L)
     return EK_OK;
 }
 
+// Host <-> device copies of blocking host-memory calls.  A pageable hipMemcpyAsync of tens to
+// hundreds of KiB costs 20-75 us here; the same bytes through pinned memory (a CPU memcpy and
+// a DMA the stream can queue) 10-20 us, and the two meet at about 1 MiB (measured on the
+// MI355X box, both directions).  So transfers up to kBounceMax go through a pinned bounce
+// buffer while it has room; results are copied out of it once the stream has been waited for
+// (bounce_flush).  One call at a time uses the buffers: host-memory calls hold the layer's
+// lock and end with a synchronisation.
+// The buffers start at 2 MiB each and grow with what calls ask for, up to kBounceCapMax (a
+// batch of many small requests, each of which is worth staging).
+constexpr size_t kBounceMax = 1u << 20, kBounceCapMin = 2u << 20, kBounceCapMax = 16u << 20;
+
+ek_status bounce_begin(ek_layer *L, hipStream_t s, size_t want = 0)
+{
+    if (L->pin_in_used || L->pin_out_used || !L->pin_pending.empty()) {
+        // a call that failed half way left transfers behind: let them finish, drop their results
+        EK_HIP(hipStreamSynchronize(s));
+        L->pin_pending.clear();
+        L->pin_in_used = L->pin_out_used = 0;
+    }
+    size_t cap = L->pin_cap ? L->pin_cap : kBounceCapMin;
+    while (cap < want && cap < kBounceCapMax) cap *= 2;
+    if (cap != L->pin_cap) {
+        // nothing is in flight here: host-memory calls end with a synchronisation
+        if (L->pin_in) (void)hipHostFree(L->pin_in);
+        if (L->pin_out) (void)hipHostFree(L->pin_out);
+        L->pin_in = L->pin_out = nullptr;
+        L->pin_cap = 0;
+        EK_HIP(hipHostMalloc((void **)&L->pin_in, cap, hipHostMallocDefault));
+        EK_HIP(hipHostMalloc((void **)&L->pin_out, cap, hipHostMallocDefault));
+        L->pin_cap = cap;
+    }
+    return EK_OK;
+}
+
+ek_status h2d(ek_layer *L, void *dst, const void *src, size_t bytes, hipStream_t s)
+{
+    if (bytes == 0) return EK_OK;
+    if (L->pin_in && bytes <= kBounceMax && L->pin_in_used + bytes <= L->pin_cap) {
+        char *p = L->pin_in + L->pin_in_used;
+        memcpy(p, src, bytes);
+        L->pin_in_used += (bytes + 63) & ~(size_t)63;
+        EK_HIP(hipMemcpyAsync(dst, p, bytes, hipMemcpyHostToDevice, s));
+    } else {
+        EK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
+    }
+    return EK_OK;
+}
+
+ek_status d2h(ek_layer *L, void *dst, const void *src, size_t bytes, hipStream_t s)
+{
+    if (bytes == 0) return EK_OK;
+    if (L->pin_out && bytes <= kBounceMax && L->pin_out_used + bytes <= L->pin_cap) {
+        char *p = L->pin_out + L->pin_out_used;
+        L->pin_out_used += (bytes + 63) & ~(size_t)63;
+        EK_HIP(hipMemcpyAsync(p, src, bytes, hipMemcpyDeviceToHost, s));
+        L->pin_pending.push_back({dst, p, bytes});
+    } else {
+        EK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
+    }
+    return EK_OK;
+}
+
+// after the stream has been waited for
+void bounce_flush(ek_layer *L)
+{
+    for (const auto &p : L->pin_pending) memcpy(p.dst, p.src, p.bytes);
+    L->pin_pending.clear();
+    L->pin_in_used = L->pin_out_used = 0;
+}
+
 ek_status err_to_status(int32_t err)
 {
     if (err & 1) return fail(EK_INVALID_INPUT, "expert id outside [0, n_experts)");
@@ -484,12 +561,16 @@ ek_status err_to_status(int32_t err)
 ek_status copy_route_out(ek_layer *L, const ek_route_out *r, int64_t P, int mem, hipStream_t s)
 {
     if (!r) return EK_OK;
-    const hipMemcpyKind kind = mem == EK_DEVICE ? hipMemcpyDeviceToDevice : hipMemcpyDeviceToHost;
     const int E = L->cfg.n_experts;
-    if (r->counts) EK_HIP(hipMemcpyAsync(r->counts, L->counts, sizeof(int32_t) * E, kind, s));
-    if (r->offsets) EK_HIP(hipMemcpyAsync(r->offsets, L->offsets, sizeof(int32_t) * (E + 1), kind, s));
-    if (P > 0 && r->perm) EK_HIP(hipMemcpyAsync(r->perm, L->perm, sizeof(int32_t) * P, kind, s));
-    if (P > 0 && r->inv_perm) EK_HIP(hipMemcpyAsync(r->inv_perm, L->inv_perm, sizeof(int32_t) * P, kind, s));
+    auto out = [&](void *dst, const void *src, size_t bytes) -> ek_status {
+        if (mem == EK_HOST) return d2h(L, dst, src, bytes, s);
+        EK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s));
+        return EK_OK;
+    };
+    if (r->counts) EK_TRY(out(r->counts, L->counts, sizeof(int32_t) * E));
+    if (r->offsets) EK_TRY(out(r->offsets, L->offsets, sizeof(int32_t) * (E + 1)));
+    if (P > 0 && r->perm) EK_TRY(out(r->perm, L->perm, sizeof(int32_t) * P));
+    if (P > 0 && r->inv_perm) EK_TRY(out(r->inv_perm, L->inv_perm, sizeof(int32_t) * P));
     return EK_OK;
 }
 
@@ -612,6 +693,7 @@ ek_status finish_blocking(ek_layer *L, hipStream_t s)
 {
     EK_HIP(hipMemcpyAsync(L->h_err, L->err, sizeof(int32_t), hipMemcpyDeviceToHost, s));
     EK_HIP(hipStreamSynchronize(s));
+    bounce_flush(L);
     return err_to_status(L->h_err[0]);
 }
 
@@ -748,14 +830,15 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
             if (!stream) st = finish_blocking(layer, s);
         } else {
             EK_TRY(ensure_io_staging(layer));
+            EK_TRY(bounce_begin(layer, s));
             if (T > 0) {
-                EK_HIP(hipMemcpyAsync(layer->st_x, x, (size_t)T * H * 2, hipMemcpyHostToDevice, s));
-                EK_HIP(hipMemcpyAsync(layer->st_ids, ids, (size_t)P * 4, hipMemcpyHostToDevice, s));
-                EK_HIP(hipMemcpyAsync(layer->st_w, w, (size_t)P * (w_f32 ? 4 : 2), hipMemcpyHostToDevice, s));
+                EK_TRY(h2d(layer, layer->st_x, x, (size_t)T * H * 2, s));
+                EK_TRY(h2d(layer, layer->st_ids, ids, (size_t)P * 4, s));
+                EK_TRY(h2d(layer, layer->st_w, w, (size_t)P * (w_f32 ? 4 : 2), s));
             }
             EK_TRY(enqueue_forward(layer, layer->st_x, layer->st_ids, layer->st_w, w_f32, T,
                                    layer->st_y, s));
-            if (T > 0) EK_HIP(hipMemcpyAsync(y, layer->st_y, (size_t)T * H * 2, hipMemcpyDeviceToHost, s));
+            if (T > 0) EK_TRY(d2h(layer, y, layer->st_y, (size_t)T * H * 2, s));
             EK_TRY(copy_route_out(layer, route, P, mem, s));
             st = finish_blocking(layer, s);
         }
@@ -794,10 +877,11 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
         void *d_xp = xp;
         if (mem == EK_HOST) {
             EK_TRY(ensure_io_staging(layer));
-            if (P > 0) EK_HIP(hipMemcpyAsync(layer->st_ids, ids, (size_t)P * 4, hipMemcpyHostToDevice, s));
+            EK_TRY(bounce_begin(layer, s));
+            if (P > 0) EK_TRY(h2d(layer, layer->st_ids, ids, (size_t)P * 4, s));
             d_ids = layer->st_ids;
             if (xp && T > 0) {
-                EK_HIP(hipMemcpyAsync(layer->st_x, x, (size_t)T * H * 2, hipMemcpyHostToDevice, s));
+                EK_TRY(h2d(layer, layer->st_x, x, (size_t)T * H * 2, s));
                 d_x = layer->st_x;
                 d_xp = layer->yp;   // [Pmax, H] scratch of the right size
             }
@@ -805,8 +889,7 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
         ek::launch_pack(pack_args(layer, d_ids, P, false), s);
         if (xp) ek::launch_gather(d_x, layer->row_token, P, H * 2, d_xp, s);
         EK_HIP(hipGetLastError());
-        if (mem == EK_HOST && xp && P > 0)
-            EK_HIP(hipMemcpyAsync(xp, d_xp, (size_t)P * H * 2, hipMemcpyDeviceToHost, s));
+        if (mem == EK_HOST && xp && P > 0) EK_TRY(d2h(layer, xp, d_xp, (size_t)P * H * 2, s));
         EK_TRY(copy_route_out(layer, route, P, mem, s));
         if (!stream) return finish_blocking(layer, s);
         return EK_OK;
@@ -841,7 +924,8 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
             void *d_out = out;
             if (mem == EK_HOST) {
                 EK_TRY(ensure_io_staging(layer));
-                EK_HIP(hipMemcpyAsync(layer->st_x, x, (size_t)n * H * 2, hipMemcpyHostToDevice, s));
+                EK_TRY(bounce_begin(layer, s));
+                EK_TRY(h2d(layer, layer->st_x, x, (size_t)n * H * 2, s));
                 d_x = layer->st_x;
                 d_out = layer->st_y;
             }
@@ -851,10 +935,12 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
                               wide_items <= layer->list_cap[ek::kListStream];
             ek::launch_single_lists(layer->lists, expert, (int32_t)n, wide, s);
             EK_TRY(enqueue_ffn(layer, d_x, nullptr, d_out, n, 1, s, nullptr, wide ? wide_items : 0));
-            if (mem == EK_HOST)
-                EK_HIP(hipMemcpyAsync(out, layer->st_y, (size_t)n * H * 2, hipMemcpyDeviceToHost, s));
+            if (mem == EK_HOST) EK_TRY(d2h(layer, out, layer->st_y, (size_t)n * H * 2, s));
         }
-        if (!stream) EK_HIP(hipStreamSynchronize(s));
+        if (!stream) {
+            EK_HIP(hipStreamSynchronize(s));
+            bounce_flush(layer);
+        }
         {
             std::lock_guard<std::mutex> sl(layer->stats_mu);
             layer->stats.expert_forward_calls += 1;
@@ -964,24 +1050,57 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             EK_HIP(hipMemcpyAsync(layer->lists.count, cnt, sizeof(int32_t) * ek::kNumLists, hipMemcpyHostToDevice, s));
             EK_HIP(hipEventRecord(layer->ev_items, s));
             EK_TRY(ensure_io_staging(layer));
-            const hipMemcpyKind in_kind = mem == EK_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice;
-            const hipMemcpyKind out_kind = mem == EK_HOST ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice;
+            // Many small host requests: their rows are gathered in pinned memory and cross the
+            // bus as one transfer each way (an asynchronous copy costs ~5 us of host time per
+            // call, as much as the memcpy of a decode-sized request).
+            const size_t all_bytes = (size_t)P * H * 2;
+            bool one_transfer = false;
+            if (mem == EK_HOST) {
+                EK_TRY(bounce_begin(layer, s, all_bytes));
+                one_transfer = n_calls > 1 && all_bytes <= layer->pin_cap;
+            }
+            if (one_transfer) {
+                row0 = 0;
+                for (int i = 0; i < n_calls; ++i) {
+                    if (rows[i]) memcpy(layer->pin_in + row0 * H * 2, xs[i], (size_t)rows[i] * H * 2);
+                    row0 += rows[i];
+                }
+                layer->pin_in_used = all_bytes;
+                EK_HIP(hipMemcpyAsync(layer->st_x, layer->pin_in, all_bytes, hipMemcpyHostToDevice, s));
+            }
             row0 = 0;
-            for (int i = 0; i < n_calls; ++i) {
-                if (rows[i])
-                    EK_HIP(hipMemcpyAsync((char *)layer->st_x + row0 * H * 2, xs[i], (size_t)rows[i] * H * 2, in_kind, s));
+            for (int i = 0; i < n_calls && !one_transfer; ++i) {
+                if (rows[i] && mem == EK_HOST)
+                    EK_TRY(h2d(layer, (char *)layer->st_x + row0 * H * 2, xs[i], (size_t)rows[i] * H * 2, s));
+                else if (rows[i])
+                    EK_HIP(hipMemcpyAsync((char *)layer->st_x + row0 * H * 2, xs[i], (size_t)rows[i] * H * 2,
+                                          hipMemcpyDeviceToDevice, s));
                 row0 += rows[i];
             }
             EK_TRY(enqueue_ffn(layer, layer->st_x, nullptr, layer->st_y, P, n_calls, s, nullptr, wide ? wide_items : 0));
             EK_HIP(hipGetLastError());
             row0 = 0;
-            for (int i = 0; i < n_calls; ++i) {
-                if (rows[i])
-                    EK_HIP(hipMemcpyAsync(outs[i], (char *)layer->st_y + row0 * H * 2, (size_t)rows[i] * H * 2, out_kind, s));
+            if (one_transfer) {
+                EK_HIP(hipMemcpyAsync(layer->pin_out, layer->st_y, all_bytes, hipMemcpyDeviceToHost, s));
+                layer->pin_out_used = all_bytes;
+                for (int i = 0; i < n_calls; ++i) {
+                    if (rows[i]) layer->pin_pending.push_back({outs[i], layer->pin_out + row0 * H * 2, (size_t)rows[i] * H * 2});
+                    row0 += rows[i];
+                }
+            }
+            for (int i = 0; i < n_calls && !one_transfer; ++i) {
+                if (rows[i] && mem == EK_HOST)
+                    EK_TRY(d2h(layer, outs[i], (char *)layer->st_y + row0 * H * 2, (size_t)rows[i] * H * 2, s));
+                else if (rows[i])
+                    EK_HIP(hipMemcpyAsync(outs[i], (char *)layer->st_y + row0 * H * 2, (size_t)rows[i] * H * 2,
+                                          hipMemcpyDeviceToDevice, s));
                 row0 += rows[i];
             }
         }
-        if (!stream) EK_HIP(hipStreamSynchronize(s));
+        if (!stream) {
+            EK_HIP(hipStreamSynchronize(s));
+            bounce_flush(layer);
+        }
         {
             std::lock_guard<std::mutex> sl(layer->stats_mu);
             layer->stats.expert_forward_calls += n_calls;
@@ -1373,15 +1492,15 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
     const void *d_logits = logits, *d_x = x;
     const float *d_bias = (const float *)rcfg->bias;
     void *d_y = y;
-    const hipMemcpyKind back = mem == EK_HOST ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice;
     if (mem == EK_HOST) {
         if (forward) EK_TRY(ensure_io_staging(layer));
+        EK_TRY(bounce_begin(layer, s));
         if (T > 0) {
-            EK_HIP(hipMemcpyAsync(layer->st_logits, logits, l_bytes, hipMemcpyHostToDevice, s));
-            if (forward) EK_HIP(hipMemcpyAsync(layer->st_x, x, (size_t)T * H * 2, hipMemcpyHostToDevice, s));
+            EK_TRY(h2d(layer, layer->st_logits, logits, l_bytes, s));
+            if (forward) EK_TRY(h2d(layer, layer->st_x, x, (size_t)T * H * 2, s));
         }
         if (rcfg->bias) {
-            EK_HIP(hipMemcpyAsync(layer->st_bias, rcfg->bias, (size_t)E * 4, hipMemcpyHostToDevice, s));
+            EK_TRY(h2d(layer, layer->st_bias, rcfg->bias, (size_t)E * 4, s));
             d_bias = layer->st_bias;
         }
         d_logits = layer->st_logits;
@@ -1389,12 +1508,17 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
         d_y = layer->st_y;
     }
     EK_TRY(enqueue_router(layer, rcfg, d_logits, d_bias, T, layer->rt_ids, layer->rt_w, s));
-    if (P > 0 && ids_out) EK_HIP(hipMemcpyAsync(ids_out, layer->rt_ids, (size_t)P * 4, back, s));
-    if (P > 0 && w_out) EK_HIP(hipMemcpyAsync(w_out, layer->rt_w, w_bytes, back, s));
+    auto give = [&](void *dst, const void *src, size_t bytes) -> ek_status {
+        if (mem == EK_HOST) return d2h(layer, dst, src, bytes, s);
+        EK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s));
+        return EK_OK;
+    };
+    if (P > 0 && ids_out) EK_TRY(give(ids_out, layer->rt_ids, (size_t)P * 4));
+    if (P > 0 && w_out) EK_TRY(give(w_out, layer->rt_w, w_bytes));
     ek_status st = EK_OK;
     if (forward) {
         EK_TRY(enqueue_forward(layer, d_x, layer->rt_ids, layer->rt_w, w_f32, T, d_y, s));
-        if (mem == EK_HOST && T > 0) EK_HIP(hipMemcpyAsync(y, layer->st_y, (size_t)T * H * 2, hipMemcpyDeviceToHost, s));
+        if (mem == EK_HOST && T > 0) EK_TRY(d2h(layer, y, layer->st_y, (size_t)T * H * 2, s));
         EK_TRY(copy_route_out(layer, route, P, mem, s));
         if (!stream) st = finish_blocking(layer, s);
         std::lock_guard<std::mutex> sl(layer->stats_mu);
@@ -1404,6 +1528,7 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
         if (!stream) { layer->stats.last_forward_us = tm.us(); observe_forward(layer, layer->stats.last_forward_us); }
     } else if (!stream) {
         EK_HIP(hipStreamSynchronize(s));
+        bounce_flush(layer);
     }
     return st;
 }

@@ -55,6 +55,10 @@ class ek_histogram(ctypes.Structure):
                 ("count", ctypes.c_int64)]
 
 
+class ek_batcher_stats(ctypes.Structure):
+    _fields_ = [("calls", ctypes.c_int64), ("batches", ctypes.c_int64), ("largest_batch", ctypes.c_int64)]
+
+
 class ek_router_cfg(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int32), ("renorm", ctypes.c_int32), ("n_group", ctypes.c_int32),
                 ("topk_group", ctypes.c_int32), ("routed_scaling", ctypes.c_float), ("flags", ctypes.c_int32),
@@ -101,6 +105,10 @@ PROTOTYPES = {
     "ek_worker_forward": (_I32, [_P, ctypes.c_char_p, _P, _SZ, _P, _SZ, ctypes.POINTER(_SZ)]),
     "ek_worker_forward_batch": (_I32, [_P, _I32, _STRS, _PP, ctypes.POINTER(_SZ), _PP, ctypes.POINTER(_SZ),
                                        ctypes.POINTER(_SZ)]),
+    "ek_batcher_create": (_I32, [_P, _I64, _I32, _PP]),
+    "ek_batcher_forward": (_I32, [_P, ctypes.c_char_p, _P, _SZ, _P, _SZ, ctypes.POINTER(_SZ)]),
+    "ek_batcher_get_stats": (_I32, [_P, ctypes.POINTER(ek_batcher_stats)]),
+    "ek_batcher_destroy": (_I32, [_P]),
     "ek_layer_route": (_I32, [_P, _P, ctypes.POINTER(ek_router_cfg), _I64, _P, _P, _I32, _P]),
     "ek_layer_forward_logits": (_I32, [_P, _P, _P, ctypes.POINTER(ek_router_cfg), _I64, _P, _P, _P,
                                        ctypes.POINTER(ek_route_out), _I32, _P]),

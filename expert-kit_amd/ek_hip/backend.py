@@ -365,6 +365,41 @@ class HipChain:
             pass
 
 
+class HipBatcher:
+    """Collector of concurrent per-expert requests (one Forward RPC per expert and task,
+    worker/server.rs:39-63): `forward` may be called from many threads at once; the calls in
+    flight together are answered by one grouped launch."""
+
+    def __init__(self, layer: HipLayer, max_wait_us: int = 0, max_calls: int = 256):
+        self._lib = C.load()
+        self.layer = layer
+        self._h = ctypes.c_void_p()
+        C.check(self._lib.ek_batcher_create(layer._h, max_wait_us, max_calls, ctypes.byref(self._h)))
+
+    def forward(self, expert_id: str, req: bytes) -> bytes:
+        cap = len(req) + 64                     # a response is never larger than its request
+        buf = ctypes.create_string_buffer(cap)
+        n = ctypes.c_size_t()
+        C.check(self._lib.ek_batcher_forward(self._h, expert_id.encode(), req, len(req), buf, cap, ctypes.byref(n)))
+        return buf.raw[:n.value]
+
+    def stats(self) -> dict:
+        st = C.ek_batcher_stats()
+        C.check(self._lib.ek_batcher_get_stats(self._h, ctypes.byref(st)))
+        return {"calls": st.calls, "batches": st.batches, "largest_batch": st.largest_batch}
+
+    def close(self) -> None:
+        if getattr(self, "_h", None) is not None and self._h.value:
+            C.check(self._lib.ek_batcher_destroy(self._h))
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class HipFFN:
     """One expert behind trait Expert<T> (ffn/meta.rs:30-39)."""
 

@@ -267,6 +267,30 @@ ek_status ek_worker_forward_batch(ek_layer *layer, int32_t n_calls, const char *
                                   const void *const *reqs, const size_t *req_lens, void *const *resps,
                                   const size_t *resp_caps, size_t *resp_lens);
 
+/* The worker-side collector for the above.  The reference serves each Forward
+ * RPC on its own task (worker/server.rs:39-63 -> worker/core.rs:47-74) and the
+ * controller has one in flight per active expert (controller/executor.rs:
+ * 141-195).  ek_batcher_forward has ek_worker_forward's contract and may be
+ * called from any number of threads: callers that are in flight together are
+ * answered by one grouped launch.  The first caller to arrive leads: it waits
+ * up to max_wait_us for others to join (0: takes what is there), runs up to
+ * max_calls requests as one ek_worker_forward_batch and hands every caller its
+ * own status (a request that fails does not fail its neighbours; the error
+ * text is the caller's ek_last_error()).  Callers arriving while a batch runs
+ * form the next one.  The layer must outlive the batcher; destroy fails while
+ * calls are in flight. */
+typedef struct ek_batcher ek_batcher;
+typedef struct {
+    int64_t calls;          /* requests answered */
+    int64_t batches;        /* grouped launches they were answered by */
+    int64_t largest_batch;
+} ek_batcher_stats;
+ek_status ek_batcher_create(ek_layer *layer, int64_t max_wait_us, int32_t max_calls, ek_batcher **out);
+ek_status ek_batcher_forward(ek_batcher *batcher, const char *expert_id, const void *req, size_t req_len,
+                             void *resp, size_t resp_cap, size_t *resp_len);
+ek_status ek_batcher_get_stats(ek_batcher *batcher, ek_batcher_stats *out);
+ek_status ek_batcher_destroy(ek_batcher *batcher);
+
 /* Turns per-phase HIP-event timing of ek_layer_forward on (1) or off (0) and
  * clears the accumulated kernel_us.  Stands for the PerfTimer checkpoints of
  * the reference (ek-base/src/utils.rs:4-45; controller/executor.rs:136,201,228).

@@ -132,3 +132,16 @@ int main(void) {
     out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, (out.returncode, out.stdout, out.stderr)
     assert out.stdout.strip() == "hip ds-tiny/l3-e17"
+
+
+def test_batcher_rejects_bad_arguments_without_a_gpu(ek):
+    from ek_hip import _capi as C
+    lib = ek.load()
+    out = ctypes.c_void_p()
+    assert lib.ek_batcher_create(None, 0, 1, ctypes.byref(out)) == C.EK_INVALID_INPUT
+    n = ctypes.c_size_t()
+    buf = ctypes.create_string_buffer(8)
+    assert lib.ek_batcher_forward(None, b"m/l0-e0", buf, 8, buf, 8, ctypes.byref(n)) == C.EK_INVALID_INPUT
+    assert lib.ek_batcher_get_stats(None, None) == C.EK_INVALID_INPUT
+    assert lib.ek_batcher_destroy(None) == C.EK_OK
+    assert b"NULL" in lib.ek_last_error()
