@@ -483,14 +483,14 @@ ek_status ensure_io_staging(ek_layer *L)
 
 // Host <-> device copies of blocking host-memory calls.  A pageable hipMemcpyAsync of tens to
 // hundreds of KiB costs 20-75 us here; the same bytes through pinned memory (a CPU memcpy and
-// a DMA the stream can queue) 10-20 us, and the two meet at about 1 MiB (measured on the
-// MI355X box, both directions).  So transfers up to kBounceMax go through a pinned bounce
-// buffer while it has room; results are copied out of it once the stream has been waited for
-// (bounce_flush).  One call at a time uses the buffers: host-memory calls hold the layer's
-// lock and end with a synchronisation.
-// The buffers start at 2 MiB each and grow with what calls ask for, up to kBounceCapMax (a
-// batch of many small requests, each of which is worth staging).
-constexpr size_t kBounceMax = 1u << 20, kBounceCapMin = 2u << 20, kBounceCapMax = 16u << 20;
+// a DMA the stream can queue) 10-20 us; alone the two forms meet between 1 and 4 MiB, inside
+// a call the staged form still wins at 1.8 MiB (DeepSeek-V3 decode layer call with host
+// tensors: 2.67 -> 2.01 ms; measured on the MI355X box).  So transfers up to kBounceMax go
+// through a pinned bounce buffer while it has room; results are copied out of it once the
+// stream has been waited for (bounce_flush).  One call at a time uses the buffers:
+// host-memory calls hold the layer's lock and end with a synchronisation.
+// The buffers start at 2 MiB each; the first call that wants more makes them kBounceCapMax.
+constexpr size_t kBounceMax = 4u << 20, kBounceCapMin = 2u << 20, kBounceCapMax = 16u << 20;
 
 ek_status bounce_begin(ek_layer *L, hipStream_t s, size_t want = 0)
 {
@@ -501,7 +501,7 @@ ek_status bounce_begin(ek_layer *L, hipStream_t s, size_t want = 0)
         L->pin_in_used = L->pin_out_used = 0;
     }
     size_t cap = L->pin_cap ? L->pin_cap : kBounceCapMin;
-    while (cap < want && cap < kBounceCapMax) cap *= 2;
+    if (cap < want) cap = kBounceCapMax;
     if (cap != L->pin_cap) {
         // nothing is in flight here: host-memory calls end with a synchronisation
         if (L->pin_in) (void)hipHostFree(L->pin_in);
@@ -830,7 +830,7 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
             if (!stream) st = finish_blocking(layer, s);
         } else {
             EK_TRY(ensure_io_staging(layer));
-            EK_TRY(bounce_begin(layer, s));
+            EK_TRY(bounce_begin(layer, s, (size_t)T * H * 2 + (size_t)P * 8));
             if (T > 0) {
                 EK_TRY(h2d(layer, layer->st_x, x, (size_t)T * H * 2, s));
                 EK_TRY(h2d(layer, layer->st_ids, ids, (size_t)P * 4, s));
@@ -877,7 +877,7 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
         void *d_xp = xp;
         if (mem == EK_HOST) {
             EK_TRY(ensure_io_staging(layer));
-            EK_TRY(bounce_begin(layer, s));
+            EK_TRY(bounce_begin(layer, s, (size_t)P * H * 2 + (size_t)P * 8));
             if (P > 0) EK_TRY(h2d(layer, layer->st_ids, ids, (size_t)P * 4, s));
             d_ids = layer->st_ids;
             if (xp && T > 0) {
@@ -924,7 +924,7 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
             void *d_out = out;
             if (mem == EK_HOST) {
                 EK_TRY(ensure_io_staging(layer));
-                EK_TRY(bounce_begin(layer, s));
+                EK_TRY(bounce_begin(layer, s, (size_t)n * H * 2));
                 EK_TRY(h2d(layer, layer->st_x, x, (size_t)n * H * 2, s));
                 d_x = layer->st_x;
                 d_out = layer->st_y;
@@ -1494,7 +1494,7 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
     void *d_y = y;
     if (mem == EK_HOST) {
         if (forward) EK_TRY(ensure_io_staging(layer));
-        EK_TRY(bounce_begin(layer, s));
+        EK_TRY(bounce_begin(layer, s, l_bytes + (size_t)T * H * 2 + (size_t)E * 4));
         if (T > 0) {
             EK_TRY(h2d(layer, layer->st_logits, logits, l_bytes, s));
             if (forward) EK_TRY(h2d(layer, layer->st_x, x, (size_t)T * H * 2, s));
