@@ -96,7 +96,11 @@ template <typename T> __device__ __forceinline__ T swiglu_rounded(float acc_up, 
 {
     const float up = rnd<T>(acc_up);
     const float gate = rnd<T>(acc_gate);
-    const float sg = rnd<T>(gate / (1.0f + expf(-gate)));
+    // gate * 1/(1 + 2^(-gate * log2 e)) with the hardware's exp2 and reciprocal (1 ulp each):
+    // the value is rounded to 8 or 11 significant bits next, so this differs from a
+    // correctly rounded quotient in about one element in 10^4, by one 16-bit ulp, and costs a
+    // fifth of the instructions of expf and an IEEE division
+    const float sg = rnd<T>(gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(gate * -1.4426950408889634f)));
     return (T)(up * sg);
 }
 
