@@ -317,6 +317,40 @@ def test_layer_c3_sampled(ek, oracle, cuda):
     layer.close()
 
 
+@pytest.mark.parametrize("name", ["c3", "c4"])
+def test_layer_full_size_sampled_tokens(ek, oracle, cuda, name):
+    """The two DeepSeek-V3 configurations at full size (256 experts resident; 128 decode tokens /
+    8192 prefill tokens with hot-expert skew): the whole layer call on the GPU; the oracle
+    recomputes a handful of tokens (rows are independent in the reference) that between them
+    sit in the longest segment, in a segment short enough for the streaming kernel, in
+    segments whose remainder is cut into a 128-, 64- and 32-row tile (prefill), and four
+    tokens drawn at random."""
+    w = wl.CONFIGS[name]
+    print(f"{name} full size: building {w.n_experts} experts on the GPU", flush=True)
+    layer, ws = load_layer(ek, w, device="cuda")
+    x = wl.make_x(w)
+    ids, gw = wl.make_routing(w)
+    counts = torch.bincount(ids.flatten().long(), minlength=w.n_experts)
+    y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
+    assert torch.equal(rt.counts.cpu().long(), counts)
+    rem = counts % 128
+    classes = [counts == counts.max(), (counts > 0) & (counts <= 16), (counts > 128) & (rem > 64),
+               (counts > 128) & (rem > 32) & (rem <= 64), (counts > 128) & (rem > 16) & (rem <= 32)]
+    tokens = torch.randint(0, w.tokens, (4,), generator=torch.Generator().manual_seed(5)).tolist()
+    for c in classes:                     # the last token routed there: it sits in the segment's remainder
+        if bool(c.any()):
+            e = int(torch.where(c)[0][0])
+            tokens.append(int(torch.where((ids == e).any(dim=1))[0][-1]))
+    tokens = sorted(set(tokens))
+    need = sorted(set(ids[tokens].flatten().tolist()))
+    print(f"{name} full size: tokens {tokens}, {len(need)} experts recomputed by the oracle", flush=True)
+    wu, wg, wd = oracle_weights(oracle, {e: ws[e] for e in need}, w.n_experts)
+    ref, _, _, _, _, y3 = oracle.layer_forward(x[tokens], ids[tokens], gw[tokens], wu, wg, wd, mode=2, return_y3=True)
+    layer_gate(y[tokens], ref, y3, gw[tokens], f"{name} full size, sampled tokens")
+    assert layer.stats()["pairs"] == w.pairs
+    layer.close()
+
+
 # ------------------------------------------------------------ error paths
 
 def test_error_paths(ek, cuda):
