@@ -236,6 +236,8 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.f;
 
+        u32x4 af[2][CB];
+        V8 bf[2][RB];
         for (int step = 0; step < nsteps; ++step) {
             // the DMAs of this step are older than those of the next one (of this tile or of
             // the next tile) and than the previous epilogue's stores: wait until only those remain
@@ -262,59 +264,78 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) aq[tt][cb] = *(const u32x4 *)(wreg + aoff[cb] + tt * 512);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
 
             // A operands of k-group grp: int8 -> half (grp & 1) of read grp >> 1, dequantised;
             // 16-bit -> read grp as it is.  Software pipeline, pinned with scheduling fences:
             // per row block 2 MFMAs, the B fragment read of the next k-group, and a share of
-            // the next k-group's dequantisation.
-            u32x4 af[2][CB];
+            // the next k-group's dequantisation.  The pipeline is rotated by one k-group across
+            // steps: the MFMAs of a step's last k-group (operands already in af[1] / bf[1]) run
+            // at the start of the next step, where they cover the latency of the reads above and
+            // the conversion of that step's first k-group, which nothing else could overlap.
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-                if constexpr (W8) {
-                    const u32x2 lo = dequant_u8x4<T>(aq[0][cb][0], cur.as[cb], cur.ac[cb]);
-                    const u32x2 hi = dequant_u8x4<T>(aq[0][cb][1], cur.as[cb], cur.ac[cb]);
-                    af[0][cb] = (u32x4){lo[0], lo[1], hi[0], hi[1]};
-                } else {
-                    af[0][cb] = aq[0][cb];
+            for (int rb = 0; rb < RB; ++rb) {
+                if (step > 0) {
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb)
+                        acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[1][cb]), bf[1][rb], acc[rb][cb]);
                 }
+                if constexpr (W8) {
+                    constexpr int DW = 4 / RB;
+#pragma unroll
+                    for (int d = 0; d < DW; ++d) {
+                        const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
+                        const u32x2 v = dequant_u8x4<T>(aq[0][cb][part], cur.as[cb], cur.ac[cb]);
+                        af[0][cb][part * 2] = v[0];
+                        af[0][cb][part * 2 + 1] = v[1];
+                    }
+                } else {
+                    if (rb == RB - 1) {
+#pragma unroll
+                        for (int cb = 0; cb < CB; ++cb) af[0][cb] = aq[0][cb];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            V8 bf[2][RB];
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
-#pragma unroll
-            for (int grp = 0; grp < NGRP; ++grp) {
+            for (int grp = 0; grp + 1 < NGRP; ++grp) {
                 const int cg = grp & 1, ng = cg ^ 1;
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
-                    if (grp + 1 < NGRP)
-                        bf[ng][rb] = *(const V8 *)(stage + boff[(grp + 1) % NGRP] + rb * kRowBlockBytes);
+                    bf[ng][rb] = *(const V8 *)(stage + boff[grp + 1] + rb * kRowBlockBytes);
 #pragma unroll
                     for (int cb = 0; cb < CB; ++cb)
                         acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cg][cb]), bf[cg][rb], acc[rb][cb]);
-                    if (grp + 1 < NGRP) {
-                        if constexpr (W8) {
-                            // next group's A operands: 4 dwords (2 per column block) spread over the row blocks
-                            constexpr int DW = 4 / RB;
+                    if constexpr (W8) {
+                        // next group's A operands: 4 dwords (2 per column block) spread over the row blocks
+                        constexpr int DW = 4 / RB;
 #pragma unroll
-                            for (int d = 0; d < DW; ++d) {
-                                const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
-                                const int g1 = grp + 1;
-                                const u32x2 v = dequant_u8x4<T>(aq[g1 >> 1][cb][(g1 & 1) * 2 + part], cur.as[cb], cur.ac[cb]);
-                                af[ng][cb][part * 2] = v[0];
-                                af[ng][cb][part * 2 + 1] = v[1];
-                            }
-                        } else {
-                            if (rb == 0) {
+                        for (int d = 0; d < DW; ++d) {
+                            const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
+                            const int g1 = grp + 1;
+                            const u32x2 v = dequant_u8x4<T>(aq[g1 >> 1][cb][(g1 & 1) * 2 + part], cur.as[cb], cur.ac[cb]);
+                            af[ng][cb][part * 2] = v[0];
+                            af[ng][cb][part * 2 + 1] = v[1];
+                        }
+                    } else {
+                        if (rb == 0) {
 #pragma unroll
-                                for (int cb = 0; cb < CB; ++cb) af[ng][cb] = aq[(grp + 1) % 2][cb];
-                            }
+                            for (int cb = 0; cb < CB; ++cb) af[ng][cb] = aq[(grp + 1) % 2][cb];
                         }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
+            static_assert(((NGRP - 1) & 1) == 1, "the last k-group's operands sit in af[1] / bf[1]");
             ring = ring == 2 ? 0 : ring + 1;
         }
+        // the last step's last k-group
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+                acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[1][cb]), bf[1][rb], acc[rb][cb]);
 
         // ---- epilogue.  A lane holds, for row rb*32 + l%32, channels q*8 + kg*4 + (0..3),
         //      q = 0..3, of each column block: written as they are, a store instruction would
