@@ -131,6 +131,39 @@ def test_pack_bit_exact(ek, oracle, cuda, T, K, E):
     layer.close()
 
 
+def test_pack_random_shapes(ek, oracle, cuda):
+    """Forty seeded draws of (T, K, E) and of the routing's shape -- uniform, one hot expert,
+    a handful of experts only, every pair to the last expert -- around the kernels' own
+    boundaries (the fused / three-kernel switch at 4096 pairs, 64-pair waves, 1024 experts),
+    each on a layer sized for a larger T than the call uses."""
+    g = torch.Generator().manual_seed(20240611)
+    draw = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    for case in range(40):
+        K = draw(1, 8)
+        E = max(K, [1, 2, 7, 64, 129, 256, 1000, 1024][draw(0, 7)])
+        T = [draw(1, 70), draw(500, 530), 4096 // K + draw(-2, 2), draw(2000, 9000)][case % 4]
+        kind = case % 5
+        if kind == 0:
+            ids = torch.randint(0, E, (T, K), generator=g)
+        elif kind == 1:
+            ids = torch.where(torch.rand(T, K, generator=g) < 0.8, torch.full((T, K), E // 2), torch.randint(0, E, (T, K), generator=g))
+        elif kind == 2:
+            ids = torch.randint(0, min(E, 3), (T, K), generator=g) * (E // 3 if E >= 3 else 1)
+        elif kind == 3:
+            ids = torch.full((T, K), E - 1)
+        else:
+            ids = torch.randint(0, E, (T, K), generator=g).sort(dim=0, descending=True).values
+        ids = ids.to(torch.int32)
+        print(f"pack case {case}: T={T} K={K} E={E} kind={kind}", flush=True)
+        layer = ek.HipLayer(64, 64, E, K, max_tokens=T + draw(0, 100))
+        rt = layer.pack(ids.to(cuda))
+        ref = oracle.pack(ids, E)
+        for name, a, b in zip(("counts", "offsets", "perm", "inv_perm"), (rt.counts, rt.offsets, rt.perm, rt.inv_perm), ref):
+            assert torch.equal(a.cpu(), b), (case, name)
+        layer.close()
+
+
+
 @pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
 def test_pack_benchmark_routing(ek, oracle, cuda, name):
     w = wl.resolve(wl.CONFIGS[name])
