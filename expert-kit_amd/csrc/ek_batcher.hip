@@ -12,6 +12,7 @@
 // Host code only.
 #include "../../include/ek_hip.h"
 
+#include <algorithm>
 #include <chrono>
 #include <condition_variable>
 #include <deque>
@@ -34,6 +35,7 @@ struct Slot {
     std::string err;
     bool done = false;
     bool lead = false;
+    bool oom = false;       // failed without room for an error text
 };
 
 }  // namespace
@@ -110,47 +112,62 @@ ek_status ek_batcher_forward(ek_batcher *b, const char *expert_id, const void *r
                              size_t resp_cap, size_t *resp_len)
 {
     if (!b || !expert_id || !req || !resp || !resp_len) { ek::set_last_error("NULL argument"); return EK_INVALID_INPUT; }
+    Slot me;
+    me.expert_id = expert_id; me.req = req; me.req_len = req_len; me.resp = resp; me.resp_cap = resp_cap;
+    std::unique_lock<std::mutex> lk(b->mu);
     try {
-        Slot me;
-        me.expert_id = expert_id; me.req = req; me.req_len = req_len; me.resp = resp; me.resp_cap = resp_cap;
-        std::unique_lock<std::mutex> lk(b->mu);
         b->pending.push_back(&me);
-        b->stats.calls += 1;
-        if (b->active) {
-            b->cv_arrive.notify_one();
-            b->cv_done.wait(lk, [&] { return me.done || me.lead; });
-        } else {
-            b->active = true;
-            me.lead = true;
-        }
-        if (!me.done) {
-            // leading: this slot is at the front of the queue
-            if (b->max_wait_us > 0 && (int32_t)b->pending.size() < b->max_calls)
-                b->cv_arrive.wait_for(lk, std::chrono::microseconds(b->max_wait_us),
-                                      [&] { return (int32_t)b->pending.size() >= b->max_calls; });
-            std::vector<Slot *> batch;
-            while (!b->pending.empty() && (int32_t)batch.size() < b->max_calls) {
-                batch.push_back(b->pending.front());
-                b->pending.pop_front();
-            }
+    } catch (...) {
+        ek::set_last_error("out of host memory");
+        return EK_OOM;
+    }
+    b->stats.calls += 1;
+    if (b->active) {
+        b->cv_arrive.notify_one();
+        b->cv_done.wait(lk, [&] { return me.done || me.lead; });
+    } else {
+        b->active = true;
+        me.lead = true;
+    }
+    if (!me.done) {
+        // leading: this slot is at the front of the queue
+        if (b->max_wait_us > 0 && (int32_t)b->pending.size() < b->max_calls)
+            b->cv_arrive.wait_for(lk, std::chrono::microseconds(b->max_wait_us),
+                                  [&] { return (int32_t)b->pending.size() >= b->max_calls; });
+        std::vector<Slot *> batch;
+        bool ran = false;
+        try {
+            const size_t n = std::min<size_t>(b->pending.size(), (size_t)b->max_calls);
+            batch.assign(b->pending.begin(), b->pending.begin() + (std::ptrdiff_t)n);
+            b->pending.erase(b->pending.begin(), b->pending.begin() + (std::ptrdiff_t)n);
             b->stats.batches += 1;
-            if ((int64_t)batch.size() > b->stats.largest_batch) b->stats.largest_batch = (int64_t)batch.size();
+            if ((int64_t)n > b->stats.largest_batch) b->stats.largest_batch = (int64_t)n;
             lk.unlock();
             run_batch(b, batch);
-            lk.lock();
-            for (Slot *s : batch) s->done = true;
-            if (!b->pending.empty()) b->pending.front()->lead = true;   // the next batch has its leader
-            else b->active = false;
-            b->cv_done.notify_all();
+            ran = true;
+        } catch (...) {
+            // host memory ran out while the batch was cut or run: nobody may be left waiting
         }
-        lk.unlock();
-        if (me.st != EK_OK) ek::set_last_error(me.err.c_str());
-        else *resp_len = me.resp_len;
-        return me.st;
-    } catch (...) {
-        ek::set_last_error("exception in ek_batcher_forward");
-        return EK_INTERNAL;
+        if (!lk.owns_lock()) lk.lock();
+        if (!ran) {
+            if (batch.empty()) {              // never cut: this caller fails alone and the queue moves on
+                b->pending.pop_front();
+                me.st = EK_OOM;
+                me.oom = true;
+                me.done = true;
+            }
+            for (Slot *s : batch) { s->st = EK_OOM; s->oom = true; }
+        }
+        for (Slot *s : batch) s->done = true;
+        if (!b->pending.empty()) b->pending.front()->lead = true;   // the next batch has its leader
+        else b->active = false;
+        b->cv_done.notify_all();
     }
+    lk.unlock();
+    if (me.oom) ek::set_last_error("out of host memory");
+    else if (me.st != EK_OK) ek::set_last_error(me.err.c_str());
+    else *resp_len = me.resp_len;
+    return me.st;
 }
 
 ek_status ek_batcher_get_stats(ek_batcher *b, ek_batcher_stats *out)
