@@ -85,7 +85,8 @@ int64_t elem_size(int dt)
 struct ek_layer {
     ek_cfg cfg{};
     int act = 0;        // 0 bf16, 1 f16
-    bool w8 = false;
+    bool w8 = false;          // one-byte weights (int8 per channel or fp8 per block)
+    int wmode = 0;            // ek::WeightMode
     int64_t Pmax = 0;
     hipStream_t stream = nullptr;
     std::mutex mu;       // serialises users of the workspace and the slab table
@@ -204,11 +205,14 @@ ek_status validate_cfg(const ek_cfg *c)
     if (!c) return fail(EK_INVALID_INPUT, "cfg is NULL");
     if (c->act_dtype != EK_BF16 && c->act_dtype != EK_F16)
         return fail(EK_INVALID_INPUT, "act_dtype must be EK_BF16 or EK_F16 (got %d)", c->act_dtype);
-    if (c->w_dtype != c->act_dtype && c->w_dtype != EK_I8)
-        return fail(EK_INVALID_INPUT, "w_dtype must equal act_dtype or be EK_I8 (got %d)", c->w_dtype);
+    if (c->w_dtype != c->act_dtype && c->w_dtype != EK_I8 && c->w_dtype != EK_F8E4M3)
+        return fail(EK_INVALID_INPUT, "w_dtype must equal act_dtype or be EK_I8 or EK_F8E4M3 (got %d)", c->w_dtype);
+    if (c->w_dtype == EK_F8E4M3 && (c->hidden > 8192 || c->inter > 8192))
+        return fail(EK_INVALID_INPUT, "fp8 block-scaled layers hold at most 64 scale blocks per row: hidden and "
+                    "inter must not exceed 8192");
     const int64_t ke = 64;   // contraction step of the tile kernel; int8 chunk width
     // the tile kernel's pipeline needs two contraction steps (64 wide for int8, 32 for 16-bit)
-    const int64_t kmin = c->w_dtype == EK_I8 ? 128 : 64;
+    const int64_t kmin = c->w_dtype == EK_I8 || c->w_dtype == EK_F8E4M3 ? 128 : 64;
     if (c->hidden < kmin || c->inter < kmin || c->hidden % ke || c->inter % ke)
         return fail(EK_INVALID_INPUT, "hidden (%lld) and inter (%lld) must be multiples of %lld (at least 128 for int8)",
                     (long long)c->hidden, (long long)c->inter, (long long)ke);
@@ -234,7 +238,8 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     if (!L) return fail(EK_OOM, "host allocation failed");
     L->cfg = *cfg;
     L->act = cfg->act_dtype == EK_BF16 ? 0 : 1;
-    L->w8 = cfg->w_dtype == EK_I8;
+    L->w8 = cfg->w_dtype == EK_I8 || cfg->w_dtype == EK_F8E4M3;
+    L->wmode = cfg->w_dtype == EK_I8 ? ek::kWI8 : cfg->w_dtype == EK_F8E4M3 ? ek::kWF8Block : ek::kW16;
     L->Pmax = pmax;
     const int E = cfg->n_experts;
     // slot E of the tables is the shared expert; its segment (one row per token) follows the
@@ -302,15 +307,25 @@ ek_status expert_slot(ek_layer *L, int32_t expert, int32_t *slot)
     return EK_OK;
 }
 
-ek_status check_desc(const ek_weight_desc *d, const char *name, int64_t rows, int64_t cols, bool w8)
+ek_status check_desc(const ek_weight_desc *d, const char *name, int64_t rows, int64_t cols, int wmode)
 {
+    const bool w8 = wmode == ek::kWI8;
     if (!d || !d->ptr) return fail(EK_WEIGHT_NOT_FOUND, "%s weight is missing", name);
     if (d->rows != rows || d->cols != cols)
         return fail(EK_INVALID_INPUT, "%s weight is [%lld,%lld], expected [%lld,%lld]", name,
                     (long long)d->rows, (long long)d->cols, (long long)rows, (long long)cols);
     if (d->mem != EK_HOST && d->mem != EK_DEVICE)
         return fail(EK_INVALID_INPUT, "%s weight: bad mem %d", name, d->mem);
-    if (w8) {
+    if (wmode == ek::kWF8Block) {
+        // kept as stored: fp8 bytes and the checkpoint's 128 x 128 scale blocks
+        if (d->dtype != EK_F8E4M3)
+            return fail(EK_INVALID_INPUT, "%s weight must be EK_F8E4M3 for an fp8 layer (got %d)", name, d->dtype);
+        if (d->scale_kind != EK_SCALE_BLOCK128)
+            return fail(EK_INVALID_INPUT, "%s weight: fp8 needs EK_SCALE_BLOCK128", name);
+        if (!d->scale) return fail(EK_WEIGHT_NOT_FOUND, "%s block scale is missing", name);
+        if (d->scale_dtype != EK_BF16 && d->scale_dtype != EK_F32 && d->scale_dtype != EK_F16)
+            return fail(EK_INVALID_INPUT, "%s scale: bad dtype %d", name, d->scale_dtype);
+    } else if (w8) {
         if (d->dtype != EK_I8)
             return fail(EK_INVALID_INPUT, "%s weight must be EK_I8 for an int8 layer (got %d)", name,
                         d->dtype);
@@ -362,12 +377,16 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
                             const ek_weight_desc *gate, const ek_weight_desc *down)
 {
     const int64_t H = L->cfg.hidden, I = L->cfg.inter;
-    EK_TRY(check_desc(up, "up", I, H, L->w8));
-    EK_TRY(check_desc(gate, "gate", I, H, L->w8));
-    EK_TRY(check_desc(down, "down", H, I, L->w8));
+    EK_TRY(check_desc(up, "up", I, H, L->wmode));
+    EK_TRY(check_desc(gate, "gate", I, H, L->wmode));
+    EK_TRY(check_desc(down, "down", H, I, L->wmode));
     const size_t wsz = L->w8 ? 1 : 2;
     const size_t mat_bytes = (size_t)H * I * wsz;
-    const size_t scale_floats = L->w8 ? (size_t)(2 * I + H) : 0;
+    const bool blocks = L->wmode == ek::kWF8Block;
+    // scales kept beside the weights: one per output channel (int8) or per 128 x 128 block (fp8)
+    const size_t nb_ih = (size_t)((I + 127) / 128) * (size_t)((H + 127) / 128);
+    const size_t s_upgate = blocks ? nb_ih : (size_t)I, s_dn = blocks ? nb_ih : (size_t)H;
+    const size_t scale_floats = L->w8 ? 2 * s_upgate + s_dn : 0;
     const size_t total = 3 * mat_bytes + scale_floats * sizeof(float);
 
     // staging for host sources: three raw matrices (+ scales) back to back
@@ -400,13 +419,13 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
     slab.down = base + 2 * mat_bytes;
     float *sc = (float *)(base + 3 * mat_bytes);
     slab.s_up = L->w8 ? sc : nullptr;
-    slab.s_gate = L->w8 ? sc + I : nullptr;
-    slab.s_down = L->w8 ? sc + 2 * I : nullptr;
+    slab.s_gate = L->w8 ? sc + s_upgate : nullptr;
+    slab.s_down = L->w8 ? sc + 2 * s_upgate : nullptr;
 
     ek_status st = EK_OK;
     size_t off = 0;
-    const int dst_dt = L->w8 ? EK_I8 : L->cfg.act_dtype;
-    float *sdst[3] = {sc, sc + I, sc + 2 * I};
+    const int dst_dt = L->w8 ? L->cfg.w_dtype : L->cfg.act_dtype;
+    float *sdst[3] = {sc, sc + s_upgate, sc + 2 * s_upgate};
     uint8_t *wdst[3] = {base, base, base + 2 * mat_bytes};
     const int mi[3] = {0, 1, 0}, nmat[3] = {2, 2, 1};
     for (int i = 0; i < 3 && st == EK_OK; ++i) {
@@ -424,9 +443,11 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
             if (st != EK_OK) break;
         }
         ek::launch_tile_weights(src, d->dtype, d->rows, d->cols, wdst[i], dst_dt, mi[i], nmat[i],
-                                d->scale_kind == EK_SCALE_BLOCK128 ? ssrc : nullptr, d->scale_dtype,
+                                d->scale_kind == EK_SCALE_BLOCK128 && !blocks ? ssrc : nullptr, d->scale_dtype,
                                 L->load_stream);
-        if (L->w8) ek::launch_scales_to_f32(ssrc, d->scale_dtype, d->rows, sdst[i], L->load_stream);
+        if (L->w8)
+            ek::launch_scales_to_f32(ssrc, d->scale_dtype, blocks ? (int64_t)(i == 2 ? s_dn : s_upgate) : d->rows,
+                                     sdst[i], L->load_stream);
     }
     if (st == EK_OK) {
         hipError_t e = hipGetLastError();
@@ -619,9 +640,9 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
         if (cap[l] < 0) cap[l] = 0;
     }
     if (wide_items > 0) {
-        EK_HIP(ek::launch_ffn_stream(a1, 1, L->act, L->w8, wide_items, true, s));
+        EK_HIP(ek::launch_ffn_stream(a1, 1, L->act, L->wmode, wide_items, true, s));
         if (ev) EK_HIP(hipEventRecord(ev[2], s));
-        EK_HIP(ek::launch_ffn_stream(a2, 2, L->act, L->w8, wide_items, true, s));
+        EK_HIP(ek::launch_ffn_stream(a2, 2, L->act, L->wmode, wide_items, true, s));
         return EK_OK;
     }
     // Two independent chains: the weight-streaming kernel (items of <= 16 rows) and the
@@ -643,8 +664,8 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
     }
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
-        if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->w8, cap[ek::kListStream], false, s_stream));
-        if (have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->w8, cap, s_tiles));
+        if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, cap[ek::kListStream], false, s_stream));
+        if (have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
     }
     if (fork) {

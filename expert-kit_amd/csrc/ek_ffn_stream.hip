@@ -45,9 +45,12 @@ namespace ek {
 
 constexpr int kSlices = 8;
 
-template <typename T, bool W8, int NMAT, int NG, int D, int SK, int RS>
+constexpr int kMaxScaleBlocks = 64;   // 128-wide scale blocks along the contraction: K <= 8192
+
+template <typename T, int WM, int NMAT, int NG, int D, int SK, int RS>
 __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kernel(FfnArgs a)
 {
+    constexpr bool W8 = WM != kW16;    // one-byte weights: 64 contraction elements per chunk
     static_assert(SK == 1 || SK == kSlices, "one wave per launch shape or one wave per slice");
     static_assert(RS == 1 || SK == kSlices, "wide items only in the sliced form");
     using V8 = typename Act<T>::V8;
@@ -80,13 +83,32 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
 #pragma unroll
         for (int m = 0; m < NMAT; ++m) {
             float sv = 1.f;
-            if constexpr (W8) {
+            if constexpr (WM == kWI8) {
                 const int ch = (nt0 + gi) * 16 + j;
                 sv = NMAT == 2 ? (m == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
             }
             ws[gi * NMAT + m] = sv;
             wc[gi * NMAT + m] = -128.f * sv;
         }
+
+    // Block scales: the wave's 16 channels lie in one 128-row block, so the scale of a chunk is
+    // one number per 128 contraction elements: the wave keeps its rows of the scale matrices in
+    // LDS (lane b holds block b) and reads one back per chunk.
+    __shared__ float srow[WM == kWF8Block ? (SK == 1 ? 4 : kSlices) : 1][WM == kWF8Block ? NW : 1]
+                         [WM == kWF8Block ? kMaxScaleBlocks : 1];
+    if constexpr (WM == kWF8Block) {
+        const int KB = (a.Kdim + 127) >> 7;
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+            for (int m = 0; m < NMAT; ++m) {
+                const float *smat = NMAT == 2 ? (m == 0 ? slab.s_up : slab.s_gate) : slab.s_down;
+                if (lane < KB) srow[wave][gi * NMAT + m][lane] = smat[(int64_t)(((nt0 + gi) * 16) >> 7) * KB + lane];
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
 
     const int nfr = RS == 1 ? 1 : (n + 15) >> 4;   // 16-row fragments that hold rows
     const T *xp[RS];
@@ -145,8 +167,16 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
                 for (int m = 0; m < NMAT; ++m) {
                     const uint4 q = wq[d][gi * NMAT + m];
                     if constexpr (W8) {
-                        const float sv = ws[gi * NMAT + m], cv = wc[gi * NMAT + m];
-                        const V8 w0 = dequant_u8x8<T>(q.x, q.y, sv, cv), w1 = dequant_u8x8<T>(q.z, q.w, sv, cv);
+                        V8 w0, w1;
+                        if constexpr (WM == kWI8) {
+                            const float sv = ws[gi * NMAT + m], cv = wc[gi * NMAT + m];
+                            w0 = dequant_u8x8<T>(q.x, q.y, sv, cv);
+                            w1 = dequant_u8x8<T>(q.z, q.w, sv, cv);
+                        } else {
+                            const float sv = srow[wave][gi * NMAT + m][kt >> 1];
+                            w0 = dequant_f8x8<T>(q.x, q.y, sv);
+                            w1 = dequant_f8x8<T>(q.z, q.w, sv);
+                        }
 #pragma unroll
                         for (int rs = 0; rs < RS; ++rs)
                             if (RS == 1 || rs < nfr) {
@@ -240,17 +270,17 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
 #define EK_TUNE_S2_D 8
 #endif
 
-template <typename T, bool W8, int NMAT, int NG, int D>
+template <typename T, int WM, int NMAT, int NG, int D>
 static hipError_t launch_d(const FfnArgs &a, int32_t nseg, hipStream_t s)
 {
-    constexpr int KE = W8 ? 64 : 32;
+    constexpr int KE = WM != kW16 ? 64 : 32;
     const int KT = a.Kdim / KE;
     const int NT = a.N / 16;
     if constexpr (D > 1) {
-        if (KT % D != 0) return launch_d<T, W8, NMAT, NG, D / 2>(a, nseg, s);
+        if (KT % D != 0) return launch_d<T, WM, NMAT, NG, D / 2>(a, nseg, s);
     }
     dim3 grid((NT + 4 * NG - 1) / (4 * NG), nseg);
-    hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, D, 1, 1>), grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((ffn_stream_kernel<T, WM, NMAT, NG, D, 1, 1>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
@@ -258,7 +288,7 @@ static hipError_t launch_d(const FfnArgs &a, int32_t nseg, hipStream_t s)
 // system idle: one wave per slice instead.
 constexpr int64_t kSplitBelow = 1536;
 
-template <typename T, bool W8, int NMAT>
+template <typename T, int WM, int NMAT>
 static hipError_t launch_g(const FfnArgs &a, int32_t nseg, bool wide, hipStream_t s)
 {
     constexpr int NG = NMAT == 2 ? EK_TUNE_S1_NG : EK_TUNE_S2_NG;
@@ -266,40 +296,46 @@ static hipError_t launch_g(const FfnArgs &a, int32_t nseg, bool wide, hipStream_
     const int NT = a.N / 16;
     if (wide) {
         // four activation fragments per prefetch slot: shallower, the eight slices make up for it
-        constexpr int DW = W8 ? 2 : 4;
+        constexpr int DW = WM != kW16 ? 2 : 4;
         if (NT % NG == 0)
-            hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, DW, kSlices, 4>), dim3(NT / NG, nseg),
+            hipLaunchKernelGGL((ffn_stream_kernel<T, WM, NMAT, NG, DW, kSlices, 4>), dim3(NT / NG, nseg),
                                dim3(64 * kSlices), 0, s, a);
         else
-            hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, 1, DW, kSlices, 4>), dim3(NT, nseg),
+            hipLaunchKernelGGL((ffn_stream_kernel<T, WM, NMAT, 1, DW, kSlices, 4>), dim3(NT, nseg),
                                dim3(64 * kSlices), 0, s, a);
         return hipGetLastError();
     }
     if (NT % NG == 0 && (int64_t)nseg * (NT / NG) < kSplitBelow) {
-        hipLaunchKernelGGL((ffn_stream_kernel<T, W8, NMAT, NG, D, kSlices, 1>), dim3(NT / NG, nseg),
+        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, NMAT, NG, D, kSlices, 1>), dim3(NT / NG, nseg),
                            dim3(64 * kSlices), 0, s, a);
         return hipGetLastError();
     }
-    if (NT % NG == 0) return launch_d<T, W8, NMAT, NG, D>(a, nseg, s);
-    if (NT % 2 == 0) return launch_d<T, W8, NMAT, 2, D>(a, nseg, s);
-    return launch_d<T, W8, NMAT, 1, D>(a, nseg, s);
+    if (NT % NG == 0) return launch_d<T, WM, NMAT, NG, D>(a, nseg, s);
+    if (NT % 2 == 0) return launch_d<T, WM, NMAT, 2, D>(a, nseg, s);
+    return launch_d<T, WM, NMAT, 1, D>(a, nseg, s);
 }
 
-hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items, bool wide,
+template <typename T>
+static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, int32_t n_segments, bool wide, hipStream_t s)
+{
+    switch (wmode) {
+    case kWI8:
+        return stage == 1 ? launch_g<T, kWI8, 2>(a, n_segments, wide, s) : launch_g<T, kWI8, 1>(a, n_segments, wide, s);
+    case kWF8Block:
+        return stage == 1 ? launch_g<T, kWF8Block, 2>(a, n_segments, wide, s)
+                          : launch_g<T, kWF8Block, 1>(a, n_segments, wide, s);
+    default:
+        return stage == 1 ? launch_g<T, kW16, 2>(a, n_segments, wide, s) : launch_g<T, kW16, 1>(a, n_segments, wide, s);
+    }
+}
+
+hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, int wmode, int64_t max_items, bool wide,
                              hipStream_t s)
 {
     const int32_t n_segments = (int32_t)max_items;
     if (n_segments <= 0) return hipSuccess;
-    if (act == 0) {
-        if (w8) return stage == 1 ? launch_g<__bf16, true, 2>(a, n_segments, wide, s)
-                                  : launch_g<__bf16, true, 1>(a, n_segments, wide, s);
-        return stage == 1 ? launch_g<__bf16, false, 2>(a, n_segments, wide, s)
-                          : launch_g<__bf16, false, 1>(a, n_segments, wide, s);
-    }
-    if (w8) return stage == 1 ? launch_g<_Float16, true, 2>(a, n_segments, wide, s)
-                              : launch_g<_Float16, true, 1>(a, n_segments, wide, s);
-    return stage == 1 ? launch_g<_Float16, false, 2>(a, n_segments, wide, s)
-                      : launch_g<_Float16, false, 1>(a, n_segments, wide, s);
+    return act == 0 ? launch_w<__bf16>(a, stage, wmode, n_segments, wide, s)
+                    : launch_w<_Float16>(a, stage, wmode, n_segments, wide, s);
 }
 
 }  // namespace ek

@@ -92,18 +92,23 @@ template <typename T, int NR, int LX> struct TileCtx {
     float as[2], ac[2];      // dequantisation constants of the lane's channel, per column block
     int row0, nrows;         // the item's packed rows
     int chan0;               // first output channel of the wave's block
+    int sslot;               // block-scaled weights: which of the two LDS scale areas holds this tile's rows
 };
 
 // All tiles of one class (MR*16-row items) that fall to this workgroup: tiles first,
 // first + stride, ... of `ntiles`, tile = (item, channel block).  The LDS-DMA pipeline
 // runs across tile boundaries: the first two steps of the next tile are issued during the
 // last two steps of the current one, so only the epilogue separates two tiles.
-template <typename T, bool W8, int NMAT, int MR>
+constexpr int kTileScaleBlocks = 64;   // 128-wide scale blocks along the contraction: K <= 8192
+constexpr int kTileScaleBytes = 2 * kTileWaves * 2 * kTileScaleBlocks * 4;   // [tile parity][wave][column block][block]
+
+template <typename T, int WM, int NMAT, int MR>
 __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *items, const int ntiles,
                                           const int nb_count, const int first, const int stride,
                                           uint8_t *lds, const uint32_t lds_base)
 {
     using V8 = typename Act<T>::V8;
+    constexpr bool W8 = WM != kW16;            // one-byte weights
     using G = TileGeom<W8>;
     constexpr int NR = NMAT == 2 ? 2 : 4;      // channel tiles per wave and matrix
     constexpr int NWC = NR * NMAT;             // weight chunks per wave and step (always 4)
@@ -162,7 +167,13 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 
     // Fills `c` for the first tile at or after index t (stepping by stride) whose expert is
     // loaded; returns its index or -1.
-    auto fetch = [&](int t, Ctx &c) -> int {
+    // block scales (fp8 weights): the wave's 32-channel column blocks lie in one 128-row block
+    // each, so a step's scale is one number per column block; the tile's rows of the scale
+    // matrices sit in a wave-private LDS area (two areas: the next tile's rows are fetched while
+    // this one's are in use)
+    float *const sc_area = (float *)(lds + kTileStages * G::STAGE) + wave * (2 * kTileScaleBlocks);
+    constexpr int kScaleSlotFloats = kTileWaves * 2 * kTileScaleBlocks;
+    auto fetch = [&](int t, Ctx &c, int sslot) -> int {
         for (; t < ntiles; t += stride) {
             const WorkItem item = items[t / nb_count];
             const int nb = t % nb_count;
@@ -181,13 +192,25 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 float sv = 1.f;
-                if constexpr (W8) {
+                if constexpr (WM == kWI8) {
                     const int nr = NMAT == 2 ? hh : cb * 2 + hh;
                     const int ch = min(cblock * NR + nr, NT - 1) * 16 + j;
                     sv = NMAT == 2 ? (cb == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
                 }
                 c.as[cb] = sv;
                 c.ac[cb] = -128.f * sv;
+                if constexpr (WM == kWF8Block) {
+                    const int KB = (a.Kdim + 127) >> 7;
+                    const int ct = min(cblock * NR + (NMAT == 2 ? 0 : cb * 2), NT - 1);
+                    const float *smat = NMAT == 2 ? (cb == 0 ? slab.s_up : slab.s_gate) : slab.s_down;
+                    if (lane < KB)
+                        sc_area[sslot * kScaleSlotFloats + cb * kTileScaleBlocks + lane] = smat[(int64_t)((ct * 16) >> 7) * KB + lane];
+                }
+            }
+            c.sslot = sslot;
+            if constexpr (WM == kWF8Block) {
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
             }
 #pragma unroll
             for (int i = 0; i < LX; ++i) {
@@ -211,7 +234,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     }
 
     Ctx cur, nxt;
-    int tc = fetch(first, cur);
+    int tc = fetch(first, cur, 0);
     if (tc < 0) return;
     int ring = 0;                                // stage of the current step
     block_barrier();                             // every wave has left the previous class's stages
@@ -249,7 +272,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             }
             block_barrier();   // this step's tile is visible to all waves; the stage of the
                                // previous step is free again
-            if (step == fstep) tn = fetch(tc + stride, nxt);
+            if (step == fstep) tn = fetch(tc + stride, nxt, cur.sslot ^ 1);
             const int ring2 = ring == 0 ? 2 : ring - 1;          // (ring + 2) % 3
             if (step + 2 < nsteps) {
                 EK_ISSUE(cur, step + 2, ring2);
@@ -266,6 +289,16 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                 for (int cb = 0; cb < CB; ++cb) aq[tt][cb] = *(const u32x4 *)(wreg + aoff[cb] + tt * 512);
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
+            float sblk[CB] = {};        // block-scaled weights: this step's scale per column block
+            if constexpr (WM == kWF8Block) {
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+                    sblk[cb] = sc_area[cur.sslot * kScaleSlotFloats + cb * kTileScaleBlocks + (step >> 1)];
+            }
+            auto dq = [&](uint32_t w, int cb) -> u32x2 {
+                if constexpr (WM == kWF8Block) return dequant_f8x4<T>(w, sblk[cb]);
+                else return dequant_u8x4<T>(w, cur.as[cb], cur.ac[cb]);
+            };
 
             // A operands of k-group grp: int8 -> half (grp & 1) of read grp >> 1, dequantised;
             // 16-bit -> read grp as it is.  Software pipeline, pinned with scheduling fences:
@@ -286,7 +319,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 #pragma unroll
                     for (int d = 0; d < DW; ++d) {
                         const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
-                        const u32x2 v = dequant_u8x4<T>(aq[0][cb][part], cur.as[cb], cur.ac[cb]);
+                        const u32x2 v = dq(aq[0][cb][part], cb);
                         af[0][cb][part * 2] = v[0];
                         af[0][cb][part * 2 + 1] = v[1];
                     }
@@ -314,7 +347,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                         for (int d = 0; d < DW; ++d) {
                             const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
                             const int g1 = grp + 1;
-                            const u32x2 v = dequant_u8x4<T>(aq[g1 >> 1][cb][(g1 & 1) * 2 + part], cur.as[cb], cur.ac[cb]);
+                            const u32x2 v = dq(aq[g1 >> 1][cb][(g1 & 1) * 2 + part], cb);
                             af[ng][cb][part * 2] = v[0];
                             af[ng][cb][part * 2 + 1] = v[1];
                         }
@@ -401,25 +434,26 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 // neighbouring CUs share the activation tile (same item) and mostly the expert's weights
 // in the XCD's L2.  Every workgroup's tile sequence is fixed by its index: no queues, no
 // spinning, and it ends when its indices run out.
-template <typename T, bool W8, int NMAT>
+template <typename T, int WM, int NMAT>
 __global__ __launch_bounds__(kTileThreads, 1) void ffn_tile_kernel(FfnArgs a, int nb_count)
 {
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[kTileStages * TileGeom<W8>::STAGE];
+    __shared__ __attribute__((aligned(1024)))
+    uint8_t lds[kTileStages * TileGeom<WM != kW16>::STAGE + (WM == kWF8Block ? kTileScaleBytes : 0)];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)lds;
     const int x = blockIdx.x & 7, slot = blockIdx.x >> 3, nslots = gridDim.x >> 3;
     const int n128 = a.lists.count[kListT128], n64 = a.lists.count[kListT64], n32 = a.lists.count[kListT32];
     const int lo128 = x * n128 / 8, s128 = (x + 1) * n128 / 8 - lo128;
     const int lo64 = x * n64 / 8, s64 = (x + 1) * n64 / 8 - lo64;
     const int lo32 = x * n32 / 8, s32 = (x + 1) * n32 / 8 - lo32;
-    run_tiles<T, W8, NMAT, 8>(a, a.lists.items[kListT128] + lo128, s128 * nb_count, nb_count, slot, nslots, lds, lds_base);
+    run_tiles<T, WM, NMAT, 8>(a, a.lists.items[kListT128] + lo128, s128 * nb_count, nb_count, slot, nslots, lds, lds_base);
     // the shorter classes start where the long one left the CUs least loaded
     const int r64 = (slot + nslots - (s128 * nb_count) % nslots) % nslots;
-    run_tiles<T, W8, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds, lds_base);
+    run_tiles<T, WM, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds, lds_base);
     const int r32 = (r64 + nslots - (s64 * nb_count) % nslots) % nslots;
-    run_tiles<T, W8, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32, nslots, lds, lds_base);
+    run_tiles<T, WM, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32, nslots, lds, lds_base);
 }
 
-template <typename T, bool W8, int NMAT>
+template <typename T, int WM, int NMAT>
 static hipError_t launch_t(const FfnArgs &a, const int64_t max_items[kNumLists], hipStream_t s)
 {
     constexpr int NR = NMAT == 2 ? 2 : 4;
@@ -430,24 +464,28 @@ static hipError_t launch_t(const FfnArgs &a, const int64_t max_items[kNumLists],
     int64_t slots = per_xcd * nb_count;          // tiles an XCD can get at most
     if (slots <= 0) return hipSuccess;
     if (slots > kCusPerXcd) slots = kCusPerXcd;
-    hipLaunchKernelGGL((ffn_tile_kernel<T, W8, NMAT>), dim3((unsigned)(slots * 8)), dim3(kTileThreads), 0, s, a,
+    hipLaunchKernelGGL((ffn_tile_kernel<T, WM, NMAT>), dim3((unsigned)(slots * 8)), dim3(kTileThreads), 0, s, a,
                        nb_count);
     return hipGetLastError();
 }
 
-hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, bool w8,
+template <typename T>
+static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, const int64_t max_items[kNumLists], hipStream_t s)
+{
+    switch (wmode) {
+    case kWI8:
+        return stage == 1 ? launch_t<T, kWI8, 2>(a, max_items, s) : launch_t<T, kWI8, 1>(a, max_items, s);
+    case kWF8Block:
+        return stage == 1 ? launch_t<T, kWF8Block, 2>(a, max_items, s) : launch_t<T, kWF8Block, 1>(a, max_items, s);
+    default:
+        return stage == 1 ? launch_t<T, kW16, 2>(a, max_items, s) : launch_t<T, kW16, 1>(a, max_items, s);
+    }
+}
+
+hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, int wmode,
                            const int64_t max_items[kNumLists], hipStream_t s)
 {
-    if (act == 0) {
-        if (w8) return stage == 1 ? launch_t<__bf16, true, 2>(a, max_items, s)
-                                  : launch_t<__bf16, true, 1>(a, max_items, s);
-        return stage == 1 ? launch_t<__bf16, false, 2>(a, max_items, s)
-                          : launch_t<__bf16, false, 1>(a, max_items, s);
-    }
-    if (w8) return stage == 1 ? launch_t<_Float16, true, 2>(a, max_items, s)
-                              : launch_t<_Float16, true, 1>(a, max_items, s);
-    return stage == 1 ? launch_t<_Float16, false, 2>(a, max_items, s)
-                      : launch_t<_Float16, false, 1>(a, max_items, s);
+    return act == 0 ? launch_w<__bf16>(a, stage, wmode, max_items, s) : launch_w<_Float16>(a, stage, wmode, max_items, s);
 }
 
 }  // namespace ek

@@ -20,12 +20,19 @@ namespace ek {
 // dequantisation fma.
 constexpr int kChunkBytes = 1024;
 
+// How a layer keeps its weights in HBM.
+enum WeightMode {
+    kW16 = 0,        // the activation type (bf16 / fp16): 32 contraction elements per 1 KiB chunk
+    kWI8 = 1,        // int8, offset-binary, one fp32 scale per output channel: 64 per chunk
+    kWF8Block = 2    // fp8 e4m3fn, one fp32 scale per 128 x 128 block: 64 per chunk
+};
+
 struct ExpertSlab {           // device addresses of one expert's tensors
     const uint8_t *upgate;    // matrix group {up, gate}: N = I, K = H
     const uint8_t *down;      // matrix group {down}:     N = H, K = I
-    const float *s_up;        // [I] fp32 scales (int8 only, else nullptr)
-    const float *s_gate;      // [I]
-    const float *s_down;      // [H]
+    const float *s_up;        // fp32 scales: [I] per channel (kWI8), [ceil(I/128), ceil(H/128)] per block
+    const float *s_gate;      //   (kWF8Block), nullptr for 16-bit weights; same shape as s_up
+    const float *s_down;      // [H] per channel, [ceil(H/128), ceil(I/128)] per block
 };
 
 // ---- work lists ---------------------------------------------------------------
@@ -132,14 +139,14 @@ struct FfnArgs {
     WorkLists lists;          // device work lists and their lengths
 };
 // stage = 1: up/gate + SwiGLU epilogue;  stage = 2: down projection
-// act: 0 bf16, 1 f16;  w8: int8 weights with per-channel scales
+// act: 0 bf16, 1 f16;  wmode: WeightMode
 // weight-streaming kernel over lists.items[kListStream]; max_items = grid bound;
 // wide: items hold up to kWideRows rows (else up to 16)
-hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, bool w8, int64_t max_items, bool wide,
+hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, int wmode, int64_t max_items, bool wide,
                              hipStream_t s);
 // MFMA tile kernel over the three tile lists (128-row items first, then 64,
 // then 32); max_items[l] bounds list l
-hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, bool w8,
+hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, int wmode,
                            const int64_t max_items[kNumLists], hipStream_t s);
 
 // ---- combine ----------------------------------------------------------------

@@ -89,6 +89,24 @@ __device__ __forceinline__ typename Act<T>::V8 dequant_u8x8(uint32_t lo, uint32_
     return __builtin_bit_cast(typename Act<T>::V8, r);
 }
 
+// The same for OCP fp8 (e4m3fn) bytes with a block scale: rne_T(f32(b) * s), the arithmetic of
+// the reference's w8a16_activate (ek-computation/src/ffn/expert_torch.rs:24-53).
+// v_cvt_f32_fp8 converts one selected byte exactly (checked for all 256 values on gfx950).
+template <typename T> __device__ __forceinline__ u32x2 dequant_f8x4(uint32_t w, float s)
+{
+    u32x2 r;
+    r[0] = pack2<T>(__builtin_amdgcn_cvt_f32_fp8(w, 0) * s, __builtin_amdgcn_cvt_f32_fp8(w, 1) * s);
+    r[1] = pack2<T>(__builtin_amdgcn_cvt_f32_fp8(w, 2) * s, __builtin_amdgcn_cvt_f32_fp8(w, 3) * s);
+    return r;
+}
+template <typename T>
+__device__ __forceinline__ typename Act<T>::V8 dequant_f8x8(uint32_t lo, uint32_t hi, float s)
+{
+    const u32x2 a = dequant_f8x4<T>(lo, s), b = dequant_f8x4<T>(hi, s);
+    const u32x4 r = {a[0], a[1], b[0], b[1]};
+    return __builtin_bit_cast(typename Act<T>::V8, r);
+}
+
 // SwiGLU with the reference's storage roundings: up, gate, silu(gate) and the
 // product are each a materialised tensor of the activation dtype
 // (ek-computation/src/ffn/expert_torch.rs:81-83).

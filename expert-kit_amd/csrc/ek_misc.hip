@@ -111,8 +111,9 @@ __global__ __launch_bounds__(256) void tile_weights16_kernel(const void *src, in
     *(V8 *)(dst + (chunk * nmat + m) * kChunkBytes + l * 16) = v;
 }
 
+// flip: int8 is stored offset-binary (q ^ 0x80, see dequant_u8x4); fp8 bytes are kept as they are
 __global__ __launch_bounds__(256) void tile_weights8_kernel(const uint8_t *src, int64_t N, int64_t K,
-                                                           uint8_t *dst, int m, int nmat)
+                                                           uint8_t *dst, int m, int nmat, uint32_t flip)
 {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t KT = K / 64, total = (N / 16) * KT * 64;
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(256) void tile_weights8_kernel(const uint8_t *src, 
     const int64_t chunk = idx >> 6, nt = chunk / KT, kt = chunk % KT;
     const int64_t row = nt * 16 + (l & 15), col = kt * 64 + (l >> 4) * 16;
     uint4 v = *(const uint4 *)(src + row * K + col);
-    v.x ^= 0x80808080u; v.y ^= 0x80808080u; v.z ^= 0x80808080u; v.w ^= 0x80808080u;
+    v.x ^= flip; v.y ^= flip; v.z ^= flip; v.w ^= flip;
     *(uint4 *)(dst + (chunk * nmat + m) * kChunkBytes + l * 16) = v;
 }
 
@@ -129,10 +130,10 @@ void launch_tile_weights(const void *src, int src_dtype, int64_t N, int64_t K, u
                          int dst_dtype, int m, int nmat, const void *block_scale, int scale_dtype,
                          hipStream_t s)
 {
-    if (dst_dtype == 3) {
+    if (dst_dtype == 3 || dst_dtype == 4) {      // EK_I8, EK_F8E4M3: one byte per weight, kept as stored
         const int64_t total = (N / 16) * (K / 64) * 64;
         hipLaunchKernelGGL(tile_weights8_kernel, dim3((total + 255) / 256), dim3(256), 0, s,
-                           (const uint8_t *)src, N, K, dst, m, nmat);
+                           (const uint8_t *)src, N, K, dst, m, nmat, dst_dtype == 3 ? 0x80808080u : 0u);
     } else {
         const int64_t total = (N / 16) * (K / 32) * 64;
         if (dst_dtype == 0)

@@ -1,0 +1,134 @@
+"""Layers that keep fp8 (e4m3fn) weights with 128x128 block scales as the checkpoint stores them.
+
+The arithmetic is the reference's w8a16_activate (ek-computation/src/ffn/expert_torch.rs:24-53):
+W[r,c] = rne_16bit(f32(fp8[r,c]) * scale[r/128, c/128]), here applied in registers by both
+kernel families instead of once at load.  Bars: the FFN / layer gates of test_gpu_parity.py
+against the oracle fed with weights dequantised that way on the CPU; the fp8 bytes cover all
+254 finite encodings.
+"""
+import pytest
+import torch
+from safetensors.torch import save as st_save
+
+from test_gpu_parity import check_vs_rounded, ffn_gate, layer_gate
+
+pytestmark = pytest.mark.gpu
+F8 = torch.float8_e4m3fn
+
+
+def fp8_matrix(r, c, g):
+    """Shaped like a quantised checkpoint block (a Gaussian scaled so that its tail reaches the
+    format's 448), with every finite e4m3fn byte planted at a few random places."""
+    w = (torch.randn(r, c, generator=g) * 110).clamp(-448, 448).to(F8).view(torch.uint8).flatten()
+    codes = torch.tensor([b for b in range(256) if (b & 0x7f) != 0x7f], dtype=torch.uint8).repeat(3)
+    w[torch.randperm(r * c, generator=g)[:codes.numel()]] = codes
+    return w.view(r, c).view(F8)
+
+
+def block_scales(r, c, g):
+    return torch.rand((r + 127) // 128, (c + 127) // 128, generator=g) * 3e-4 + 5e-5
+
+
+def dequant(w, sc, dt):
+    full = sc.repeat_interleave(128, 0)[:w.shape[0]].repeat_interleave(128, 1)[:, :w.shape[1]]
+    return (w.float() * full).to(dt)
+
+
+def make_expert(ek, H, I, seed):
+    g = torch.Generator().manual_seed(seed)
+    return ek.ExpertWeight(up_w=fp8_matrix(I, H, g), gate_w=fp8_matrix(I, H, g), down_w=fp8_matrix(H, I, g),
+                           up_scale=block_scales(I, H, g), gate_scale=block_scales(I, H, g),
+                           down_scale=block_scales(H, I, g))
+
+
+def ref_weights(ew, dt):
+    return (dequant(ew.up_w, ew.up_scale, dt), dequant(ew.gate_w, ew.gate_scale, dt), dequant(ew.down_w, ew.down_scale, dt))
+
+
+def test_all_finite_encodings_are_drawn():
+    g = torch.Generator().manual_seed(1)
+    seen = set(fp8_matrix(64, 64, g).view(torch.uint8).flatten().tolist())
+    assert len(seen) == 254 and 0x7f not in seen and 0xff not in seen
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [1, 7, 16, 17, 40, 64, 65, 200])
+def test_one_expert_streamed(ek, oracle, cuda, dt, n):
+    """A lone per-expert call: the sliced streaming form (n <= 16) and its 64-row form."""
+    H, I = 384, 256
+    print(f"fp8 expert dt={dt} n={n}", flush=True)
+    layer = ek.HipLayer(H, I, 2, 1, act_dtype=dt, w_dtype=F8, max_tokens=256)
+    ew = make_expert(ek, H, I, 11)
+    layer.set_expert(1, ew)
+    x = torch.randn(n, H, generator=torch.Generator().manual_seed(n)).to(dt)
+    ref = oracle.ffn(x, *ref_weights(ew, dt), mode=2)
+    got = layer.expert_forward(1, x.to(cuda))
+    ffn_gate(got, ref, f"fp8 expert dt={dt} n={n}")
+    assert check_vs_rounded(got, ref) > 0.9
+    assert torch.equal(layer.expert_forward(1, x).view(torch.int16), got.cpu().view(torch.int16))   # host rows
+    layer.close()
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,K,H,I", [(24, 8, 2, 384, 256), (300, 6, 2, 512, 384), (700, 4, 1, 256, 640)])
+def test_layer_both_kernel_families(ek, oracle, cuda, dt, T, E, K, H, I):
+    """Whole layer calls whose segments span the streaming kernel (<= 16 rows) and 32-, 64- and
+    128-row tiles; routing skewed so that one expert is hot and one is never used."""
+    print(f"fp8 layer dt={dt} T={T} E={E} K={K} H={H} I={I}", flush=True)
+    g = torch.Generator().manual_seed(T + E)
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=F8, max_tokens=T)
+    ws = [make_expert(ek, H, I, 100 + e) for e in range(E)]
+    for e in range(E - 1):                       # the last expert stays unloaded and unused
+        layer.set_expert(e, ws[e])
+    p = torch.tensor([8.0] + [1.0] * (E - 3) + [0.05, 0.0])
+    ids = torch.stack([torch.multinomial(p, K, generator=g) for _ in range(T)]).to(torch.int32)
+    gw = torch.rand(T, K, generator=g) + 0.1
+    gw = (gw / gw.sum(-1, keepdim=True)).to(dt)
+    x = torch.randn(T, H, generator=g).to(dt)
+    wu, wg, wd = zip(*[ref_weights(w, dt) for w in ws])
+    ref, counts, offsets, perm, inv, y3 = oracle.layer_forward(x, ids, gw, list(wu), list(wg), list(wd), mode=2,
+                                                             return_y3=True)
+    y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
+    assert torch.equal(rt.perm.cpu(), perm) and torch.equal(rt.counts.cpu(), counts)
+    sizes = sorted(set(int(c) for c in counts))
+    print("   segment lengths:", sizes, flush=True)
+    layer_gate(y, ref, y3, gw, f"fp8 layer T={T}")
+    layer.close()
+
+
+def test_batch_of_small_calls_and_blob_ingestion(ek, oracle, cuda):
+    """Many <= 16-row calls in one launch (the one-wave-per-channel-group streaming form) and
+    experts loaded from the bytes ek-db serves (fp8 tensors with weight_scale_inv beside them)."""
+    dt, H, I, E = torch.bfloat16, 384, 256, 256
+    layer = ek.HipLayer(H, I, E, 1, act_dtype=dt, w_dtype=F8, max_tokens=4096)
+    ew = make_expert(ek, H, I, 5)
+    blob = st_save({"model.layers.3.mlp.experts.0.up_proj.weight": ew.up_w,
+                    "model.layers.3.mlp.experts.0.up_proj.weight_scale_inv": ew.up_scale,
+                    "model.layers.3.mlp.experts.0.gate_proj.weight": ew.gate_w,
+                    "model.layers.3.mlp.experts.0.gate_proj.weight_scale_inv": ew.gate_scale,
+                    "model.layers.3.mlp.experts.0.down_proj.weight": ew.down_w,
+                    "model.layers.3.mlp.experts.0.down_proj.weight_scale_inv": ew.down_scale})
+    layer.set_expert_safetensors(0, blob)
+    x = torch.randn(16 * 200, H, generator=torch.Generator().manual_seed(9)).to(dt)
+    outs = torch.cat(layer.experts_forward([0] * 200, list(x.to(cuda).split(16))))
+    ref = oracle.ffn(x, *ref_weights(ew, dt), mode=2)
+    ffn_gate(outs, ref, "fp8 batch of 200 calls")
+    one = layer.expert_forward(0, x[32:48].to(cuda))                    # the same rows alone: same bits
+    assert torch.equal(one.view(torch.int16), outs[32:48].view(torch.int16))
+    layer.close()
+
+
+def test_fp8_layer_rejects_other_weights(ek):
+    layer = ek.HipLayer(256, 128, 2, 1, w_dtype=F8, max_tokens=8)
+    bf = ek.ExpertWeight.from_rand_linear(256, 128, torch.bfloat16)
+    with pytest.raises(ek.EKError) as ei:
+        layer.set_expert(0, bf)
+    assert ei.value.status == ek.EK_INVALID_INPUT
+    ew = make_expert(ek, 256, 128, 3)
+    ew.up_scale = None
+    with pytest.raises(ek.EKError):
+        layer.set_expert(0, ew)
+    layer.close()
+    with pytest.raises(ek.EKError) as ei:
+        ek.HipLayer(16384, 128, 2, 1, w_dtype=F8, max_tokens=8)
+    assert ei.value.status == ek.EK_INVALID_INPUT
