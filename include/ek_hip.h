@@ -53,7 +53,8 @@ typedef enum ek_dtype {
     EK_F16 = 1,
     EK_F32 = 2,
     EK_I8 = 3,
-    EK_F8E4M3 = 4 /* OCP e4m3fn, DType::Float8e4m3fn (backend/mod.rs:13); load-time source type only */
+    EK_F8E4M3 = 4 /* OCP e4m3fn, DType::Float8e4m3fn (backend/mod.rs:13): a source type of
+                     block-scaled tensors, and the type an fp8 layer keeps them in (ek_cfg.w_dtype) */
 } ek_dtype;
 
 typedef enum ek_mem { EK_HOST = 0, EK_DEVICE = 1 } ek_mem;
@@ -64,8 +65,10 @@ typedef enum ek_scale_kind {
     /* one scale per 128x128 block, scale [ceil(rows/128), ceil(cols/128)] (the
      * `weight_scale_inv` tensors of DeepSeek Block-INT8 / FP8 checkpoints).  The weights are
      * dequantised once at load to the layer's 16-bit type, exactly as w8a16_activate does
-     * (ffn/expert_torch.rs:24-53): W[r,c] = rne(f32(q[r,c]) * s[r/128, c/128]); the layer's
-     * w_dtype must be its act_dtype. */
+     * (ffn/expert_torch.rs:24-53): W[r,c] = rne(f32(q[r,c]) * s[r/128, c/128]) -- for a layer
+     * whose w_dtype is its act_dtype.  A layer whose w_dtype is EK_F8E4M3 takes EK_F8E4M3
+     * tensors with these scales only, keeps both as they are and applies the same formula in
+     * the kernels. */
     EK_SCALE_BLOCK128 = 2
 } ek_scale_kind;
 
@@ -77,7 +80,11 @@ typedef struct ek_cfg {
     int32_t n_experts;  /* E  experts owned by one layer object */
     int32_t top_k;      /* K  slots per token */
     int32_t act_dtype;  /* ek_dtype of x, y and the gate weights: EK_BF16 or EK_F16 */
-    int32_t w_dtype;    /* ek_dtype weights are kept in: act_dtype, or EK_I8 (W8A16) */
+    int32_t w_dtype;    /* ek_dtype weights are kept in: act_dtype; EK_I8 (W8A16, one scale per
+                           output channel); or EK_F8E4M3: the checkpoint's fp8 bytes with their
+                           128x128 block scales, dequantised in the kernels with the arithmetic
+                           of w8a16_activate (ffn/expert_torch.rs:24-53) -- half the HBM bytes of
+                           dequantising at load; hidden, inter <= 8192 */
     int64_t max_tokens; /* largest T a forward call will pass */
     int32_t device_id;  /* HIP device ordinal */
     int32_t flags;      /* reserved, 0 */
