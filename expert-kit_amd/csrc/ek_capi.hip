@@ -207,8 +207,11 @@ ek_status validate_cfg(const ek_cfg *c)
         return fail(EK_INVALID_INPUT, "act_dtype must be EK_BF16 or EK_F16 (got %d)", c->act_dtype);
     if (c->w_dtype != c->act_dtype && c->w_dtype != EK_I8 && c->w_dtype != EK_F8E4M3)
         return fail(EK_INVALID_INPUT, "w_dtype must equal act_dtype or be EK_I8 or EK_F8E4M3 (got %d)", c->w_dtype);
-    if (c->w_dtype == EK_F8E4M3 && (c->hidden > 8192 || c->inter > 8192))
-        return fail(EK_INVALID_INPUT, "fp8 block-scaled layers hold at most 64 scale blocks per row: hidden and "
+    if (c->flags & ~EK_CFG_BLOCK_SCALES) return fail(EK_INVALID_INPUT, "unknown flags 0x%x", c->flags);
+    if ((c->flags & EK_CFG_BLOCK_SCALES) && c->w_dtype != EK_I8 && c->w_dtype != EK_F8E4M3)
+        return fail(EK_INVALID_INPUT, "EK_CFG_BLOCK_SCALES needs w_dtype EK_I8 or EK_F8E4M3");
+    if ((c->w_dtype == EK_F8E4M3 || (c->flags & EK_CFG_BLOCK_SCALES)) && (c->hidden > 8192 || c->inter > 8192))
+        return fail(EK_INVALID_INPUT, "block-scaled layers hold at most 64 scale blocks per row: hidden and "
                     "inter must not exceed 8192");
     const int64_t ke = 64;   // contraction step of the tile kernel; int8 chunk width
     // the tile kernel's pipeline needs two contraction steps (64 wide for int8, 32 for 16-bit)
@@ -239,7 +242,8 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     L->cfg = *cfg;
     L->act = cfg->act_dtype == EK_BF16 ? 0 : 1;
     L->w8 = cfg->w_dtype == EK_I8 || cfg->w_dtype == EK_F8E4M3;
-    L->wmode = cfg->w_dtype == EK_I8 ? ek::kWI8 : cfg->w_dtype == EK_F8E4M3 ? ek::kWF8Block : ek::kW16;
+    L->wmode = cfg->w_dtype == EK_I8 ? ((cfg->flags & EK_CFG_BLOCK_SCALES) ? ek::kWI8Block : ek::kWI8)
+               : cfg->w_dtype == EK_F8E4M3 ? ek::kWF8Block : ek::kW16;
     L->Pmax = pmax;
     const int E = cfg->n_experts;
     // slot E of the tables is the shared expert; its segment (one row per token) follows the
@@ -316,12 +320,13 @@ ek_status check_desc(const ek_weight_desc *d, const char *name, int64_t rows, in
                     (long long)d->rows, (long long)d->cols, (long long)rows, (long long)cols);
     if (d->mem != EK_HOST && d->mem != EK_DEVICE)
         return fail(EK_INVALID_INPUT, "%s weight: bad mem %d", name, d->mem);
-    if (wmode == ek::kWF8Block) {
-        // kept as stored: fp8 bytes and the checkpoint's 128 x 128 scale blocks
-        if (d->dtype != EK_F8E4M3)
-            return fail(EK_INVALID_INPUT, "%s weight must be EK_F8E4M3 for an fp8 layer (got %d)", name, d->dtype);
+    if (ek::block_scaled(wmode)) {
+        // kept as stored: the checkpoint's bytes and its 128 x 128 scale blocks
+        const int want = wmode == ek::kWF8Block ? EK_F8E4M3 : EK_I8;
+        if (d->dtype != want)
+            return fail(EK_INVALID_INPUT, "%s weight must be of the layer's w_dtype %d (got %d)", name, want, d->dtype);
         if (d->scale_kind != EK_SCALE_BLOCK128)
-            return fail(EK_INVALID_INPUT, "%s weight: fp8 needs EK_SCALE_BLOCK128", name);
+            return fail(EK_INVALID_INPUT, "%s weight: a block-scaled layer needs EK_SCALE_BLOCK128", name);
         if (!d->scale) return fail(EK_WEIGHT_NOT_FOUND, "%s block scale is missing", name);
         if (d->scale_dtype != EK_BF16 && d->scale_dtype != EK_F32 && d->scale_dtype != EK_F16)
             return fail(EK_INVALID_INPUT, "%s scale: bad dtype %d", name, d->scale_dtype);
@@ -382,7 +387,7 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
     EK_TRY(check_desc(down, "down", H, I, L->wmode));
     const size_t wsz = L->w8 ? 1 : 2;
     const size_t mat_bytes = (size_t)H * I * wsz;
-    const bool blocks = L->wmode == ek::kWF8Block;
+    const bool blocks = ek::block_scaled(L->wmode);
     // scales kept beside the weights: one per output channel (int8) or per 128 x 128 block (fp8)
     const size_t nb_ih = (size_t)((I + 127) / 128) * (size_t)((H + 127) / 128);
     const size_t s_upgate = blocks ? nb_ih : (size_t)I, s_dn = blocks ? nb_ih : (size_t)H;

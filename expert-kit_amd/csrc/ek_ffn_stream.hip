@@ -94,9 +94,9 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
     // Block scales: the wave's 16 channels lie in one 128-row block, so the scale of a chunk is
     // one number per 128 contraction elements: the wave keeps its rows of the scale matrices in
     // LDS (lane b holds block b) and reads one back per chunk.
-    __shared__ float srow[WM == kWF8Block ? (SK == 1 ? 4 : kSlices) : 1][WM == kWF8Block ? NW : 1]
-                         [WM == kWF8Block ? kMaxScaleBlocks : 1];
-    if constexpr (WM == kWF8Block) {
+    __shared__ float srow[block_scaled(WM) ? (SK == 1 ? 4 : kSlices) : 1][block_scaled(WM) ? NW : 1]
+                         [block_scaled(WM) ? kMaxScaleBlocks : 1];
+    if constexpr (block_scaled(WM)) {
         const int KB = (a.Kdim + 127) >> 7;
 #pragma unroll
         for (int gi = 0; gi < NG; ++gi)
@@ -172,10 +172,14 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
                             const float sv = ws[gi * NMAT + m], cv = wc[gi * NMAT + m];
                             w0 = dequant_u8x8<T>(q.x, q.y, sv, cv);
                             w1 = dequant_u8x8<T>(q.z, q.w, sv, cv);
-                        } else {
+                        } else if constexpr (WM == kWF8Block) {
                             const float sv = srow[wave][gi * NMAT + m][kt >> 1];
                             w0 = dequant_f8x8<T>(q.x, q.y, sv);
                             w1 = dequant_f8x8<T>(q.z, q.w, sv);
+                        } else {
+                            const float sv = srow[wave][gi * NMAT + m][kt >> 1], cv = -128.f * sv;
+                            w0 = dequant_u8x8<T>(q.x, q.y, sv, cv);
+                            w1 = dequant_u8x8<T>(q.z, q.w, sv, cv);
                         }
 #pragma unroll
                         for (int rs = 0; rs < RS; ++rs)
@@ -324,6 +328,9 @@ static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, int32_t n_seg
     case kWF8Block:
         return stage == 1 ? launch_g<T, kWF8Block, 2>(a, n_segments, wide, s)
                           : launch_g<T, kWF8Block, 1>(a, n_segments, wide, s);
+    case kWI8Block:
+        return stage == 1 ? launch_g<T, kWI8Block, 2>(a, n_segments, wide, s)
+                          : launch_g<T, kWI8Block, 1>(a, n_segments, wide, s);
     default:
         return stage == 1 ? launch_g<T, kW16, 2>(a, n_segments, wide, s) : launch_g<T, kW16, 1>(a, n_segments, wide, s);
     }

@@ -167,7 +167,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 
     // Fills `c` for the first tile at or after index t (stepping by stride) whose expert is
     // loaded; returns its index or -1.
-    // block scales (fp8 weights): the wave's 32-channel column blocks lie in one 128-row block
+    // block scales: the wave's 32-channel column blocks lie in one 128-row block
     // each, so a step's scale is one number per column block; the tile's rows of the scale
     // matrices sit in a wave-private LDS area (two areas: the next tile's rows are fetched while
     // this one's are in use)
@@ -199,7 +199,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                 }
                 c.as[cb] = sv;
                 c.ac[cb] = -128.f * sv;
-                if constexpr (WM == kWF8Block) {
+                if constexpr (block_scaled(WM)) {
                     const int KB = (a.Kdim + 127) >> 7;
                     const int ct = min(cblock * NR + (NMAT == 2 ? 0 : cb * 2), NT - 1);
                     const float *smat = NMAT == 2 ? (cb == 0 ? slab.s_up : slab.s_gate) : slab.s_down;
@@ -208,7 +208,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                 }
             }
             c.sslot = sslot;
-            if constexpr (WM == kWF8Block) {
+            if constexpr (block_scaled(WM)) {
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
             }
@@ -290,13 +290,14 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
             float sblk[CB] = {};        // block-scaled weights: this step's scale per column block
-            if constexpr (WM == kWF8Block) {
+            if constexpr (block_scaled(WM)) {
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
                     sblk[cb] = sc_area[cur.sslot * kScaleSlotFloats + cb * kTileScaleBlocks + (step >> 1)];
             }
             auto dq = [&](uint32_t w, int cb) -> u32x2 {
                 if constexpr (WM == kWF8Block) return dequant_f8x4<T>(w, sblk[cb]);
+                else if constexpr (WM == kWI8Block) return dequant_u8x4<T>(w, sblk[cb], -128.f * sblk[cb]);
                 else return dequant_u8x4<T>(w, cur.as[cb], cur.ac[cb]);
             };
 
@@ -438,7 +439,7 @@ template <typename T, int WM, int NMAT>
 __global__ __launch_bounds__(kTileThreads, 1) void ffn_tile_kernel(FfnArgs a, int nb_count)
 {
     __shared__ __attribute__((aligned(1024)))
-    uint8_t lds[kTileStages * TileGeom<WM != kW16>::STAGE + (WM == kWF8Block ? kTileScaleBytes : 0)];
+    uint8_t lds[kTileStages * TileGeom<WM != kW16>::STAGE + (block_scaled(WM) ? kTileScaleBytes : 0)];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)lds;
     const int x = blockIdx.x & 7, slot = blockIdx.x >> 3, nslots = gridDim.x >> 3;
     const int n128 = a.lists.count[kListT128], n64 = a.lists.count[kListT64], n32 = a.lists.count[kListT32];
@@ -477,6 +478,8 @@ static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, const int64_t
         return stage == 1 ? launch_t<T, kWI8, 2>(a, max_items, s) : launch_t<T, kWI8, 1>(a, max_items, s);
     case kWF8Block:
         return stage == 1 ? launch_t<T, kWF8Block, 2>(a, max_items, s) : launch_t<T, kWF8Block, 1>(a, max_items, s);
+    case kWI8Block:
+        return stage == 1 ? launch_t<T, kWI8Block, 2>(a, max_items, s) : launch_t<T, kWI8Block, 1>(a, max_items, s);
     default:
         return stage == 1 ? launch_t<T, kW16, 2>(a, max_items, s) : launch_t<T, kW16, 1>(a, max_items, s);
     }

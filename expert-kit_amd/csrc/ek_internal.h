@@ -24,14 +24,16 @@ constexpr int kChunkBytes = 1024;
 enum WeightMode {
     kW16 = 0,        // the activation type (bf16 / fp16): 32 contraction elements per 1 KiB chunk
     kWI8 = 1,        // int8, offset-binary, one fp32 scale per output channel: 64 per chunk
-    kWF8Block = 2    // fp8 e4m3fn, one fp32 scale per 128 x 128 block: 64 per chunk
+    kWF8Block = 2,   // fp8 e4m3fn, one fp32 scale per 128 x 128 block: 64 per chunk
+    kWI8Block = 3    // int8, offset-binary, one fp32 scale per 128 x 128 block: 64 per chunk
 };
+constexpr bool block_scaled(int wm) { return wm == kWF8Block || wm == kWI8Block; }
 
 struct ExpertSlab {           // device addresses of one expert's tensors
     const uint8_t *upgate;    // matrix group {up, gate}: N = I, K = H
     const uint8_t *down;      // matrix group {down}:     N = H, K = I
     const float *s_up;        // fp32 scales: [I] per channel (kWI8), [ceil(I/128), ceil(H/128)] per block
-    const float *s_gate;      //   (kWF8Block), nullptr for 16-bit weights; same shape as s_up
+    const float *s_gate;      //   (kWF8Block, kWI8Block), nullptr for 16-bit weights; same shape as s_up
     const float *s_down;      // [H] per channel, [ceil(H/128), ceil(I/128)] per block
 };
 

@@ -69,6 +69,7 @@ class ek_router_cfg(ctypes.Structure):
  EK_ROUTER_SIGMOID_GROUP) = range(5)
 EK_ROUTER_MASK_NEG_INF = 1
 EK_SHARED_EXPERT = -1
+EK_CFG_BLOCK_SCALES = 1
 
 _P = ctypes.c_void_p
 _PP = ctypes.POINTER(ctypes.c_void_p)

@@ -146,11 +146,15 @@ class HipLayer:
     """The experts of one MoE layer, resident in HBM, with the fused layer call."""
 
     def __init__(self, hidden: int, inter: int, n_experts: int, top_k: int, act_dtype=torch.bfloat16,
-                 w_dtype=None, max_tokens: int = 1024, device_id: int = 0):
+                 w_dtype=None, max_tokens: int = 1024, device_id: int = 0, block_scales: bool = False):
+        """w_dtype: None (= act_dtype), torch.int8 (one scale per output channel; with block_scales the
+        int8 tensors of a Block-INT8 checkpoint kept with their 128x128 scales) or torch.float8_e4m3fn
+        (an FP8 checkpoint's tensors kept with their 128x128 scales)."""
         self._lib = C.load()
         self.cfg = C.ek_cfg(hidden=hidden, inter=inter, n_experts=n_experts, top_k=top_k,
                             act_dtype=_DT[act_dtype], w_dtype=_DT[w_dtype or act_dtype],
-                            max_tokens=max_tokens, device_id=device_id, flags=0)
+                            max_tokens=max_tokens, device_id=device_id,
+                            flags=C.EK_CFG_BLOCK_SCALES if block_scales else 0)
         self.act_dtype = act_dtype
         self._h = ctypes.c_void_p()
         C.check(self._lib.ek_layer_create(ctypes.byref(self.cfg), ctypes.byref(self._h)))

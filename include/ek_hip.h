@@ -87,8 +87,11 @@ typedef struct ek_cfg {
                            dequantising at load; hidden, inter <= 8192 */
     int64_t max_tokens; /* largest T a forward call will pass */
     int32_t device_id;  /* HIP device ordinal */
-    int32_t flags;      /* reserved, 0 */
+    int32_t flags;      /* 0, or EK_CFG_BLOCK_SCALES */
 } ek_cfg;
+/* With w_dtype EK_I8: the weights are the int8 tensors of a Block-INT8 checkpoint, kept with
+ * their 128x128 block scales like the fp8 form (EK_F8E4M3 implies it). */
+#define EK_CFG_BLOCK_SCALES 1
 
 /* One weight matrix of ExpertWeight<T> (ek-computation/src/ffn/meta.rs:10-23),
  * row-major [rows = out_features, cols = in_features] as HF nn.Linear stores

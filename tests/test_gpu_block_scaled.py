@@ -1,10 +1,10 @@
-"""Layers that keep fp8 (e4m3fn) weights with 128x128 block scales as the checkpoint stores them.
+"""Layers that keep fp8 (e4m3fn) or int8 weights with 128x128 block scales as the checkpoint stores them.
 
 The arithmetic is the reference's w8a16_activate (ek-computation/src/ffn/expert_torch.rs:24-53):
 W[r,c] = rne_16bit(f32(fp8[r,c]) * scale[r/128, c/128]), here applied in registers by both
 kernel families instead of once at load.  Bars: the FFN / layer gates of test_gpu_parity.py
 against the oracle fed with weights dequantised that way on the CPU; the fp8 bytes cover all
-254 finite encodings.
+254 finite encodings, the int8 ones all 256 values.
 """
 import pytest
 import torch
@@ -34,9 +34,17 @@ def dequant(w, sc, dt):
     return (w.float() * full).to(dt)
 
 
-def make_expert(ek, H, I, seed):
+def int8_matrix(r, c, g):
+    return torch.randint(-128, 128, (r, c), generator=g, dtype=torch.int8)
+
+
+KINDS = {"fp8": dict(w_dtype=F8), "int8": dict(w_dtype=torch.int8, block_scales=True)}
+
+
+def make_expert(ek, H, I, seed, kind="fp8"):
     g = torch.Generator().manual_seed(seed)
-    return ek.ExpertWeight(up_w=fp8_matrix(I, H, g), gate_w=fp8_matrix(I, H, g), down_w=fp8_matrix(H, I, g),
+    mat = fp8_matrix if kind == "fp8" else int8_matrix
+    return ek.ExpertWeight(up_w=mat(I, H, g), gate_w=mat(I, H, g), down_w=mat(H, I, g),
                            up_scale=block_scales(I, H, g), gate_scale=block_scales(I, H, g),
                            down_scale=block_scales(H, I, g))
 
@@ -51,14 +59,15 @@ def test_all_finite_encodings_are_drawn():
     assert len(seen) == 254 and 0x7f not in seen and 0xff not in seen
 
 
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("n", [1, 7, 16, 17, 40, 64, 65, 200])
-def test_one_expert_streamed(ek, oracle, cuda, dt, n):
+def test_one_expert_streamed(ek, oracle, cuda, dt, n, kind):
     """A lone per-expert call: the sliced streaming form (n <= 16) and its 64-row form."""
     H, I = 384, 256
     print(f"fp8 expert dt={dt} n={n}", flush=True)
-    layer = ek.HipLayer(H, I, 2, 1, act_dtype=dt, w_dtype=F8, max_tokens=256)
-    ew = make_expert(ek, H, I, 11)
+    layer = ek.HipLayer(H, I, 2, 1, act_dtype=dt, max_tokens=256, **KINDS[kind])
+    ew = make_expert(ek, H, I, 11, kind)
     layer.set_expert(1, ew)
     x = torch.randn(n, H, generator=torch.Generator().manual_seed(n)).to(dt)
     ref = oracle.ffn(x, *ref_weights(ew, dt), mode=2)
@@ -69,15 +78,16 @@ def test_one_expert_streamed(ek, oracle, cuda, dt, n):
     layer.close()
 
 
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,E,K,H,I", [(24, 8, 2, 384, 256), (300, 6, 2, 512, 384), (700, 4, 1, 256, 640)])
-def test_layer_both_kernel_families(ek, oracle, cuda, dt, T, E, K, H, I):
+def test_layer_both_kernel_families(ek, oracle, cuda, dt, T, E, K, H, I, kind):
     """Whole layer calls whose segments span the streaming kernel (<= 16 rows) and 32-, 64- and
     128-row tiles; routing skewed so that one expert is hot and one is never used."""
     print(f"fp8 layer dt={dt} T={T} E={E} K={K} H={H} I={I}", flush=True)
     g = torch.Generator().manual_seed(T + E)
-    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=F8, max_tokens=T)
-    ws = [make_expert(ek, H, I, 100 + e) for e in range(E)]
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, max_tokens=T, **KINDS[kind])
+    ws = [make_expert(ek, H, I, 100 + e, kind) for e in range(E)]
     for e in range(E - 1):                       # the last expert stays unloaded and unused
         layer.set_expert(e, ws[e])
     p = torch.tensor([8.0] + [1.0] * (E - 3) + [0.05, 0.0])
@@ -96,12 +106,13 @@ def test_layer_both_kernel_families(ek, oracle, cuda, dt, T, E, K, H, I):
     layer.close()
 
 
-def test_batch_of_small_calls_and_blob_ingestion(ek, oracle, cuda):
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
+def test_batch_of_small_calls_and_blob_ingestion(ek, oracle, cuda, kind):
     """Many <= 16-row calls in one launch (the one-wave-per-channel-group streaming form) and
     experts loaded from the bytes ek-db serves (fp8 tensors with weight_scale_inv beside them)."""
     dt, H, I, E = torch.bfloat16, 384, 256, 256
-    layer = ek.HipLayer(H, I, E, 1, act_dtype=dt, w_dtype=F8, max_tokens=4096)
-    ew = make_expert(ek, H, I, 5)
+    layer = ek.HipLayer(H, I, E, 1, act_dtype=dt, max_tokens=4096, **KINDS[kind])
+    ew = make_expert(ek, H, I, 5, kind)
     blob = st_save({"model.layers.3.mlp.experts.0.up_proj.weight": ew.up_w,
                     "model.layers.3.mlp.experts.0.up_proj.weight_scale_inv": ew.up_scale,
                     "model.layers.3.mlp.experts.0.gate_proj.weight": ew.gate_w,
@@ -118,7 +129,13 @@ def test_batch_of_small_calls_and_blob_ingestion(ek, oracle, cuda):
     layer.close()
 
 
-def test_fp8_layer_rejects_other_weights(ek):
+def test_block_scaled_layer_rejects_other_weights(ek):
+    with pytest.raises(ek.EKError):
+        ek.HipLayer(256, 128, 2, 1, block_scales=True, max_tokens=8)         # needs one-byte weights
+    i8 = ek.HipLayer(256, 128, 2, 1, w_dtype=torch.int8, block_scales=True, max_tokens=8)
+    with pytest.raises(ek.EKError):
+        i8.set_expert(0, make_expert(ek, 256, 128, 3, "fp8"))
+    i8.close()
     layer = ek.HipLayer(256, 128, 2, 1, w_dtype=F8, max_tokens=8)
     bf = ek.ExpertWeight.from_rand_linear(256, 128, torch.bfloat16)
     with pytest.raises(ek.EKError) as ei:
