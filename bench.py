@@ -53,7 +53,12 @@ def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
     E = w.n_experts
     wu, wg, wd = [None] * E, [None] * E, [None] * E
     for e, ew in ws_sample.items():
-        if w.w8:
+        if w.fp8_block:
+            def blk(t, sc):     # w8a16_activate's arithmetic: fp32 product, one rounding
+                full = sc.repeat_interleave(128, 0)[:t.shape[0]].repeat_interleave(128, 1)[:, :t.shape[1]]
+                return (t.float() * full).to(w.act_dtype)
+            wu[e], wg[e], wd[e] = blk(ew.up_w, ew.up_scale), blk(ew.gate_w, ew.gate_scale), blk(ew.down_w, ew.down_scale)
+        elif w.w8:
             wu[e] = oracle.torch_dequant_channel(ew.up_w, ew.up_scale)
             wg[e] = oracle.torch_dequant_channel(ew.gate_w, ew.gate_scale)
             wd[e] = oracle.torch_dequant_channel(ew.down_w, ew.down_scale)
@@ -134,6 +139,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--weights", choices=["config", "fp8"], default="config",
+                    help="fp8: the c3 / c4 layer with fp8 e4m3fn weights and 128x128 block scales kept as a "
+                         "DeepSeek-V3 checkpoint stores them, instead of the configuration's int8 per channel")
     ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
@@ -151,10 +159,15 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     w = wl.resolve(wl.CONFIGS[args.workload])
+    if args.weights == "fp8":
+        assert w.w8, "--weights fp8 applies to the W8A16 configurations (c3, c4)"
+        from dataclasses import replace
+        w = replace(w, fp8_block=True)
     if w.n_layers > 1:
         return bench_chain(args, w, dev)
-    layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype,
-                            w_dtype=torch.int8 if w.w8 else w.act_dtype, max_tokens=w.tokens)
+    w_dtype = torch.float8_e4m3fn if w.fp8_block else torch.int8 if w.w8 else w.act_dtype
+    layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype, w_dtype=w_dtype,
+                            max_tokens=w.tokens)
     ids, gw = wl.make_routing(w)
     counts = torch.bincount(ids.reshape(-1).long(), minlength=w.n_experts)
     order = torch.argsort(counts, descending=True, stable=True).tolist()
@@ -208,8 +221,11 @@ def main():
     wsz = 1 if w.w8 else 2
     a = 2
     # algorithmic bytes of each phase (weights of active experts once, activations in/out once)
-    b_ffn1 = active * (2 * w.hidden * w.inter * wsz + (2 * w.inter * 2 if w.w8 else 0)) + w.tokens * w.hidden * a + w.pairs * w.inter * a
-    b_ffn2 = active * (w.hidden * w.inter * wsz + (w.hidden * 2 if w.w8 else 0)) + w.pairs * w.inter * a + w.pairs * w.hidden * a
+    nblk = ((w.inter + 127) // 128) * ((w.hidden + 127) // 128)
+    s_ffn1 = 2 * nblk * 4 if w.fp8_block else 2 * w.inter * 2 if w.w8 else 0      # scale bytes per expert and stage
+    s_ffn2 = nblk * 4 if w.fp8_block else w.hidden * 2 if w.w8 else 0
+    b_ffn1 = active * (2 * w.hidden * w.inter * wsz + s_ffn1) + w.tokens * w.hidden * a + w.pairs * w.inter * a
+    b_ffn2 = active * (w.hidden * w.inter * wsz + s_ffn2) + w.pairs * w.inter * a + w.pairs * w.hidden * a
     b_layer = wl.algorithmic_bytes(w, counts)
     f_layer = w.pairs * w.flops_per_pair()
     hbm_frac = b_layer / step_s / HBM_PEAK
@@ -239,7 +255,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": w.name, "hidden": w.hidden, "moe_intermediate": w.inter, "experts": w.n_experts,
                    "top_k": w.top_k, "tokens": w.tokens, "pairs": w.pairs, "active_experts": active,
-                   "zipf_s": w.zipf_s, "weights": "int8 per-channel" if w.w8 else "16-bit"},
+                   "zipf_s": w.zipf_s, "weights": "fp8 e4m3fn, 128x128 block scales" if w.fp8_block else "int8 per-channel" if w.w8 else "16-bit"},
         "roofline": roof,
         "layer": {"algorithmic_bytes": b_layer, "algorithmic_flops": f_layer, "hbm_frac": hbm_frac,
                   "mfma_frac": mfma_frac,

@@ -31,6 +31,7 @@ class Workload:
     zipf_s: float = 0.0           # hot-expert bias b_e = -s * ln(rank_e)
     n_layers: int = 1
     ragged: bool = False          # tokens come from a continuous-batching request mix
+    fp8_block: bool = False       # with w8: fp8 e4m3fn weights + fp32 scales per 128x128 block, kept as stored
 
     @property
     def pairs(self) -> int:
@@ -39,6 +40,8 @@ class Workload:
     def expert_weight_bytes(self) -> int:
         wsz = 1 if self.w8 else 2
         scales = (2 * self.inter + self.hidden) * 2 if self.w8 else 0
+        if self.fp8_block:
+            scales = 3 * ((self.inter + 127) // 128) * ((self.hidden + 127) // 128) * 4
         return 3 * self.hidden * self.inter * wsz + scales
 
     def flops_per_pair(self) -> int:
@@ -106,6 +109,15 @@ def make_expert(w: Workload, e: int, layer: int = 0, device: str = "cpu", std: f
     seed = (1000 + layer) * 1_000_003 + e
     g = torch.Generator(device=device).manual_seed(seed)
     H, I = w.hidden, w.inter
+    if w.fp8_block:
+        def f8(r, c):       # a Gaussian scaled so that its tail reaches the format's 448, like a quantised block
+            return (torch.randn(r, c, generator=g, device=device) * 110).clamp(-448, 448).to(torch.float8_e4m3fn)
+
+        def sb(r, c):
+            return torch.rand((r + 127) // 128, (c + 127) // 128, generator=g, device=device) * 3e-4 + 5e-5
+
+        return ExpertWeight(up_w=f8(I, H), gate_w=f8(I, H), down_w=f8(H, I), up_scale=sb(I, H), gate_scale=sb(I, H),
+                            down_scale=sb(H, I))
     if w.w8:
         def q(r, c):
             return torch.randint(-127, 128, (r, c), generator=g, device=device, dtype=torch.int8)
