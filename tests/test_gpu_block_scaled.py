@@ -149,3 +149,42 @@ def test_block_scaled_layer_rejects_other_weights(ek):
     with pytest.raises(ek.EKError) as ei:
         ek.HipLayer(16384, 128, 2, 1, w_dtype=F8, max_tokens=8)
     assert ei.value.status == ek.EK_INVALID_INPUT
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8", "int8 per channel"])
+def test_every_weight_byte_is_converted_exactly(ek, cuda, kind):
+    """Reads the kernels' weight conversion back bit for bit.  With one-hot activation rows,
+    gate weights of 64 (silu(64) = 64 in fp32 and in 16 bits), an identity down projection and
+    unit scales, out[k, j] = 64 * up[j, k] with no rounding anywhere, so every one of the 256
+    byte values planted in `up` must come back as the value its format assigns to it -- through
+    the streaming kernel (16-row calls, a 128-row call) and through the tile kernel (a layer
+    call that routes every token to the expert)."""
+    n = 128
+    codes = torch.arange(n * n, dtype=torch.int32).remainder(256).reshape(n, n).roll(3, 1).to(torch.uint8)
+    if kind == "fp8":
+        codes = torch.where((codes & 0x7f) == 0x7f, torch.zeros_like(codes), codes)     # the two NaN encodings
+        up = codes.view(F8)
+        sign, e, m = (codes >> 7).float(), ((codes >> 3) & 15).float(), (codes & 7).float()
+        want = torch.where(e == 0, m / 8 * 2.0 ** -6, (1 + m / 8) * torch.exp2(e - 7)) * (1 - 2 * sign)   # OCP e4m3fn
+        mk = lambda v: torch.full((n, n), v).to(F8)
+        eye = torch.eye(n).to(F8)
+    else:
+        up = codes.view(torch.int8)
+        want = up.float()
+        mk = lambda v: torch.full((n, n), int(v), dtype=torch.int8)
+        eye = torch.eye(n).to(torch.int8)
+    ones = torch.ones(n) if kind == "int8 per channel" else torch.ones(1, 1)
+    ew = ek.ExpertWeight(up_w=up, gate_w=mk(64.0), down_w=eye, up_scale=ones, gate_scale=ones, down_scale=ones)
+    layer = ek.HipLayer(n, n, 2, 1, max_tokens=n, **KINDS.get(kind, dict(w_dtype=torch.int8)))
+    layer.set_expert(1, ew)
+    x = torch.eye(n).to(torch.bfloat16).to(cuda)
+    expect = (64 * want.t() + 0.0).to(torch.bfloat16).view(torch.int16)      # exact: at most 8 significant bits;
+                                                                             # a sum that starts at +0 turns -0 into +0
+    got = {"128-row call": layer.expert_forward(1, x),
+           "16-row calls": torch.cat(layer.experts_forward([1] * 8, list(x.split(16)))),
+           "layer call": layer.forward(x, torch.ones(n, 1, dtype=torch.int32, device=cuda),
+                                       torch.ones(n, 1, dtype=torch.bfloat16, device=cuda))}
+    for name, y in got.items():
+        bad = (y.cpu().view(torch.int16) != expect).nonzero()
+        assert bad.numel() == 0, (name, bad[:5].tolist())
+    layer.close()
