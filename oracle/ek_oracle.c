@@ -406,6 +406,25 @@ void eko_dequant_block(const float *q, const float *s, int64_t N, int64_t C, int
             w_bf16[r * C + c] = f32_to_bf16(q[r * C + c] * s[(r / B) * sc + (c / B)]);
 }
 
+/*
+ * OCP fp8 e4m3fn -> fp32: the element type of DeepSeek FP8 checkpoint tensors,
+ * DType::Float8e4m3fn of the reference (ek-computation/src/backend/mod.rs:13), which
+ * w8a16_activate converts with to_kind(Float) before scaling (expert_torch.rs:39).
+ * 1 sign, 4 exponent (bias 7), 3 mantissa bits; no infinities; 0x7f / 0xff are NaN;
+ * exponent 0 holds subnormals m/8 * 2^-6.
+ */
+void eko_fp8_e4m3fn_to_f32(const uint8_t *b, int64_t n, float *out)
+{
+    for (int64_t i = 0; i < n; ++i) {
+        const int s = b[i] >> 7, e = (b[i] >> 3) & 15, m = b[i] & 7;
+        float v;
+        if (e == 15 && m == 7) v = NAN;
+        else if (e == 0) v = ldexpf((float)m, -9);
+        else v = ldexpf((float)(8 + m), e - 10);
+        out[i] = s ? -v : v;
+    }
+}
+
 /* ------------------------------------------------------------------- FFN */
 
 static inline double silu_d(double v) { return v / (1.0 + exp(-v)); }

@@ -168,6 +168,14 @@ def dequant_block(q: torch.Tensor, s: torch.Tensor, block: int = 128) -> torch.T
     return w
 
 
+def fp8_e4m3fn_to_f32(b: torch.Tensor) -> torch.Tensor:
+    """Bytes of an fp8 e4m3fn tensor (uint8 or float8_e4m3fn) -> fp32 values (backend/mod.rs:13)."""
+    raw = b.contiguous().view(torch.uint8)
+    out = torch.empty(raw.shape, dtype=torch.float32)
+    lib().eko_fp8_e4m3fn_to_f32(_p(raw), _i64(raw.numel()), _p(out))
+    return out
+
+
 def ffn(x, w_up, w_gate, w_down, mode: int = 0, return_h: bool = False):
     """One expert SwiGLU FFN (ffn/expert_torch.rs:80-85).
 

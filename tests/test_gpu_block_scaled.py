@@ -29,9 +29,14 @@ def block_scales(r, c, g):
     return torch.rand((r + 127) // 128, (c + 127) // 128, generator=g) * 3e-4 + 5e-5
 
 
-def dequant(w, sc, dt):
+def dequant(oracle, w, sc, dt):
+    """The oracle's w8a16_activate: its own fp8 widening, its block dequantisation for bf16; the
+    fp16 layer's form (same product, rounded to fp16) written out."""
+    wf = oracle.fp8_e4m3fn_to_f32(w) if w.dtype == F8 else w.float()
+    if dt == torch.bfloat16:
+        return oracle.dequant_block(wf, sc)
     full = sc.repeat_interleave(128, 0)[:w.shape[0]].repeat_interleave(128, 1)[:, :w.shape[1]]
-    return (w.float() * full).to(dt)
+    return (wf * full).to(dt)
 
 
 def int8_matrix(r, c, g):
@@ -49,8 +54,9 @@ def make_expert(ek, H, I, seed, kind="fp8"):
                            down_scale=block_scales(H, I, g))
 
 
-def ref_weights(ew, dt):
-    return (dequant(ew.up_w, ew.up_scale, dt), dequant(ew.gate_w, ew.gate_scale, dt), dequant(ew.down_w, ew.down_scale, dt))
+def ref_weights(oracle, ew, dt):
+    return (dequant(oracle, ew.up_w, ew.up_scale, dt), dequant(oracle, ew.gate_w, ew.gate_scale, dt),
+            dequant(oracle, ew.down_w, ew.down_scale, dt))
 
 
 def test_all_finite_encodings_are_drawn():
@@ -70,7 +76,7 @@ def test_one_expert_streamed(ek, oracle, cuda, dt, n, kind):
     ew = make_expert(ek, H, I, 11, kind)
     layer.set_expert(1, ew)
     x = torch.randn(n, H, generator=torch.Generator().manual_seed(n)).to(dt)
-    ref = oracle.ffn(x, *ref_weights(ew, dt), mode=2)
+    ref = oracle.ffn(x, *ref_weights(oracle, ew, dt), mode=2)
     got = layer.expert_forward(1, x.to(cuda))
     ffn_gate(got, ref, f"fp8 expert dt={dt} n={n}")
     assert check_vs_rounded(got, ref) > 0.9
@@ -95,7 +101,7 @@ def test_layer_both_kernel_families(ek, oracle, cuda, dt, T, E, K, H, I, kind):
     gw = torch.rand(T, K, generator=g) + 0.1
     gw = (gw / gw.sum(-1, keepdim=True)).to(dt)
     x = torch.randn(T, H, generator=g).to(dt)
-    wu, wg, wd = zip(*[ref_weights(w, dt) for w in ws])
+    wu, wg, wd = zip(*[ref_weights(oracle, w, dt) for w in ws])
     ref, counts, offsets, perm, inv, y3 = oracle.layer_forward(x, ids, gw, list(wu), list(wg), list(wd), mode=2,
                                                              return_y3=True)
     y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
@@ -122,7 +128,7 @@ def test_batch_of_small_calls_and_blob_ingestion(ek, oracle, cuda, kind):
     layer.set_expert_safetensors(0, blob)
     x = torch.randn(16 * 200, H, generator=torch.Generator().manual_seed(9)).to(dt)
     outs = torch.cat(layer.experts_forward([0] * 200, list(x.to(cuda).split(16))))
-    ref = oracle.ffn(x, *ref_weights(ew, dt), mode=2)
+    ref = oracle.ffn(x, *ref_weights(oracle, ew, dt), mode=2)
     ffn_gate(outs, ref, "fp8 batch of 200 calls")
     one = layer.expert_forward(0, x[32:48].to(cuda))                    # the same rows alone: same bits
     assert torch.equal(one.view(torch.int16), outs[32:48].view(torch.int16))

@@ -63,3 +63,21 @@ def test_narrowing_nan(oracle):
     lib = oracle.lib()
     assert np.isnan(lib.eko_bf16_to_f32(lib.eko_f32_to_bf16(float("nan"))))
     assert np.isnan(lib.eko_f16_to_f32(lib.eko_f32_to_f16(float("nan"))))
+
+
+def test_fp8_e4m3fn_exhaustive(oracle):
+    """All 256 encodings: against libtorch's float8_e4m3fn widening (bit for bit, NaNs as NaNs)
+    and against facts of the format that a wrong bias, a missing subnormal branch or an
+    infinity would break: max finite 448, smallest subnormal 2^-9, 0x38 = 1, sign symmetry,
+    monotone over the positive finite codes."""
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    got = oracle.fp8_e4m3fn_to_f32(codes)
+    ref = codes.view(torch.float8_e4m3fn).float()
+    nan = torch.isnan(ref)
+    assert nan.tolist() == [(c & 0x7f) == 0x7f for c in range(256)] and torch.equal(torch.isnan(got), nan)
+    assert torch.equal(got[~nan].view(torch.int32), ref[~nan].view(torch.int32))          # signed zeros included
+    assert float(got[0x7e]) == 448.0 and float(got[0x01]) == 2.0 ** -9 and float(got[0x38]) == 1.0
+    assert float(got[0x08]) == 2.0 ** -6 and float(got[0x07]) == 7 * 2.0 ** -9              # first normal, last subnormal
+    pos = got[:0x7f]
+    assert bool((pos[1:] > pos[:-1]).all()) and not bool(torch.isinf(got).any())
+    assert torch.equal(got[0x80:0xff], -got[:0x7f])
