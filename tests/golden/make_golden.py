@@ -20,11 +20,13 @@ from oracle import oracle  # noqa: E402
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
-# name: (H, I, E, K, T, activation dtype, int8 weights, gate weights kept in fp32)
+# name: (H, I, E, K, T, activation dtype, one-byte weights: False | True (int8 per channel) | "fp8" (e4m3fn
+#        with 128x128 block scales), gate weights kept in fp32)
 CASES = {
     "layer_bf16": (128, 64, 6, 2, 37, torch.bfloat16, False, False),
     "layer_f16_w32": (64, 128, 5, 3, 29, torch.float16, False, True),
     "layer_w8a16": (128, 128, 4, 2, 33, torch.bfloat16, True, False),
+    "layer_fp8_block": (256, 128, 3, 2, 35, torch.bfloat16, "fp8", False),
 }
 
 
@@ -38,7 +40,13 @@ def make_case(name):
     ids, w = oracle.route(0, logits, K, True, w_dtype=torch.float32 if w_f32 else dt)
     wu, wg, wd = [], [], []
     for e in range(E):
-        if w8:
+        if w8 == "fp8":
+            q = [(torch.randn(s, generator=g) * 110).clamp(-448, 448).to(torch.float8_e4m3fn) for s in ((I, H), (I, H), (H, I))]
+            sc = [torch.rand((r + 127) // 128, (c + 127) // 128, generator=g) * 3e-4 + 5e-5 for r, c in ((I, H), (I, H), (H, I))]
+            for m, (qq, ss) in zip(("up", "gate", "down"), zip(q, sc)):
+                out[f"e{e}.{m}_q"], out[f"e{e}.{m}_scale"] = qq, ss
+            deq = [oracle.dequant_block(oracle.fp8_e4m3fn_to_f32(qq), ss) for qq, ss in zip(q, sc)]
+        elif w8:
             q = [torch.randint(-127, 128, s, generator=g, dtype=torch.int8) for s in ((I, H), (I, H), (H, I))]
             sc = [(torch.rand(n, generator=g) * 3e-3 + 1e-3).to(torch.bfloat16) for n in (I, I, H)]
             for m, (qq, ss) in zip(("up", "gate", "down"), zip(q, sc)):

@@ -10,7 +10,7 @@ import torch
 from safetensors.torch import load_file
 
 HERE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-LAYER_CASES = ["layer_bf16", "layer_f16_w32", "layer_w8a16"]
+LAYER_CASES = ["layer_bf16", "layer_f16_w32", "layer_w8a16", "layer_fp8_block"]
 
 
 def load_case(name):
@@ -36,10 +36,12 @@ def test_oracle_reproduces_the_vectors(oracle, name):
     assert torch.equal(bits(y3), bits(t["y3"])) and torch.equal(bits(y), bits(t["y"]))
     assert torch.equal(bits(oracle.gather(t["x"], perm, K)), bits(t["xp"]))
     assert int(t["counts"][E - 1]) == 0                     # the case holds an empty segment
-    if name == "layer_w8a16":
+    if name in ("layer_w8a16", "layer_fp8_block"):
         for e in range(E):
             for m in ("up", "gate", "down"):
-                deq = oracle.dequant_channel(t[f"e{e}.{m}_q"], t[f"e{e}.{m}_scale"], torch.bfloat16)
+                q, sc = t[f"e{e}.{m}_q"], t[f"e{e}.{m}_scale"]
+                deq = oracle.dequant_channel(q, sc, torch.bfloat16) if name == "layer_w8a16" else \
+                    oracle.dequant_block(oracle.fp8_e4m3fn_to_f32(q), sc)
                 assert torch.equal(bits(deq), bits(t[f"e{e}.{m}_w"]))
 
 
@@ -87,6 +89,13 @@ def test_vectors_against_independent_forms(oracle, name):
         q, s = t["e1.down_q"], t["e1.down_scale"]
         exact = (q.double() * s.double().unsqueeze(1))
         assert torch.equal(bits(exact.float().to(torch.bfloat16)), bits(t["e1.down_w"]))
+    # fp8 with block scales: libtorch's widening, the fp32 product w8a16_activate forms
+    # (expert_torch.rs:45-52), one rounding; the down matrix [256,128] spans two row blocks
+    if name == "layer_fp8_block":
+        q, s = t["e1.down_q"], t["e1.down_scale"]
+        assert tuple(s.shape) == (2, 1) and q.dtype == torch.float8_e4m3fn
+        full = s.repeat_interleave(128, 0).repeat_interleave(128, 1)
+        assert torch.equal(bits((q.float() * full).to(torch.bfloat16)), bits(t["e1.down_w"]))
 
 
 def test_router_vectors(oracle):

@@ -20,8 +20,9 @@ def test_layer_matches_golden(ek, cuda, name, mem):
     T, K = t["ids"].shape
     H, I = t["x"].shape[1], wu[0].shape[0]
     dt = t["x"].dtype
-    w8 = name == "layer_w8a16"
-    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=torch.int8 if w8 else dt, max_tokens=64)
+    w8 = name in ("layer_w8a16", "layer_fp8_block")          # one-byte weights with their scales, as stored
+    w_dtype = torch.float8_e4m3fn if name == "layer_fp8_block" else torch.int8 if w8 else dt
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=w_dtype, max_tokens=64)
     for e in range(E):
         if w8:
             layer.set_expert(e, ek.ExpertWeight(up_w=t[f"e{e}.up_q"], gate_w=t[f"e{e}.gate_q"], down_w=t[f"e{e}.down_q"],
