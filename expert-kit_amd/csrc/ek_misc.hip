@@ -23,16 +23,31 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a)
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-    for (int k = 0; k < a.K; ++k) {
-        const int32_t pos = a.inv_perm[t * a.K + k];
-        if (pos < 0) continue;
-        const float wv = WF32 ? ((const float *)a.w)[t * a.K + k] : (float)((const T *)a.w)[t * a.K + k];
-        const V8 v = *(const V8 *)((const T *)a.yp + (int64_t)pos * a.H + c);
+    // the rows of up to 8 slots are requested together, then added in slot order
+    for (int k0 = 0; k0 < a.K; k0 += 8) {
+        int32_t pos[8];
+        float wv[8];
+        V8 v[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float p = wv * (float)v[i];
-            if (!WF32) p = (float)(T)p;
-            acc[i] = acc[i] + p;
+        for (int j = 0; j < 8; ++j) {
+            const int k = k0 + j;
+            pos[j] = k < a.K ? a.inv_perm[t * a.K + k] : -1;
+            wv[j] = 0.f;
+            if (pos[j] >= 0)
+                wv[j] = WF32 ? ((const float *)a.w)[t * a.K + k] : (float)((const T *)a.w)[t * a.K + k];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (pos[j] >= 0) v[j] = *(const V8 *)((const T *)a.yp + (int64_t)pos[j] * a.H + c);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (pos[j] < 0) continue;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float p = wv[j] * (float)v[j][i];
+                if (!WF32) p = (float)(T)p;
+                acc[i] = acc[i] + p;
+            }
         }
     }
     V8 o;
