@@ -33,15 +33,17 @@ def ulp_of(v: torch.Tensor, dtype) -> torch.Tensor:
     return torch.exp2(torch.floor(torch.log2(v.float().abs().clamp_min(1e-30))) - bits)
 
 
-def ffn_gate(got: torch.Tensor, ref32: torch.Tensor, name: str) -> float:
-    """One expert's gate: 2e-2 * rms plus half an output ulp (the output's own storage rounding)."""
+def ffn_gate(got: torch.Tensor, ref32: torch.Tensor, name: str, small: int = 0) -> float:
+    """One expert's gate: 2e-2 * rms plus half an output ulp (the output's own storage rounding).
+    small: outputs of a few thousand elements cannot resolve a fraction of 1e-4; that many
+    elements may then exceed the plain bound (never the full one)."""
     rms = float(ref32.pow(2).mean().sqrt())
     err = (got.float().cpu() - ref32).abs()
     strict_viol = float((err > TOL * rms).float().mean())
     worst = float(err.max()) / rms
     print(f"{name}: max|err|/rms = {worst:.3e}, elements over 2e-2*rms: {strict_viol:.2e}", flush=True)
     assert bool((err <= TOL * rms + 0.5 * ulp_of(ref32, got.dtype) * 1.0001).all()), worst
-    assert strict_viol <= 1e-4
+    assert strict_viol <= 1e-4 or int((err > TOL * rms).sum()) <= small
     return worst
 
 
@@ -58,7 +60,8 @@ def check_vs_rounded(got: torch.Tensor, ref32: torch.Tensor, name: str = ""):
     return same
 
 
-def layer_gate(y: torch.Tensor, ref32: torch.Tensor, y3: torch.Tensor, gw: torch.Tensor, name: str) -> float:
+def layer_gate(y: torch.Tensor, ref32: torch.Tensor, y3: torch.Tensor, gw: torch.Tensor, name: str,
+               small: int = 0) -> float:
     """The layer's parity gate.
 
     strict : max|y - y_ref| <= 2e-2 * rms(y_ref) -- must hold for all but 1e-4 of the
@@ -80,7 +83,7 @@ def layer_gate(y: torch.Tensor, ref32: torch.Tensor, y3: torch.Tensor, gw: torch
     worst = float(err.max()) / rms
     print(f"{name}: max|err|/rms = {worst:.3e}, elements over 2e-2*rms: {strict_viol:.2e}", flush=True)
     assert bool((err <= TOL * rms + flip).all()), worst
-    assert strict_viol <= 1e-4
+    assert strict_viol <= 1e-4 or int((err > TOL * rms).sum()) <= small      # see ffn_gate
     return worst
 
 

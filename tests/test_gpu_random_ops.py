@@ -1,0 +1,145 @@
+"""A seeded random walk over the layer object's entry points.
+
+Each step draws one operation -- load or remove an expert, a per-expert call, a grouped call, a
+wire call, a whole-layer call, or a call that must be refused -- on host or device tensors, and
+holds its result to what the state of the registry implies: the oracle's output within the parity
+gates when every expert involved is loaded, the reference's error otherwise (ExpertDB::load of a
+missing expert, worker/manager.rs:57-66), and nothing from a refused call may leak into the calls
+after it.
+"""
+import pytest
+import torch
+from safetensors.torch import load as st_load
+from safetensors.torch import save as st_save
+
+from ek_hip import workloads as wl
+from test_gpu_parity import ffn_gate, layer_gate, oracle_weights
+
+pytestmark = pytest.mark.gpu
+
+H, I, E, K, TMAX = 256, 128, 6, 2, 96
+
+
+@pytest.mark.parametrize("w8", [False, True])
+def test_random_walk(ek, oracle, cuda, w8):
+    dt = torch.bfloat16
+    g = torch.Generator().manual_seed(424242 + w8)
+    draw = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=torch.int8 if w8 else dt, max_tokens=TMAX)
+    work = wl.Workload("walk", H, I, E, K, 1, dt, w8=w8)
+    loaded, version = {}, 0
+    done = {k: 0 for k in ("set", "remove", "expert", "experts", "wire", "layer", "refused")}
+
+    # With 128 terms per output the products of two near-Gaussians give these small layers heavier
+    # tails than the benchmark shapes: an output at 7 sigma is further than 2e-2 * rms from its own
+    # 16-bit neighbour.  The full gate (bound + storage quanta) holds for every element; the share
+    # allowed over the plain bound is 5e-4 here instead of 1e-4.
+    def tails(n_rows):
+        return 2 + int(5e-4 * n_rows * H)
+
+    def ref_ws():
+        return oracle_weights(oracle, loaded, E, dt)
+
+    def rows(n):
+        return torch.randn(n, H, generator=g).to(dt)
+
+    def place(t):
+        return t.to(cuda) if draw(0, 1) else t
+
+    for step in range(240):
+        op = draw(0, 9)
+        if op <= 1 or (len(loaded) < 3 and op != 9):                  # load (or replace) an expert
+            e = draw(0, E - 1)
+            version += 1
+            ew = wl.make_expert(work, e, layer=version, std=0.05)
+            layer.set_expert(e, ew)
+            loaded[e] = ew
+            done["set"] += 1
+        elif op == 2:                                                 # remove one
+            e = draw(0, E - 1)
+            if e in loaded:
+                layer.remove_expert(e)
+                del loaded[e]
+            else:
+                with pytest.raises(ek.EKError) as ei:
+                    layer.remove_expert(e)
+                assert ei.value.status == ek.EK_EXPERT_NOT_FOUND
+            assert layer.has_expert(e) is False
+            done["remove"] += 1
+        elif op in (3, 4):                                            # one expert, n rows
+            e = sorted(loaded)[draw(0, len(loaded) - 1)] if draw(0, 3) else draw(0, E - 1)
+            n = [0, 1, 7, 16, 17, 40, 64, 100, 192][draw(0, 8)]
+            x = rows(n)
+            if e not in loaded:
+                with pytest.raises(ek.EKError) as ei:
+                    layer.expert_forward(e, place(x))
+                assert ei.value.status == ek.EK_EXPERT_NOT_FOUND
+                done["refused"] += 1
+                continue
+            if op == 3:
+                got = layer.expert_forward(e, place(x))
+                done["expert"] += 1
+            else:
+                got = st_load(layer.worker_forward(f"walk/l0-e{e}", st_save({"data": x})))["data"]
+                done["wire"] += 1
+            if n:
+                wu, wg, wd = ref_ws()
+                ffn_gate(got, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: expert {e}, {n} rows", small=tails(n))
+            assert tuple(got.shape) == (n, H)
+        elif op == 5:                                                 # several per-expert calls, one launch
+            among = sorted(loaded) if draw(0, 3) else list(range(E))
+            calls = [(among[draw(0, len(among) - 1)], draw(0, 24)) for _ in range(draw(1, 7))]
+            xs = [rows(n) for _, n in calls]
+            dev = draw(0, 1)
+            if any(e not in loaded for e, _ in calls):
+                with pytest.raises(ek.EKError) as ei:
+                    layer.experts_forward([e for e, _ in calls], [x.to(cuda) if dev else x for x in xs])
+                assert ei.value.status == ek.EK_EXPERT_NOT_FOUND
+                done["refused"] += 1
+                continue
+            outs = layer.experts_forward([e for e, _ in calls], [x.to(cuda) if dev else x for x in xs])
+            wu, wg, wd = ref_ws()
+            for (e, n), x, out in zip(calls, xs, outs):
+                if n:
+                    ffn_gate(out, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: batch, expert {e}, {n} rows", small=tails(n))
+            done["experts"] += 1
+        elif op in (6, 7, 8):                                         # the whole layer
+            T = draw(0, TMAX)
+            pool = torch.tensor(sorted(loaded)) if draw(0, 3) else torch.arange(E)      # mostly among the loaded ones
+            ids = torch.stack([pool[torch.randperm(len(pool), generator=g)[:K]] for _ in range(T)]
+                              or [torch.zeros(0, dtype=torch.int64)])
+            ids = ids.to(torch.int32).reshape(T, K)
+            gw = torch.rand(T, K, generator=g) + 0.1
+            gw = (gw / gw.sum(-1, keepdim=True)).to(dt)
+            x = rows(T)
+            dev = draw(0, 1)
+            args = [t.to(cuda) if dev else t for t in (x, ids, gw)]
+            if T and any(int(e) not in loaded for e in ids.unique()):
+                with pytest.raises(ek.EKError) as ei:
+                    layer.forward(*args)
+                assert ei.value.status == ek.EK_EXPERT_NOT_FOUND
+                done["refused"] += 1
+                continue
+            y = layer.forward(*args)
+            if T:
+                wu, wg, wd = ref_ws()
+                ref, _, _, _, _, y3 = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=2, return_y3=True)
+                layer_gate(y, ref, y3, gw, f"step {step}: layer, T={T}", small=tails(T))
+            done["layer"] += 1
+        else:                                                         # calls that must be refused
+            kind = draw(0, 3)
+            with pytest.raises(ek.EKError) as ei:
+                if kind == 0:
+                    layer.expert_forward(E + draw(0, 3), rows(4))                      # no such expert index
+                elif kind == 1:
+                    layer.expert_forward(0, rows(TMAX * K + 1))                        # more rows than the workspace
+                elif kind == 2:
+                    bad = torch.full((4, K), E, dtype=torch.int32)
+                    layer.forward(rows(4), bad, torch.ones(4, K).to(dt))               # id outside [0, E)
+                else:
+                    layer.worker_forward("walk/l0-e0", st_save({"data": rows(3).float()}))   # wrong dtype on the wire
+            assert ei.value.status in (ek.EK_INVALID_INPUT, ek.EK_EXPERT_NOT_FOUND), ei.value
+            done["refused"] += 1
+    print("random walk:", done, flush=True)
+    assert all(v > 0 for v in done.values()), done
+    layer.close()
