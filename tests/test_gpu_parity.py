@@ -387,6 +387,26 @@ def test_layer_full_size_sampled_tokens(ek, oracle, cuda, name):
     layer.close()
 
 
+@pytest.mark.parametrize("H,I,w8", [(2048, 1408, False), (5120, 1536, True), (4096, 14336, False), (7168, 2048, True)])
+def test_model_shapes(ek, oracle, cuda, H, I, w8):
+    """Expert shapes of published MoE models (DeepSeek-V2-Lite, Qwen3-235B, Mixtral-8x7B, DeepSeek-V3):
+    channel-tile counts that are not multiples of the kernels' block sizes (1408 / 16 = 88 tiles, 1536 / 16
+    = 96), the longest contraction (14336) and the benchmark's own shape.  Five rows through the
+    streaming kernel, 33 rows through the tile kernel (every token routed to the expert)."""
+    dt = torch.bfloat16
+    print(f"model shape H={H} I={I} w8={w8}", flush=True)
+    w = wl.Workload("shape", H, I, 2, 1, 33, dt, w8=w8)
+    layer, ws = load_layer(ek, w, experts=[1], device="cuda")
+    wu, wg, wd = [t[1] for t in oracle_weights(oracle, ws, 2, dt)]
+    x = torch.randn(33, H, generator=torch.Generator().manual_seed(H + I)).to(dt)
+    got5 = layer.expert_forward(1, x[:5].to(cuda))
+    ffn_gate(got5, oracle.ffn(x[:5], wu, wg, wd, mode=2), f"H={H} I={I}: 5 rows, streaming kernel", small=2)
+    got33 = layer.forward(x.to(cuda), torch.ones(33, 1, dtype=torch.int32, device=cuda),
+                          torch.ones(33, 1, dtype=dt, device=cuda))
+    ffn_gate(got33, oracle.ffn(x, wu, wg, wd, mode=2), f"H={H} I={I}: 33 rows, tile kernel", small=2)
+    layer.close()
+
+
 # ------------------------------------------------------------ error paths
 
 def test_error_paths(ek, cuda):
