@@ -628,8 +628,10 @@ ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_lo
 // wide_items > 0: the lists hold that many weight-streaming items of up to kWideRows rows and
 // nothing else (the per-expert entry points' cut for calls that would leave the tile kernel
 // most of the chip idle).
+// extra_stream: streaming items the lists hold beyond what P rows over E experts can give (a
+// shared segment cut into 16-row items).
 ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out, int64_t P, int64_t E,
-                      hipStream_t s, hipEvent_t *ev, int64_t wide_items = 0)
+                      hipStream_t s, hipEvent_t *ev, int64_t wide_items = 0, int64_t extra_stream = 0)
 {
     const int64_t H = L->cfg.hidden, I = L->cfg.inter;
     ek::FfnArgs a1;
@@ -640,7 +642,7 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
     a2.N = (int32_t)H; a2.Kdim = (int32_t)I;
     int64_t cap[ek::kNumLists];
     for (int l = 0; l < ek::kNumLists; ++l) {
-        cap[l] = ek::list_capacity(l, P, E);
+        cap[l] = ek::list_capacity(l, P, E) + (l == ek::kListStream ? extra_stream : 0);
         if (cap[l] > L->list_cap[l]) cap[l] = L->list_cap[l];
         if (cap[l] < 0) cap[l] = 0;
     }
@@ -696,10 +698,18 @@ ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const 
     ek::launch_pack(pack_args(L, ids, P, true), s);
     // the shared expert is one more segment: every token once, rows P .. P+T-1 of the packed buffers
     const bool shared = L->expert_mem[E] != nullptr && T > 0;
-    if (shared) ek::launch_append_segment(L->lists, E, (int32_t)P, (int32_t)T, L->row_token, s);
+    // Up to kSharedStreamRows tokens the shared segment is cut into 16-row streaming items: as a
+    // tile it would occupy 8 to 14 CUs for the length of the whole contraction (measured on the
+    // DeepSeek-V3 shape at 64 tokens: 1.62 ms against 1.76 ms; at 128 and 256 tokens the two
+    // cuts are within 1 % of each other and from 512 on the tiles win, each item re-reading
+    // the expert's weights).
+    constexpr int64_t kSharedStreamRows = 64;
+    const bool shared_streamed = shared && T <= kSharedStreamRows;
+    if (shared) ek::launch_append_segment(L->lists, E, (int32_t)P, (int32_t)T, L->row_token, shared_streamed, s);
     if (ev) EK_HIP(hipEventRecord(ev[1], s));
     if (P > 0) {
-        EK_TRY(enqueue_ffn(L, x, L->row_token, L->yp, shared ? P + T : P, shared ? E + 1 : E, s, ev));
+        EK_TRY(enqueue_ffn(L, x, L->row_token, L->yp, shared ? P + T : P, shared ? E + 1 : E, s, ev, 0,
+                           shared_streamed ? (T + 15) / 16 : 0));
         if (ev) EK_HIP(hipEventRecord(ev[3], s));
         ek::CombineArgs c;
         c.yp = L->yp; c.inv_perm = L->inv_perm; c.w = w; c.y = y; c.T = T; c.K = K; c.H = H;

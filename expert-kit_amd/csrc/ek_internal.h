@@ -124,7 +124,7 @@ void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool
 // appends the segment (expert, rows row0 .. row0+n-1) to the lists pack has built and maps
 // its rows to tokens 0 .. n-1
 void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token,
-                           hipStream_t s);
+                           bool as_stream, hipStream_t s);
 void launch_gather(const void *x, const int32_t *row_token, int64_t P, int64_t row_bytes, void *xp,
                    hipStream_t s);
 

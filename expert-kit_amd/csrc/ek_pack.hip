@@ -144,11 +144,21 @@ __global__ void single_lists_kernel(WorkLists l, int32_t e, int32_t n, int32_t w
 }
 
 __global__ __launch_bounds__(256) void append_segment_kernel(WorkLists l, int32_t e, int32_t row0, int32_t n,
-                                                             int32_t *row_token)
+                                                             int32_t *row_token, int32_t as_stream)
 {
     const int32_t p128 = l.count[kListT128], p64 = l.count[kListT64], p32 = l.count[kListT32],
                   ps = l.count[kListStream];
     __syncthreads();   // every thread has read the old lengths before thread 0 replaces them
+    if (as_stream) {
+        // a decode-sized segment: as one tile per 128 rows it would run on a handful of CUs for
+        // the length of the whole contraction; as 16-row streaming items it spreads over the chip
+        const int32_t items = (n + 15) >> 4;
+        for (int32_t t = threadIdx.x; t < items; t += 256)
+            l.items[kListStream][ps + t] = WorkItem{e, row0 + t * 16, min(16, n - t * 16), 0};
+        for (int32_t t = threadIdx.x; t < n; t += 256) row_token[row0 + t] = t;
+        if (threadIdx.x == 0) l.count[kListStream] = ps + items;
+        return;
+    }
     const SegmentCut c = cut_segment(n);
     const int32_t full = n >> 7, r = n & 127;
     for (int32_t t = threadIdx.x; t < full; t += 256) l.items[kListT128][p128 + t] = WorkItem{e, row0 + t * 128, 128, 0};
@@ -167,9 +177,10 @@ __global__ __launch_bounds__(256) void append_segment_kernel(WorkLists l, int32_
 }
 
 void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token,
-                           hipStream_t s)
+                           bool as_stream, hipStream_t s)
 {
-    hipLaunchKernelGGL(append_segment_kernel, dim3(1), dim3(256), 0, s, lists, expert, row0, n, row_token);
+    hipLaunchKernelGGL(append_segment_kernel, dim3(1), dim3(256), 0, s, lists, expert, row0, n, row_token,
+                       as_stream ? 1 : 0);
 }
 
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool wide, hipStream_t s)

@@ -51,8 +51,12 @@ def test_shared_expert_segment(ek, oracle, cuda, dt, w8):
         y = layer.forward(x.to(cuda), ids.to(cuda), w.to(cuda))
         # (1) composition: the same expert as the only routed one with gate weight 1 is cut like the
         # shared segment (a per-expert call of this size may be cut for the other kernel family)
-        y_sh = single.forward(x.to(cuda), torch.zeros(T, 1, dtype=torch.int32, device=cuda),
-                              torch.ones(T, 1, dtype=dt, device=cuda))
+        # (up to 64 tokens the shared segment is a run of 16-row streaming items)
+        if T <= 64:
+            y_sh = torch.cat(single.experts_forward([0] * ((T + 15) // 16), list(x.to(cuda).split(16))))
+        else:
+            y_sh = single.forward(x.to(cuda), torch.zeros(T, 1, dtype=torch.int32, device=cuda),
+                                  torch.ones(T, 1, dtype=dt, device=cuda))
         want = (y_plain.float() + y_sh.float()).to(dt)
         assert torch.equal(y.view(torch.int16), want.view(torch.int16)), T
         assert not torch.equal(y, y_plain)
