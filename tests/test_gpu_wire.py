@@ -87,14 +87,19 @@ def test_batch_is_one_grouped_launch_per_stage(ek):
     for _ in range(3):
         layer.experts_forward(ex, xs)
         [layer.expert_forward(e, x) for e, x in zip(ex, xs)]
-    t0 = time.perf_counter()
-    for _ in range(20):
-        layer.experts_forward(ex, xs)
-    t_batch = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    for _ in range(20):
-        [layer.expert_forward(e, x) for e, x in zip(ex, xs)]
-    t_single = time.perf_counter() - t0
+    def best_of(fn, reps=5, n=20):          # wall clock of n calls with the device drained, best of reps
+        best = float("inf")
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t0)
+        return best
+
+    t_batch = best_of(lambda: layer.experts_forward(ex, xs))
+    t_single = best_of(lambda: [layer.expert_forward(e, x) for e, x in zip(ex, xs)])
     print(f"batch of {E}: {t_batch / 20 * 1e6:.0f} us, one by one: {t_single / 20 * 1e6:.0f} us", flush=True)
     assert t_batch < 1.25 * t_single
     layer.close()
