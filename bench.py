@@ -75,6 +75,19 @@ def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
     return pairs / med, pairs, len(times)
 
 
+def calibration_copy(args, dev):
+    """A plain device copy of --calib-copy-mib MiB: a kernel of known traffic for the profiler's counters."""
+    import torch
+    if not args.calib_copy_mib:
+        return
+    src = torch.empty(args.calib_copy_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def bench_chain(args, w, dev):
     """The ragged continuous-batching mix over n_layers consecutive layers, one hipGraph."""
     import torch
@@ -95,6 +108,7 @@ def bench_chain(args, w, dev):
     chain = ek_hip.HipChain(layers)
     stream = torch.cuda.current_stream()
     y_eager = chain.forward(xd, ids, gw, use_graph=False).clone()
+    calibration_copy(args, dev)
     res = {}
     for mode, use_graph in (("eager", False), ("graph", True)):
         for _ in range(args.warmup):
@@ -190,13 +204,7 @@ def main():
     ref_perm = torch.argsort(ids.reshape(-1).long(), stable=True).to(torch.int32)
     assert torch.equal(rt.perm.cpu(), ref_perm), "routing permutation mismatch"
 
-    if args.calib_copy_mib:
-        src = torch.empty(args.calib_copy_mib << 20, dtype=torch.uint8, device=dev).random_(0, 255)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+    calibration_copy(args, dev)
     for _ in range(args.warmup):
         layer.forward(xd, idd, gwd, stream=stream, out=y)
     torch.cuda.synchronize()
