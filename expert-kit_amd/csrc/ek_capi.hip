@@ -467,10 +467,14 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
         std::lock_guard<std::mutex> lk(L->mu);
         old = L->expert_mem[e];
         if (old) (void)hipDeviceSynchronize();   // drain work that may read the old copy
+        hipError_t er = hipMemcpy(L->d_slabs + e, &slab, sizeof slab, hipMemcpyHostToDevice);
+        if (er != hipSuccess) {
+            // the table still names the old copy (if any): keep it, drop the new one
+            (void)hipFree(mem);
+            return hip_fail(er, "slab table update");
+        }
         L->expert_mem[e] = mem;
         L->h_slabs[e] = slab;
-        hipError_t er = hipMemcpy(L->d_slabs + e, &slab, sizeof slab, hipMemcpyHostToDevice);
-        if (er != hipSuccess) return hip_fail(er, "slab table update");
     }
     if (old) (void)hipFree(old);
     return EK_OK;
@@ -795,6 +799,7 @@ ek_status ek_layer_set_expert(ek_layer *layer, int32_t expert, const ek_weight_d
         if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
         EK_TRY(expert_slot(layer, expert, &expert));
         DeviceGuard dg(layer->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
         std::lock_guard<std::mutex> lk(layer->load_mu);
         return set_expert_locked(layer, expert, up, gate, down);
     )
@@ -806,6 +811,7 @@ ek_status ek_layer_remove_expert(ek_layer *layer, int32_t expert)
         if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
         EK_TRY(expert_slot(layer, expert, &expert));
         DeviceGuard dg(layer->cfg.device_id);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
         std::lock_guard<std::mutex> lk0(layer->load_mu);
         void *old = nullptr;
         {
