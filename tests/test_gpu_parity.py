@@ -353,15 +353,16 @@ def test_layer_c3_sampled(ek, oracle, cuda):
     layer.close()
 
 
-@pytest.mark.parametrize("name", ["c3", "c4"])
+@pytest.mark.parametrize("name", ["c2", "c3", "c4", "c5"])
 def test_layer_full_size_sampled_tokens(ek, oracle, cuda, name):
-    """The two DeepSeek-V3 configurations at full size (256 experts resident; 128 decode tokens /
-    8192 prefill tokens with hot-expert skew): the whole layer call on the GPU; the oracle
-    recomputes a handful of tokens (rows are independent in the reference) that between them
-    sit in the longest segment, in a segment short enough for the streaming kernel, in
-    segments whose remainder is cut into a 128-, 64- and 32-row tile (prefill), and four
-    tokens drawn at random."""
-    w = wl.CONFIGS[name]
+    """The configurations at full size (c3 / c4: DeepSeek-V3 shape, 256 experts resident, 128
+    decode tokens / 8192 prefill tokens with hot-expert skew; c2: Qwen3 shape, fp16, 256 decode
+    tokens; c5: the first layer of the ragged mix, 5052 tokens): the whole layer call on the
+    GPU; the oracle recomputes a handful of tokens (rows are independent in the reference) that
+    between them sit in the longest segment, in a segment short enough for the streaming
+    kernel, in segments whose remainder is cut into a 128-, 64- and 32-row tile (prefill), and
+    four tokens drawn at random."""
+    w = wl.resolve(wl.CONFIGS[name])
     print(f"{name} full size: building {w.n_experts} experts on the GPU", flush=True)
     layer, ws = load_layer(ek, w, device="cuda")
     x = wl.make_x(w)
@@ -380,7 +381,7 @@ def test_layer_full_size_sampled_tokens(ek, oracle, cuda, name):
     tokens = sorted(set(tokens))
     need = sorted(set(ids[tokens].flatten().tolist()))
     print(f"{name} full size: tokens {tokens}, {len(need)} experts recomputed by the oracle", flush=True)
-    wu, wg, wd = oracle_weights(oracle, {e: ws[e] for e in need}, w.n_experts)
+    wu, wg, wd = oracle_weights(oracle, {e: ws[e] for e in need}, w.n_experts, w.act_dtype)
     ref, _, _, _, _, y3 = oracle.layer_forward(x[tokens], ids[tokens], gw[tokens], wu, wg, wd, mode=2, return_y3=True)
     layer_gate(y[tokens], ref, y3, gw[tokens], f"{name} full size, sampled tokens")
     assert layer.stats()["pairs"] == w.pairs
