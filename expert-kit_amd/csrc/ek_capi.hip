@@ -102,6 +102,9 @@ struct ek_layer {
     void *h = nullptr, *yp = nullptr;
     ek::WorkLists lists{};                   // device work lists (see ek_internal.h)
     int64_t list_cap[ek::kNumLists] = {0, 0, 0, 0};
+    // a list of its own for a shared expert's segment cut into wide streaming items
+    ek::WorkItem *wide_items = nullptr;
+    int32_t *wide_count = nullptr;           // [kNumLists], only [kListStream] is used
     int32_t *h_err = nullptr;                // pinned
     // host-built work lists (ek_layer_experts_forward): pinned image of the device lists,
     // reused once ev_items says the previous copy has been consumed
@@ -164,6 +167,13 @@ struct ek_chain {
 
 namespace {
 
+// A shared expert's segment (one row per token) is cut by the number of tokens T:
+// up to kSharedStreamRows into 16-row streaming items in the routed pairs' list, up to
+// kSharedWideRows into streaming items of up to ek::kWideRows rows with a launch of their own
+// beside the others, beyond that into tiles like any segment (see enqueue_forward).
+constexpr int64_t kSharedStreamRows = 64, kSharedWideRows = 256;
+constexpr int64_t kSharedWideItems = kSharedWideRows / ek::kWideRows;
+
 ek_status dev_alloc(void **p, size_t bytes, const char *what)
 {
     hipError_t e = hipMalloc(p, bytes ? bytes : 16);
@@ -184,7 +194,7 @@ void free_layer(ek_layer *L)
     void *bufs[] = {L->d_slabs, L->counts, L->offsets, L->perm, L->inv_perm, L->row_token,
                     L->block_hist, L->err, L->h, L->yp, L->st_x, L->st_w, L->st_y, L->st_xp,
                     L->d_activation, L->st_ids, L->st_raw, L->rt_ids, L->rt_w, L->st_logits, L->st_bias, L->lists.count, L->lists.items[0], L->lists.items[1],
-                    L->lists.items[2], L->lists.items[3]};
+                    L->lists.items[2], L->lists.items[3], L->wide_items, L->wide_count};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
     if (L->h_err) (void)hipHostFree(L->h_err);
@@ -270,6 +280,8 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     A(&L->h, (size_t)rows_max * cfg->inter * 2, "h");
     A(&L->yp, (size_t)rows_max * cfg->hidden * 2, "yp");
     A((void **)&L->lists.count, sizeof(int32_t) * ek::kNumLists, "work list counts");
+    A((void **)&L->wide_items, sizeof(ek::WorkItem) * kSharedWideItems, "shared expert's work list");
+    A((void **)&L->wide_count, sizeof(int32_t) * ek::kNumLists, "shared expert's work list count");
     for (int l = 0; l < ek::kNumLists; ++l) {
         // the per-expert entry point cuts one segment of up to pmax rows: capacity for E = 1 too
         // (and the wide cut, see wide_cut_pays: fewer than 128 tile items of at most 128 rows
@@ -283,6 +295,7 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         if (e == hipSuccess) e = hipMemset(L->err, 0, sizeof(int32_t) * 4);
         if (e == hipSuccess) e = hipMemset(L->d_activation, 0, sizeof(uint64_t) * E);
         if (e == hipSuccess) e = hipMemset(L->lists.count, 0, sizeof(int32_t) * ek::kNumLists);
+        if (e == hipSuccess) e = hipMemset(L->wide_count, 0, sizeof(int32_t) * ek::kNumLists);
         if (e == hipSuccess) e = hipHostMalloc((void **)&L->h_err, sizeof(int32_t) * 4, hipHostMallocDefault);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->load_stream, hipStreamNonBlocking);
@@ -634,8 +647,11 @@ ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_lo
 // most of the chip idle).
 // extra_stream: streaming items the lists hold beyond what P rows over E experts can give (a
 // shared segment cut into 16-row items).
+// shared_wide: L->wide_items holds that many streaming items of up to kWideRows rows (a shared
+// segment); they get launches of their own on the side stream, beside the others.
 ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out, int64_t P, int64_t E,
-                      hipStream_t s, hipEvent_t *ev, int64_t wide_items = 0, int64_t extra_stream = 0)
+                      hipStream_t s, hipEvent_t *ev, int64_t wide_items = 0, int64_t extra_stream = 0,
+                      int64_t shared_wide = 0)
 {
     const int64_t H = L->cfg.hidden, I = L->cfg.inter;
     ek::FfnArgs a1;
@@ -668,18 +684,24 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
     const bool have_tiles = cap[ek::kListT32] + cap[ek::kListT64] + cap[ek::kListT128] > 0;
     const bool fork = have_stream && have_tiles && P > 4 * E && P <= 64 * E;
     hipStream_t s_stream = s, s_tiles = s;
-    if (fork) {
+    if (fork || shared_wide > 0) {
         EK_HIP(hipEventRecord(L->ev_fork, s));
         EK_HIP(hipStreamWaitEvent(L->side_stream, L->ev_fork, 0));
-        (tiles_main ? s_stream : s_tiles) = L->side_stream;
     }
+    if (fork) (tiles_main ? s_stream : s_tiles) = L->side_stream;
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
         if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, cap[ek::kListStream], false, s_stream));
+        if (shared_wide > 0) {
+            ek::FfnArgs aw = a;                  // the same stage over the shared segment's own list
+            aw.lists.items[ek::kListStream] = L->wide_items;
+            aw.lists.count = L->wide_count;
+            EK_HIP(ek::launch_ffn_stream(aw, stage, L->act, L->wmode, shared_wide, true, L->side_stream));
+        }
         if (have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
     }
-    if (fork) {
+    if (fork || shared_wide > 0) {
         EK_HIP(hipEventRecord(L->ev_join, L->side_stream));
         EK_HIP(hipStreamWaitEvent(s, L->ev_join, 0));
     }
@@ -702,18 +724,27 @@ ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const 
     ek::launch_pack(pack_args(L, ids, P, true), s);
     // the shared expert is one more segment: every token once, rows P .. P+T-1 of the packed buffers
     const bool shared = L->expert_mem[E] != nullptr && T > 0;
-    // Up to kSharedStreamRows tokens the shared segment is cut into 16-row streaming items: as a
-    // tile it would occupy 8 to 14 CUs for the length of the whole contraction (measured on the
-    // DeepSeek-V3 shape at 64 tokens: 1.62 ms against 1.76 ms; at 128 and 256 tokens the two
-    // cuts are within 1 % of each other and from 512 on the tiles win, each item re-reading
-    // the expert's weights).
-    constexpr int64_t kSharedStreamRows = 64;
+    // As tiles a decode-sized shared segment would occupy 8 to 14 CUs for the length of the whole
+    // contraction.  Up to kSharedStreamRows tokens it is cut into 16-row streaming items
+    // (measured on the DeepSeek-V3 shape at 64 tokens: 1.62 ms against 1.76 ms as a tile); each
+    // item re-reads the expert's weights, so beyond that it is cut into items of up to 64 rows,
+    // which the streaming kernel's wide form takes in a launch of its own.
     const bool shared_streamed = shared && T <= kSharedStreamRows;
-    if (shared) ek::launch_append_segment(L->lists, E, (int32_t)P, (int32_t)T, L->row_token, shared_streamed, s);
+    const bool shared_wide = shared && !shared_streamed && T <= kSharedWideRows;
+    if (shared_wide) {
+        ek::WorkLists own = L->lists;
+        own.items[ek::kListStream] = L->wide_items;
+        own.count = L->wide_count;
+        ek::launch_append_segment(own, E, (int32_t)P, (int32_t)T, L->row_token, 2, s);
+    } else if (shared) {
+        ek::launch_append_segment(L->lists, E, (int32_t)P, (int32_t)T, L->row_token, shared_streamed ? 1 : 0, s);
+    }
     if (ev) EK_HIP(hipEventRecord(ev[1], s));
     if (P > 0) {
-        EK_TRY(enqueue_ffn(L, x, L->row_token, L->yp, shared ? P + T : P, shared ? E + 1 : E, s, ev, 0,
-                           shared_streamed ? (T + 15) / 16 : 0));
+        const bool in_lists = shared && !shared_wide;   // the shared segment's items sit in the routed pairs' lists
+        EK_TRY(enqueue_ffn(L, x, L->row_token, L->yp, in_lists ? P + T : P, in_lists ? E + 1 : E, s, ev, 0,
+                           shared_streamed ? (T + 15) / 16 : 0,
+                           shared_wide ? (T + ek::kWideRows - 1) / ek::kWideRows : 0));
         if (ev) EK_HIP(hipEventRecord(ev[3], s));
         ek::CombineArgs c;
         c.yp = L->yp; c.inv_perm = L->inv_perm; c.w = w; c.y = y; c.T = T; c.K = K; c.H = H;

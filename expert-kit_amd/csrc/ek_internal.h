@@ -122,9 +122,11 @@ void launch_pack(const PackArgs &a, hipStream_t s);
 // work lists for one segment [0, n) of expert e (per-expert forward)
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool wide, hipStream_t s);
 // appends the segment (expert, rows row0 .. row0+n-1) to the lists pack has built and maps
-// its rows to tokens 0 .. n-1
+// its rows to tokens 0 .. n-1.  as_stream: 0 the usual cut; 1 all rows as 16-row streaming items;
+// 2 all rows as streaming items of up to kWideRows rows, which replace the streaming list (the
+// caller passes a list of their own)
 void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token,
-                           bool as_stream, hipStream_t s);
+                           int as_stream, hipStream_t s);
 void launch_gather(const void *x, const int32_t *row_token, int64_t P, int64_t row_bytes, void *xp,
                    hipStream_t s);
 

@@ -151,12 +151,15 @@ __global__ __launch_bounds__(256) void append_segment_kernel(WorkLists l, int32_
     __syncthreads();   // every thread has read the old lengths before thread 0 replaces them
     if (as_stream) {
         // a decode-sized segment: as one tile per 128 rows it would run on a handful of CUs for
-        // the length of the whole contraction; as 16-row streaming items it spreads over the chip
-        const int32_t items = (n + 15) >> 4;
+        // the length of the whole contraction; as streaming items it spreads over the chip.
+        // as_stream = 1: 16-row items appended to the list; 2: items of up to kWideRows rows
+        // that become the whole list (a list of their own, for a launch of their own)
+        const int32_t per = as_stream == 2 ? kWideRows : 16, at = as_stream == 2 ? 0 : ps;
+        const int32_t items = (n + per - 1) / per;
         for (int32_t t = threadIdx.x; t < items; t += 256)
-            l.items[kListStream][ps + t] = WorkItem{e, row0 + t * 16, min(16, n - t * 16), 0};
+            l.items[kListStream][at + t] = WorkItem{e, row0 + t * per, min(per, n - t * per), 0};
         for (int32_t t = threadIdx.x; t < n; t += 256) row_token[row0 + t] = t;
-        if (threadIdx.x == 0) l.count[kListStream] = ps + items;
+        if (threadIdx.x == 0) l.count[kListStream] = at + items;
         return;
     }
     const SegmentCut c = cut_segment(n);
@@ -177,10 +180,10 @@ __global__ __launch_bounds__(256) void append_segment_kernel(WorkLists l, int32_
 }
 
 void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token,
-                           bool as_stream, hipStream_t s)
+                           int as_stream, hipStream_t s)
 {
     hipLaunchKernelGGL(append_segment_kernel, dim3(1), dim3(256), 0, s, lists, expert, row0, n, row_token,
-                       as_stream ? 1 : 0);
+                       as_stream);
 }
 
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool wide, hipStream_t s)

@@ -41,7 +41,7 @@ def test_shared_expert_segment(ek, oracle, cuda, dt, w8):
     single = ek.HipLayer(H, I, 1, 1, act_dtype=dt, w_dtype=torch.int8 if w8 else dt, max_tokens=512)
     single.set_expert(0, ws[E])
     wu, wg, wd = oracle_weights(oracle, ws, E + 1, dt)
-    for T in (1, 16, 17, 33, 100, 130, 300):
+    for T in (1, 16, 17, 33, 64, 65, 100, 130, 256, 257, 300):
         x, ids, w = routing(T, 40 + T)
         x, w = x.to(dt), w.to(dt)
         assert not layer.has_expert(C.EK_SHARED_EXPERT)
@@ -51,9 +51,12 @@ def test_shared_expert_segment(ek, oracle, cuda, dt, w8):
         y = layer.forward(x.to(cuda), ids.to(cuda), w.to(cuda))
         # (1) composition: the same expert as the only routed one with gate weight 1 is cut like the
         # shared segment (a per-expert call of this size may be cut for the other kernel family)
-        # (up to 64 tokens the shared segment is a run of 16-row streaming items)
+        # (up to 64 tokens the shared segment is a run of 16-row streaming items, up to 256 a run
+        # of 64-row ones, which is how a lone per-expert call of that size is cut too)
         if T <= 64:
             y_sh = torch.cat(single.experts_forward([0] * ((T + 15) // 16), list(x.to(cuda).split(16))))
+        elif T <= 256:
+            y_sh = single.expert_forward(0, x.to(cuda))
         else:
             y_sh = single.forward(x.to(cuda), torch.zeros(T, 1, dtype=torch.int32, device=cuda),
                                   torch.ones(T, 1, dtype=dt, device=cuda))
