@@ -1004,7 +1004,7 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
             }
             // the ordinary cut's tile items: full 128-row tiles and a remainder of more than 16 rows
             const int64_t wide_items = (n + ek::kWideRows - 1) / ek::kWideRows;
-            const bool wide = ek::wide_cut_pays((n >> 7) + ((n & 127) > 16), layer->cfg.inter) &&
+            const bool wide = ek::wide_cut_pays((n >> 7) + ((n & 127) > 16), n, H, layer->cfg.inter, layer->w8 ? 1 : 2) &&
                               wide_items <= layer->list_cap[ek::kListStream];
             ek::launch_single_lists(layer->lists, expert, (int32_t)n, wide, s);
             EK_TRY(enqueue_ffn(layer, d_x, nullptr, d_out, n, 1, s, nullptr, wide ? wide_items : 0));
@@ -1077,7 +1077,7 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
                 tile_items += (rows[i] >> 7) + ((rows[i] & 127) > 16);
                 wide_items += (rows[i] + ek::kWideRows - 1) / ek::kWideRows;
             }
-            const bool wide = ek::wide_cut_pays(tile_items, layer->cfg.inter) &&
+            const bool wide = ek::wide_cut_pays(tile_items, P, H, layer->cfg.inter, layer->w8 ? 1 : 2) &&
                               wide_items <= layer->list_cap[ek::kListStream];
             for (int i = 0; i < n_calls; ++i) {
                 const int32_t n = (int32_t)rows[i], full = n >> 7, r = n & 127;

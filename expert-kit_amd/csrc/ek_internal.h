@@ -62,11 +62,20 @@ struct WorkLists {
 };
 constexpr int kWideRows = 64;
 // tile_items: work items the ordinary cut would give the tile kernel; one of them spreads
-// over ceil(inter / 256) workgroups in stage 1.  Below half a chip of them the streaming
-// kernel, which spreads every item over inter / 16 workgroups, is faster (measured on MI355X).
-inline bool wide_cut_pays(int64_t tile_items, int64_t inter)
+// over ceil(inter / 256) workgroups in stage 1, and below half a chip of them the call takes as
+// long as one tile's two contractions however few rows it has: ~15 us + (hidden + inter) x
+// 25 ns (one-byte weights) or 28.5 ns (16-bit).  The streaming kernel spreads every item
+// over inter / 16 workgroups, each of which reads its item's rows, and its time grows with the
+// rows: ~ rows x (53 ns + hidden x inter x 14.8 fs).  Fitted on MI355X to one DeepSeek-V3
+// expert (hidden 7168, inter 2048; int8: 219 us streamed / 245 us tiled at 768 rows, 265 / 243
+// at 896; bf16: 230 / 274 at 768, 281 / 277 at 1024) and to the Qwen3 fp16 shape (2048, 768:
+// 76 ns per row streamed, 98 us tiled).
+inline bool wide_cut_pays(int64_t tile_items, int64_t rows, int64_t hidden, int64_t inter, int64_t weight_bytes)
 {
-    return tile_items > 0 && tile_items * ((inter + 255) / 256) < 128;
+    if (tile_items <= 0 || tile_items * ((inter + 255) / 256) >= 128) return false;
+    const double tiled_us = 15.0 + (double)(hidden + inter) * (weight_bytes == 1 ? 0.025 : 0.0285);
+    const double streamed_us = (double)rows * (0.053 + 1.48e-8 * (double)hidden * (double)inter);
+    return streamed_us < 0.92 * tiled_us;
 }
 inline int64_t list_capacity(int list, int64_t P, int64_t E)
 {

@@ -56,8 +56,7 @@ def test_batch_equals_individual_calls(ek, dt, w8):
     layer = make_layer(ek, dt, w8)
     # every size class, empty calls, repeated experts, calls in no particular expert order (the batch is
     # small enough that its longer calls are cut for the streaming kernel, as they are alone)
-    calls = [(3, 5), (0, 0), (1, 1), (5, 16), (2, 17), (3, 32), (4, 33), (0, 64), (1, 65), (2, 128), (5, 129),
-             (4, 300), (0, 7), (0, 0)]
+    calls = [(3, 5), (0, 0), (1, 1), (5, 16), (2, 17), (3, 32), (4, 33), (0, 64), (1, 65), (5, 129), (0, 7), (0, 0)]
     ids = [f"m/l3-e{e}" for e, _ in calls]
     xs = [x_rows(n, dt, 200 + i) for i, (_, n) in enumerate(calls)]
     resps = layer.worker_forward_batch(ids, [st_save({"data": x}) for x in xs])
@@ -73,6 +72,17 @@ def test_batch_equals_individual_calls(ek, dt, w8):
     for out, d in zip(outs, dev):
         assert d.is_cuda and torch.equal(bits(out), bits(d))
     assert layer.stats()["expert_forward_calls"] >= 3 * len(calls)
+    # a batch with enough rows for the tile kernel: its long calls take the other kernel family than
+    # they take alone, so the results agree as two evaluations of the same product do, not bit for bit
+    big = [(2, 128), (4, 300), (1, 200), (3, 9)]
+    xs = [x_rows(n, dt, 900 + i).cuda() for i, (_, n) in enumerate(big)]
+    outs = layer.experts_forward([e for e, _ in big], xs)
+    for (e, n), x, out in zip(big, xs, outs):
+        want = layer.expert_forward(e, x).float()
+        rms = float(want.pow(2).mean().sqrt())
+        assert float((out.float() - want).abs().max()) <= 2e-2 * rms, (e, n)
+        if n <= 16:
+            assert torch.equal(bits(out), bits(layer.expert_forward(e, x)))
     layer.close()
 
 
