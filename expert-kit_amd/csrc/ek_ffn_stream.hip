@@ -143,7 +143,12 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
         for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
             for (int m = 0; m < NMAT; ++m)
-                wq[d][gi * NMAT + m] = ldg16(wp[gi] + (int64_t)(kt * NMAT + m) * kChunkBytes);
+            {
+                // items of up to 16 rows: an expert's weights are read by one item (routed pairs) or a
+                // few; wide items come several to an expert and find them in the caches
+                const uint8_t *src = wp[gi] + (int64_t)(kt * NMAT + m) * kChunkBytes;
+                wq[d][gi * NMAT + m] = RS == 1 ? ldg16_once(src) : ldg16(src);
+            }
 #pragma unroll
         for (int rs = 0; rs < RS; ++rs)
             if (RS == 1 || rs < nfr) {
@@ -271,7 +276,7 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
 #define EK_TUNE_S2_NG 2
 #endif
 #ifndef EK_TUNE_S2_D
-#define EK_TUNE_S2_D 8
+#define EK_TUNE_S2_D 4
 #endif
 
 template <typename T, int WM, int NMAT, int NG, int D>
