@@ -8,8 +8,12 @@
 //   - the eight waves split the channels; each wave keeps every row of the
 //     tile, so a weight element is fetched and dequantised once per workgroup;
 //   - everything is brought in by LDS-DMA (global_load_lds_dwordx4: global ->
-//     LDS without passing through registers), three stages deep: while step s
-//     is being multiplied, the loads of steps s+1 and s+2 are in flight.  The
+//     LDS without passing through registers) in steps of 64 contraction
+//     elements, three stages deep with one-byte weights (while step s is being
+//     multiplied, the loads of steps s+1 and s+2 are in flight) and two stages
+//     deep with 16-bit weights, whose stage is 80 KiB (measured on MI355X
+//     against 32-element steps three deep: a lone bf16 DeepSeek-V3 expert
+//     runs 6 to 13 % faster, fewer barriers and waits per MFMA).  The
 //     weight chunks of a wave land in a wave-private region in exactly the
 //     chunked HBM layout (lane l's 16 bytes at l*16), the activation rows
 //     (gathered through row_token for stage 1) in an XOR-swizzled tile whose
@@ -66,15 +70,20 @@ __device__ __forceinline__ void block_barrier()
 
 constexpr int kTileThreads = 512;
 constexpr int kTileWaves = 8;
-constexpr int kTileStages = 3;
 constexpr int kCusPerXcd = 32;   // MI355X: 8 XCDs x 32 CUs
 
+// A step covers 64 contraction elements: one weight chunk per channel tile with one-byte
+// weights, two with 16-bit ones (KC).  One-byte weights run three stages deep (two steps of
+// loads in flight), 16-bit weights, whose stage is 80 KiB, two (one step in flight, of the
+// same length in time: the step has as many MFMAs and no conversion work).
 template <bool W8> struct TileGeom {
-    static constexpr int BK = W8 ? 64 : 32;          // contraction elements per step = per weight chunk
+    static constexpr int BK = 64;                    // contraction elements per step
+    static constexpr int KC = W8 ? 1 : 2;            // weight chunks along k per channel tile and step
     static constexpr int PPR = BK / 8;               // 16-byte pieces per activation row and step
     static constexpr int XS = 128 * BK * 2;          // bytes of a 128-row activation stage
-    static constexpr int WS = kTileWaves * 4 * kChunkBytes;
+    static constexpr int WS = kTileWaves * 4 * KC * kChunkBytes;
     static constexpr int STAGE = XS + WS;
+    static constexpr int STAGES = W8 ? 3 : 2;
 };
 
 // XOR key of a row: fragment reads of 16 consecutive rows and one piece index
@@ -111,15 +120,18 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     constexpr bool W8 = WM != kW16;            // one-byte weights
     using G = TileGeom<W8>;
     constexpr int NR = NMAT == 2 ? 2 : 4;      // channel tiles per wave and matrix
-    constexpr int NWC = NR * NMAT;             // weight chunks per wave and step (always 4)
+    constexpr int NWC = NR * NMAT;             // channel tiles x matrices per wave (always 4)
+    constexpr int KC = G::KC;
+    constexpr int NWCH = NWC * KC;             // weight chunks per wave and step
+    constexpr int NS = G::STAGES, AHEAD = NS - 1;   // stages; steps of loads in flight
     constexpr int BM = MR * 16;
     constexpr int BK = G::BK, PPR = G::PPR;
     constexpr int XINSTR = BM * PPR / 64;      // DMA instructions per activation stage
     constexpr int LX = (XINSTR + kTileWaves - 1) / kTileWaves;   // ... per wave
-    constexpr int LOADS = NWC + LX;            // DMAs per wave and stage
+    constexpr int LOADS = NWCH + LX;           // DMAs per wave and stage
     constexpr int CB = 2;                      // column blocks of 32 channels per wave
     constexpr int RB = MR / 2;                 // 32-row blocks
-    constexpr int NGRP = BK / 16;              // MFMA k-groups per step (4 int8, 2 16-bit)
+    constexpr int NGRP = BK / 16;              // MFMA k-groups per step
     constexpr int kRowBlockBytes = 32 * PPR * 16;
     static_assert(NWC == 4, "wave-private weight region holds 4 chunks");
     static_assert(RB >= 1, "items have at least 32 rows");
@@ -130,7 +142,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, l32 = lane & 31, kg = lane >> 5, hh = l32 >> 4;
     const int NT = a.N >> 4;
-    const int nsteps = a.Kdim / BK;             // >= 2 (hidden, inter >= 128)
+    const int nsteps = a.Kdim / BK;             // one-byte weights: >= 2 (hidden, inter >= 128)
 
     // ---- tile-independent lane constants ---------------------------------------
     // activation tile: DMA instruction q brings pieces q*64 .. q*64+63 (row-major, PPR per
@@ -145,18 +157,19 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
         xcol[i] = ((sidx % PPR) ^ swizzle_key<PPR>(xrow[i])) * 8;
         xdst[i] = q * 1024;
     }
-    const uint32_t w_off = G::XS + wave * (NWC * kChunkBytes);   // wave-private weight region
+    const uint32_t w_off = G::XS + wave * (NWCH * kChunkBytes);  // wave-private weight region
     // MFMA 32x32x16 operands.  The wave's 4 weight chunks (16 channels each) form CB = 2
     // column blocks of 32 channels: {up, gate} of the same 32 channels (stage 1) or 64
     // consecutive channels (stage 2).  Lane l feeds channel l%32 and k-half kg = l/32 of the
     // A operand, and row l%32 of a 32-row block of the B operand.  A 16-byte LDS read of
     // weight slot (2*tt + kg) gives the lane the A operands of two MFMAs (int8) or one
-    // (16-bit); the matching B operand is the 16-byte piece with the same k.
+    // (16-bit, whose two chunks per channel tile lie side by side: k-group grp is read grp);
+    // the matching B operand is the 16-byte piece with the same k.
     int aoff[CB];
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
         const int nr = NMAT == 2 ? hh : cb * 2 + hh, m = NMAT == 2 ? cb : 0;
-        aoff[cb] = (nr * NMAT + m) * kChunkBytes + kg * 256 + j * 16;
+        aoff[cb] = (nr * NMAT + m) * KC * kChunkBytes + kg * 256 + j * 16;
     }
     int boff[NGRP];
 #pragma unroll
@@ -171,7 +184,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     // each, so a step's scale is one number per column block; the tile's rows of the scale
     // matrices sit in a wave-private LDS area (two areas: the next tile's rows are fetched while
     // this one's are in use)
-    float *const sc_area = (float *)(lds + kTileStages * G::STAGE) + wave * (2 * kTileScaleBlocks);
+    float *const sc_area = (float *)(lds + NS * G::STAGE) + wave * (2 * kTileScaleBlocks);
     constexpr int kScaleSlotFloats = kTileWaves * 2 * kTileScaleBlocks;
     auto fetch = [&](int t, Ctx &c, int sslot) -> int {
         for (; t < ntiles; t += stride) {
@@ -187,7 +200,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 #pragma unroll
             for (int nr = 0; nr < NR; ++nr) {
                 const int ctc = min(cblock * NR + nr, NT - 1);   // tiles past N recompute the last one
-                c.wp[nr] = wmat + (int64_t)ctc * nsteps * (NMAT * kChunkBytes) + lane * 16;
+                c.wp[nr] = wmat + (int64_t)ctc * (nsteps * KC) * (NMAT * kChunkBytes) + lane * 16;
             }
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
@@ -228,8 +241,9 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
         const uint32_t st_ = lds_base + (ring) * G::STAGE;                                      \
         _Pragma("unroll") for (int nr = 0; nr < NR; ++nr)                                       \
         _Pragma("unroll") for (int m = 0; m < NMAT; ++m)                                        \
-            dma16((ctx).wp[nr] + (int64_t)((step) * NMAT + m) * kChunkBytes,                    \
-                  st_ + w_off + (nr * NMAT + m) * kChunkBytes);                                 \
+        _Pragma("unroll") for (int kc = 0; kc < KC; ++kc)                                       \
+            dma16((ctx).wp[nr] + (int64_t)(((step) * KC + kc) * NMAT + m) * kChunkBytes,        \
+                  st_ + w_off + ((nr * NMAT + m) * KC + kc) * kChunkBytes);                     \
         _Pragma("unroll") for (int i = 0; i < LX; ++i) dma16((ctx).xsrc[i] + (step) * BK, st_ + xdst[i]); \
     }
 
@@ -239,13 +253,13 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     int ring = 0;                                // stage of the current step
     block_barrier();                             // every wave has left the previous class's stages
     EK_ISSUE(cur, 0, 0);
-    EK_ISSUE(cur, 1, 1);
+    if constexpr (AHEAD == 2) EK_ISSUE(cur, 1, 1);
 
-    // The next tile's addresses are needed two steps before this one ends.  Fetching them
+    // The next tile's addresses are needed AHEAD steps before this one ends.  Fetching them
     // makes the wave wait on ordinary loads, i.e. on every vector-memory operation issued
-    // before them: it is done three steps before the end, right after the barrier and before
-    // the step's DMAs are issued, when only the next step's DMAs (a step old) are in flight.
-    const int fstep = nsteps > 3 ? nsteps - 3 : 0;
+    // before them: it is done a step earlier still, right after the barrier and before
+    // the step's DMAs are issued, when only DMAs that are a step old are in flight.
+    const int fstep = nsteps > AHEAD + 1 ? nsteps - AHEAD - 1 : 0;
     int pend_st = 0;   // global stores of the previous tile's epilogue, issued after the DMAs of
                        // this tile's first two steps (stores count in vmcnt like loads)
     while (true) {
@@ -264,27 +278,34 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
         for (int step = 0; step < nsteps; ++step) {
             // the DMAs of this step are older than those of the next one (of this tile or of
             // the next tile) and than the previous epilogue's stores: wait until only those remain
-            if (step + 1 < nsteps || tn >= 0) {
-                if (step < 2 && pend_st) wait_vmcnt_dyn(LOADS + pend_st);
-                else wait_vmcnt<LOADS>();
+            if constexpr (AHEAD == 2) {
+                if (step + 1 < nsteps || tn >= 0) {
+                    if (step < 2 && pend_st) wait_vmcnt_dyn(LOADS + pend_st);
+                    else wait_vmcnt<LOADS>();
+                } else {
+                    wait_vmcnt<0>();
+                }
             } else {
-                wait_vmcnt<0>();
+                // one step in flight: nothing younger than this step's DMAs but, at a tile's first
+                // step, the previous epilogue's stores
+                if (step == 0 && pend_st) wait_vmcnt_dyn(pend_st);
+                else wait_vmcnt<0>();
             }
             block_barrier();   // this step's tile is visible to all waves; the stage of the
                                // previous step is free again
             if (step == fstep) tn = fetch(tc + stride, nxt, cur.sslot ^ 1);
-            const int ring2 = ring == 0 ? 2 : ring - 1;          // (ring + 2) % 3
-            if (step + 2 < nsteps) {
-                EK_ISSUE(cur, step + 2, ring2);
+            const int ring2 = ring + AHEAD >= NS ? ring + AHEAD - NS : ring + AHEAD;   // (ring + AHEAD) % NS
+            if (step + AHEAD < nsteps) {
+                EK_ISSUE(cur, step + AHEAD, ring2);
             } else if (tn >= 0) {
-                EK_ISSUE(nxt, step + 2 - nsteps, ring2);
+                EK_ISSUE(nxt, step + AHEAD - nsteps, ring2);
             }
 
             const uint8_t *stage = lds + ring * G::STAGE;
             const uint8_t *wreg = stage + w_off;
-            u32x4 aq[2][CB];
+            u32x4 aq[W8 ? 2 : 1][CB];   // one-byte weights: the step's A operands as stored; 16-bit: the first k-group's
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
+            for (int tt = 0; tt < (W8 ? 2 : 1); ++tt)
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) aq[tt][cb] = *(const u32x4 *)(wreg + aoff[cb] + tt * 512);
 #pragma unroll
@@ -355,14 +376,14 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                     } else {
                         if (rb == 0) {
 #pragma unroll
-                            for (int cb = 0; cb < CB; ++cb) af[ng][cb] = aq[(grp + 1) % 2][cb];
+                            for (int cb = 0; cb < CB; ++cb) af[ng][cb] = *(const u32x4 *)(wreg + aoff[cb] + (grp + 1) * 512);
                         }
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
             static_assert(((NGRP - 1) & 1) == 1, "the last k-group's operands sit in af[1] / bf[1]");
-            ring = ring == 2 ? 0 : ring + 1;
+            ring = ring == NS - 1 ? 0 : ring + 1;
         }
         // the last step's last k-group
 #pragma unroll
@@ -385,7 +406,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
         block_barrier();
         pend_st = 0;
         if (cur.chan0 < a.N) {
-            uint8_t *scr = lds + (ring == 0 ? 2 : ring - 1) * G::STAGE + wave * (32 * RS);
+            uint8_t *scr = lds + (ring == 0 ? NS - 1 : ring - 1) * G::STAGE + wave * (32 * RS);
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
                 if (rb * 32 >= cur.nrows) break;
@@ -439,7 +460,7 @@ template <typename T, int WM, int NMAT>
 __global__ __launch_bounds__(kTileThreads, 1) void ffn_tile_kernel(FfnArgs a, int nb_count)
 {
     __shared__ __attribute__((aligned(1024)))
-    uint8_t lds[kTileStages * TileGeom<WM != kW16>::STAGE + (block_scaled(WM) ? kTileScaleBytes : 0)];
+    uint8_t lds[TileGeom<WM != kW16>::STAGES * TileGeom<WM != kW16>::STAGE + (block_scaled(WM) ? kTileScaleBytes : 0)];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)lds;
     const int x = blockIdx.x & 7, slot = blockIdx.x >> 3, nslots = gridDim.x >> 3;
     const int n128 = a.lists.count[kListT128], n64 = a.lists.count[kListT64], n32 = a.lists.count[kListT32];
