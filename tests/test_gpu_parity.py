@@ -243,6 +243,25 @@ def test_tile_route_one_expert(ek, oracle, cuda, dt, w8, n):
     layer.close()
 
 
+@pytest.mark.parametrize("H,I,w8", [(128, 64, False), (64, 128, False), (64, 64, False), (128, 128, True), (256, 128, True)])
+def test_tile_route_shortest_contractions(ek, oracle, cuda, H, I, w8):
+    """The tile kernel's pipeline at its shortest: contractions of one and two 64-element steps
+    (16-bit weights: two stages, one step in flight; int8: three stages, two steps in flight),
+    several tiles per workgroup so that the loads run across tile boundaries."""
+    dt = torch.bfloat16
+    n = 128 * 40 + 77
+    print(f"shortest contractions H={H} I={I} w8={w8}", flush=True)
+    w = wl.Workload("t", H, I, 1, 1, n, dt, w8=w8)
+    layer, ws = load_layer(ek, w, experts=[0])
+    x = torch.randn(n, H, generator=torch.Generator().manual_seed(H + I)).to(dt)
+    wu, wg, wd = [t[0] for t in oracle_weights(oracle, ws, 1, dt)]
+    ref = oracle.ffn(x, wu, wg, wd, mode=2)
+    got = layer.forward(x.to(cuda), torch.zeros(n, 1, dtype=torch.int32, device=cuda), torch.ones(n, 1, dtype=dt, device=cuda))
+    ffn_gate(got, ref, f"shortest contractions H={H} I={I} w8={w8}")
+    assert check_vs_rounded(got, ref) > 0.9
+    layer.close()
+
+
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("w8", [False, True])
 def test_streaming_forms_agree_bitwise(ek, cuda, dt, w8):
