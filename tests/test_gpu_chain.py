@@ -123,3 +123,46 @@ def test_chain_c5_full_shape_properties(ek, cuda):
     chain.close()
     for layer in layers:
         layer.close()
+
+
+@pytest.mark.parametrize("T,shared", [(8, False), (48, False), (100, True), (300, False)])
+def test_layer_call_in_the_callers_graph(ek, cuda, T, shared):
+    """A caller that captures ek_layer_forward on its own stream (the library forks its side
+    stream inside the capture and joins it again; no memset nodes, no allocation, no
+    synchronisation): every replay, with eager work of the same layer between the replays,
+    gives the eager call's bits.  T spans the regimes: streaming items only, both kernel
+    families side by side, a shared expert's segment in a launch of its own, tiles."""
+    dt, H, I, E, K = torch.float16, 256, 128, 8, 2
+    w = wl.Workload("cap", H, I, E + 1, K, T, dt)
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, max_tokens=T)
+    for e in range(E):
+        layer.set_expert(e, wl.make_expert(w, e, std=0.05))
+    if shared:
+        layer.set_shared_expert(wl.make_expert(w, E, std=0.05))
+    g = torch.Generator().manual_seed(T)
+    x = torch.randn(T, H, generator=g).to(dt).to(cuda)
+    p = torch.tensor([6.0] + [1.0] * (E - 1))                       # one hot expert: long and short segments
+    ids = torch.stack([torch.multinomial(p, K, generator=g) for _ in range(T)]).to(torch.int32).to(cuda)
+    gw = torch.rand(T, K, generator=g) + 0.1
+    gw = (gw / gw.sum(-1, keepdim=True)).to(dt).to(cuda)
+    y_eager = layer.forward(x, ids, gw).clone()
+    y = torch.empty_like(x)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        layer.forward(x, ids, gw, stream=side, out=y)               # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            layer.forward(x, ids, gw, stream=torch.cuda.current_stream(), out=y)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(bits(y), bits(y_eager)), f"replay {rep}"
+        other = layer.forward(x.flip(0).contiguous(), ids, gw)      # eager work on the same workspace
+        torch.cuda.synchronize()
+        assert other.shape == x.shape
+    layer.close()
+
