@@ -186,7 +186,10 @@ ek_status ek_layer_has_expert(ek_layer *layer, int32_t expert, int32_t *loaded);
  *   y   [T,H] act_dtype        route: optional routing tables (may be NULL)
  * T == 0 is legal and does nothing.  An id outside [0,E) gives
  * EK_INVALID_INPUT, a pair routed to an unloaded expert EK_EXPERT_NOT_FOUND
- * (both reported by blocking calls; y is then unspecified). */
+ * (both reported by blocking calls; y is then unspecified).
+ * With device pointers and a stream the call only enqueues (kernels, and events
+ * on a side stream of the library's that it forks from and joins to `stream`):
+ * it may be captured into the caller's HIP graph, whose grids depend on T only. */
 ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, const void *w,
                            int32_t w_dtype, int64_t T, void *y, const ek_route_out *route,
                            int32_t mem, void *stream);
