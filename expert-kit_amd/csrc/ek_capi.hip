@@ -83,7 +83,12 @@ int64_t elem_size(int dt)
 }  // namespace
 
 struct ek_layer {
-    ek_cfg cfg{};
+    ek_cfg cfg{};             // as the kernels see it: hidden and inter rounded up to what they need
+    // The caller's hidden and inter.  A layer whose sizes are not multiples of the kernels' 64
+    // (the reference's toy configurations, e.g. ds-tiny: hidden 16, intermediate 8) runs on
+    // zero-padded weights and on zero-padded copies of the activation rows: `padded`.
+    int64_t user_hidden = 0, user_inter = 0;
+    bool padded = false;
     int act = 0;        // 0 bf16, 1 f16
     bool w8 = false;          // one-byte weights (int8 per channel or fp8 per block)
     int wmode = 0;            // ek::WeightMode
@@ -223,12 +228,11 @@ ek_status validate_cfg(const ek_cfg *c)
     if ((c->w_dtype == EK_F8E4M3 || (c->flags & EK_CFG_BLOCK_SCALES)) && (c->hidden > 8192 || c->inter > 8192))
         return fail(EK_INVALID_INPUT, "block-scaled layers hold at most 64 scale blocks per row: hidden and "
                     "inter must not exceed 8192");
-    const int64_t ke = 64;   // contraction step of the tile kernel; int8 chunk width
-    // the tile kernel's pipeline needs two contraction steps (64 wide for int8, 32 for 16-bit)
-    const int64_t kmin = c->w_dtype == EK_I8 || c->w_dtype == EK_F8E4M3 ? 128 : 64;
-    if (c->hidden < kmin || c->inter < kmin || c->hidden % ke || c->inter % ke)
-        return fail(EK_INVALID_INPUT, "hidden (%lld) and inter (%lld) must be multiples of %lld (at least 128 for int8)",
-                    (long long)c->hidden, (long long)c->inter, (long long)ke);
+    // (the kernels want multiples of 64, at least 128 with one-byte weights: create_layer rounds up
+    // and pads; rows of x and y are moved 16 bytes at a time)
+    if (c->hidden < 8 || c->hidden % 8 || c->inter < 1)
+        return fail(EK_INVALID_INPUT, "hidden (%lld) must be a positive multiple of 8 and inter (%lld) positive",
+                    (long long)c->hidden, (long long)c->inter);
     if (c->n_experts < 1 || c->n_experts > ek::kMaxExperts)
         return fail(EK_INVALID_INPUT, "n_experts must be in [1, %d] (got %d)", ek::kMaxExperts,
                     c->n_experts);
@@ -250,6 +254,16 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     ek_layer *L = new (std::nothrow) ek_layer();
     if (!L) return fail(EK_OOM, "host allocation failed");
     L->cfg = *cfg;
+    L->user_hidden = cfg->hidden;
+    L->user_inter = cfg->inter;
+    {
+        const bool one_byte = cfg->w_dtype == EK_I8 || cfg->w_dtype == EK_F8E4M3;
+        auto up = [&](int64_t v) { return std::max<int64_t>((v + 63) / 64 * 64, one_byte ? 128 : 64); };
+        L->cfg.hidden = up(cfg->hidden);
+        L->cfg.inter = up(cfg->inter);
+        L->padded = L->cfg.hidden != cfg->hidden || L->cfg.inter != cfg->inter;
+        cfg = &L->cfg;                            // from here on: the kernels' sizes
+    }
     L->act = cfg->act_dtype == EK_BF16 ? 0 : 1;
     L->w8 = cfg->w_dtype == EK_I8 || cfg->w_dtype == EK_F8E4M3;
     L->wmode = cfg->w_dtype == EK_I8 ? ((cfg->flags & EK_CFG_BLOCK_SCALES) ? ek::kWI8Block : ek::kWI8)
@@ -493,6 +507,63 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
     return EK_OK;
 }
 
+// A padded layer's weights: zero-padded device copies of the caller's matrices (and scales) in
+// the kernels' sizes, handed to set_expert_locked as device sources.  Padded channels have
+// weight 0 (and scale 0), padded contraction elements meet the zero columns of the staged rows.
+ek_status set_expert_padded(ek_layer *L, int32_t e, const ek_weight_desc *up, const ek_weight_desc *gate,
+                            const ek_weight_desc *down)
+{
+    const int64_t UH = L->user_hidden, UI = L->user_inter, H = L->cfg.hidden, I = L->cfg.inter;
+    EK_TRY(check_desc(up, "up", UI, UH, L->wmode));
+    EK_TRY(check_desc(gate, "gate", UI, UH, L->wmode));
+    EK_TRY(check_desc(down, "down", UH, UI, L->wmode));
+    const ek_weight_desc *src[3] = {up, gate, down};
+    const int64_t pr[3] = {I, I, H}, pc[3] = {H, H, I};
+    ek_weight_desc padded[3];
+    std::vector<void *> tmp;
+    ek_status st = EK_OK;
+    for (int i = 0; i < 3 && st == EK_OK; ++i) {
+        const ek_weight_desc *d = src[i];
+        const hipMemcpyKind kind = d->mem == EK_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice;
+        padded[i] = *d;
+        padded[i].rows = pr[i];
+        padded[i].cols = pc[i];
+        padded[i].mem = EK_DEVICE;
+        const size_t es = (size_t)elem_size(d->dtype);
+        void *w = nullptr;
+        st = dev_alloc(&w, (size_t)pr[i] * pc[i] * es, "padded weights");
+        if (st != EK_OK) break;
+        tmp.push_back(w);
+        padded[i].ptr = w;
+        hipError_t er = hipMemsetAsync(w, 0, (size_t)pr[i] * pc[i] * es, L->load_stream);
+        if (er == hipSuccess)
+            er = hipMemcpy2DAsync(w, (size_t)pc[i] * es, d->ptr, (size_t)d->cols * es, (size_t)d->cols * es,
+                                  (size_t)d->rows, kind, L->load_stream);
+        if (er == hipSuccess && d->scale_kind != EK_SCALE_NONE && d->scale) {
+            const size_t ses = (size_t)elem_size(d->scale_dtype);
+            const bool per_channel = d->scale_kind == EK_SCALE_PER_CHANNEL;
+            // per channel: one row of `rows` scales; per block: a [ceil(rows/128), ceil(cols/128)] grid
+            const size_t ur = per_channel ? 1 : (size_t)(d->rows + 127) / 128, uc = per_channel ? (size_t)d->rows : (size_t)(d->cols + 127) / 128;
+            const size_t qr = per_channel ? 1 : (size_t)(pr[i] + 127) / 128, qc = per_channel ? (size_t)pr[i] : (size_t)(pc[i] + 127) / 128;
+            void *sc = nullptr;
+            st = dev_alloc(&sc, qr * qc * ses, "padded scales");
+            if (st != EK_OK) break;
+            tmp.push_back(sc);
+            padded[i].scale = sc;
+            er = hipMemsetAsync(sc, 0, qr * qc * ses, L->load_stream);
+            if (er == hipSuccess)
+                er = hipMemcpy2DAsync(sc, qc * ses, d->scale, uc * ses, uc * ses, ur, kind, L->load_stream);
+        }
+        if (er != hipSuccess) st = hip_fail(er, "padding the weights");
+    }
+    if (st == EK_OK) st = set_expert_locked(L, e, &padded[0], &padded[1], &padded[2]);   // (waits for the copies)
+    std::string keep = g_last_error;
+    (void)hipStreamSynchronize(L->load_stream);
+    for (void *p : tmp) (void)hipFree(p);
+    g_last_error = keep;
+    return st;
+}
+
 struct Timer {
     std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
     double us() const
@@ -518,6 +589,10 @@ ek_status ensure_io_staging(ek_layer *L)
     // st_x / st_y also serve ek_layer_expert_forward, whose n may reach Pmax
     const int64_t rows = L->Pmax > T ? L->Pmax : T;
     EK_TRY(dev_alloc(&L->st_x, (size_t)rows * H * 2, "x staging"));
+    if (L->padded) {                                   // the padding columns stay zero from here on
+        EK_HIP(hipMemset(L->st_x, 0, (size_t)rows * H * 2));
+        EK_HIP(hipDeviceSynchronize());
+    }
     EK_TRY(dev_alloc(&L->st_y, (size_t)rows * H * 2, "y staging"));
     EK_TRY(dev_alloc(&L->st_w, (size_t)T * K * 4, "gate-weight staging"));
     EK_TRY(dev_alloc((void **)&L->st_ids, (size_t)T * K * 4, "ids staging"));
@@ -583,6 +658,27 @@ ek_status d2h(ek_layer *L, void *dst, const void *src, size_t bytes, hipStream_t
     } else {
         EK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
     }
+    return EK_OK;
+}
+
+// Rows of a padded layer: n rows of the caller's hidden size between the caller's buffer
+// (host or device, rows back to back) and a staging buffer whose rows have the kernels'
+// hidden size (its padding columns are zero and are never written).
+ek_status rows_in(ek_layer *L, void *staged, const void *src, int64_t n, int mem, hipStream_t s)
+{
+    if (n <= 0) return EK_OK;
+    const size_t w = (size_t)L->user_hidden * 2;
+    EK_HIP(hipMemcpy2DAsync(staged, (size_t)L->cfg.hidden * 2, src, w, w, (size_t)n,
+                            mem == EK_HOST ? hipMemcpyHostToDevice : hipMemcpyDeviceToDevice, s));
+    return EK_OK;
+}
+
+ek_status rows_out(ek_layer *L, void *dst, const void *staged, int64_t n, int mem, hipStream_t s)
+{
+    if (n <= 0) return EK_OK;
+    const size_t w = (size_t)L->user_hidden * 2;
+    EK_HIP(hipMemcpy2DAsync(dst, w, staged, (size_t)L->cfg.hidden * 2, w, (size_t)n,
+                            mem == EK_HOST ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice, s));
     return EK_OK;
 }
 
@@ -832,6 +928,10 @@ ek_status ek_layer_set_expert(ek_layer *layer, int32_t expert, const ek_weight_d
         DeviceGuard dg(layer->cfg.device_id);
         if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
         std::lock_guard<std::mutex> lk(layer->load_mu);
+        if (layer->padded) {
+            if (!up || !gate || !down) return fail(EK_WEIGHT_NOT_FOUND, "a weight matrix is missing");
+            return set_expert_padded(layer, expert, up, gate, down);
+        }
         return set_expert_locked(layer, expert, up, gate, down);
     )
 }
@@ -897,7 +997,22 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
         ek_status st = EK_OK;
         // a blocking call on device buffers sees everything submitted before it
         if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
-        if (mem == EK_DEVICE) {
+        if (layer->padded) {
+            EK_TRY(ensure_io_staging(layer));
+            const int32_t *d_ids = ids;
+            const void *d_w = w;
+            if (mem == EK_HOST && T > 0) {
+                EK_HIP(hipMemcpyAsync(layer->st_ids, ids, (size_t)P * 4, hipMemcpyHostToDevice, s));
+                EK_HIP(hipMemcpyAsync(layer->st_w, w, (size_t)P * (w_f32 ? 4 : 2), hipMemcpyHostToDevice, s));
+                d_ids = layer->st_ids;
+                d_w = layer->st_w;
+            }
+            EK_TRY(rows_in(layer, layer->st_x, x, T, mem, s));
+            EK_TRY(enqueue_forward(layer, layer->st_x, d_ids, d_w, w_f32, T, layer->st_y, s));
+            EK_TRY(rows_out(layer, y, layer->st_y, T, mem, s));
+            EK_TRY(copy_route_out(layer, route, P, mem, s));
+            if (!stream) st = finish_blocking(layer, s);
+        } else if (mem == EK_DEVICE) {
             EK_TRY(enqueue_forward(layer, x, ids, w, w_f32, T, y, s));
             EK_TRY(copy_route_out(layer, route, P, mem, s));
             if (!stream) st = finish_blocking(layer, s);
@@ -941,7 +1056,7 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
             return fail(EK_INVALID_INPUT, "host-memory calls are blocking: stream must be NULL");
         DeviceGuard dg(layer->cfg.device_id);
         if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", layer->cfg.device_id);
-        const int64_t H = layer->cfg.hidden, K = layer->cfg.top_k, P = T * K;
+        const int64_t H = layer->user_hidden, K = layer->cfg.top_k, P = T * K;   // rows are gathered as the caller has them
         std::lock_guard<std::mutex> lk(layer->mu);
         hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
         if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
@@ -963,6 +1078,8 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
         if (xp) ek::launch_gather(d_x, layer->row_token, P, H * 2, d_xp, s);
         EK_HIP(hipGetLastError());
         if (mem == EK_HOST && xp && P > 0) EK_TRY(d2h(layer, xp, d_xp, (size_t)P * H * 2, s));
+        // the rows went into the staging buffer back to back: give a padded layer its zero columns back
+        if (layer->padded && mem == EK_HOST && xp && T > 0) EK_HIP(hipMemsetAsync(layer->st_x, 0, (size_t)T * H * 2, s));
         EK_TRY(copy_route_out(layer, route, P, mem, s));
         if (!stream) return finish_blocking(layer, s);
         return EK_OK;
@@ -995,7 +1112,12 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
         if (n > 0) {
             const void *d_x = x;
             void *d_out = out;
-            if (mem == EK_HOST) {
+            if (layer->padded) {
+                EK_TRY(ensure_io_staging(layer));
+                EK_TRY(rows_in(layer, layer->st_x, x, n, mem, s));
+                d_x = layer->st_x;
+                d_out = layer->st_y;
+            } else if (mem == EK_HOST) {
                 EK_TRY(ensure_io_staging(layer));
                 EK_TRY(bounce_begin(layer, s, (size_t)n * H * 2));
                 EK_TRY(h2d(layer, layer->st_x, x, (size_t)n * H * 2, s));
@@ -1008,7 +1130,8 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
                               wide_items <= layer->list_cap[ek::kListStream];
             ek::launch_single_lists(layer->lists, expert, (int32_t)n, wide, s);
             EK_TRY(enqueue_ffn(layer, d_x, nullptr, d_out, n, 1, s, nullptr, wide ? wide_items : 0));
-            if (mem == EK_HOST) EK_TRY(d2h(layer, out, layer->st_y, (size_t)n * H * 2, s));
+            if (layer->padded) EK_TRY(rows_out(layer, out, layer->st_y, n, mem, s));
+            else if (mem == EK_HOST) EK_TRY(d2h(layer, out, layer->st_y, (size_t)n * H * 2, s));
         }
         if (!stream) {
             EK_HIP(hipStreamSynchronize(s));
@@ -1028,8 +1151,8 @@ ek_status ek_layer_describe(ek_layer *layer, int64_t *hidden, int64_t *inter, in
                             int32_t *top_k, int32_t *act_dtype)
 {
     if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
-    if (hidden) *hidden = layer->cfg.hidden;
-    if (inter) *inter = layer->cfg.inter;
+    if (hidden) *hidden = layer->user_hidden;
+    if (inter) *inter = layer->user_inter;
     if (n_experts) *n_experts = layer->cfg.n_experts;
     if (top_k) *top_k = layer->cfg.top_k;
     if (act_dtype) *act_dtype = layer->cfg.act_dtype;
@@ -1128,7 +1251,7 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             // call, as much as the memcpy of a decode-sized request).
             const size_t all_bytes = (size_t)P * H * 2;
             bool one_transfer = false;
-            if (mem == EK_HOST) {
+            if (mem == EK_HOST && !layer->padded) {
                 EK_TRY(bounce_begin(layer, s, all_bytes));
                 one_transfer = n_calls > 1 && all_bytes <= layer->pin_cap;
             }
@@ -1143,7 +1266,9 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             }
             row0 = 0;
             for (int i = 0; i < n_calls && !one_transfer; ++i) {
-                if (rows[i] && mem == EK_HOST)
+                if (layer->padded)
+                    EK_TRY(rows_in(layer, (char *)layer->st_x + row0 * H * 2, xs[i], rows[i], mem, s));
+                else if (rows[i] && mem == EK_HOST)
                     EK_TRY(h2d(layer, (char *)layer->st_x + row0 * H * 2, xs[i], (size_t)rows[i] * H * 2, s));
                 else if (rows[i])
                     EK_HIP(hipMemcpyAsync((char *)layer->st_x + row0 * H * 2, xs[i], (size_t)rows[i] * H * 2,
@@ -1162,7 +1287,9 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
                 }
             }
             for (int i = 0; i < n_calls && !one_transfer; ++i) {
-                if (rows[i] && mem == EK_HOST)
+                if (layer->padded)
+                    EK_TRY(rows_out(layer, outs[i], (char *)layer->st_y + row0 * H * 2, rows[i], mem, s));
+                else if (rows[i] && mem == EK_HOST)
                     EK_TRY(d2h(layer, outs[i], (char *)layer->st_y + row0 * H * 2, (size_t)rows[i] * H * 2, s));
                 else if (rows[i])
                     EK_HIP(hipMemcpyAsync(outs[i], (char *)layer->st_y + row0 * H * 2, (size_t)rows[i] * H * 2,
@@ -1282,6 +1409,9 @@ ek_status ek_chain_create(ek_layer *const *layers, int32_t n_layers, ek_chain **
             return fail(EK_INVALID_INPUT, "n_layers must be in [1, 1024]");
         for (int i = 0; i < n_layers; ++i) {
             if (!layers[i]) return fail(EK_INVALID_INPUT, "layer %d is NULL", i);
+            if (layers[i]->padded)
+                return fail(EK_INVALID_INPUT, "layer %d runs on padded copies of its rows (hidden or inter is not a "
+                            "multiple of 64): not in a chain", i);
             const ek_cfg &a = layers[0]->cfg, &b = layers[i]->cfg;
             if (a.hidden != b.hidden || a.top_k != b.top_k || a.act_dtype != b.act_dtype ||
                 a.device_id != b.device_id || a.max_tokens != b.max_tokens)
@@ -1437,7 +1567,8 @@ ek_status ek_expert_create(const ek_cfg *cfg, int64_t max_rows, const ek_weight_
         ek_status st;
         {
             std::lock_guard<std::mutex> lk(L->load_mu);
-            st = set_expert_locked(L, 0, up, gate, down);
+            if (L->padded && (!up || !gate || !down)) st = fail(EK_WEIGHT_NOT_FOUND, "a weight matrix is missing");
+            else st = L->padded ? set_expert_padded(L, 0, up, gate, down) : set_expert_locked(L, 0, up, gate, down);
         }
         if (st != EK_OK) {
             std::string keep = g_last_error;
@@ -1463,8 +1594,8 @@ ek_status ek_expert_forward(ek_expert *expert, const void *x, int64_t n, void *o
 ek_status ek_expert_shape(ek_expert *expert, int64_t *hidden, int64_t *inter)
 {
     if (!expert || !expert->layer || !hidden || !inter) return fail(EK_INVALID_INPUT, "NULL argument");
-    *hidden = expert->layer->cfg.hidden;
-    *inter = expert->layer->cfg.inter;
+    *hidden = expert->layer->user_hidden;
+    *inter = expert->layer->user_inter;
     return EK_OK;
 }
 
@@ -1570,13 +1701,19 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
         EK_TRY(bounce_begin(layer, s, l_bytes + (size_t)T * H * 2 + (size_t)E * 4));
         if (T > 0) {
             EK_TRY(h2d(layer, layer->st_logits, logits, l_bytes, s));
-            if (forward) EK_TRY(h2d(layer, layer->st_x, x, (size_t)T * H * 2, s));
+            if (forward && !layer->padded) EK_TRY(h2d(layer, layer->st_x, x, (size_t)T * H * 2, s));
         }
         if (rcfg->bias) {
             EK_TRY(h2d(layer, layer->st_bias, rcfg->bias, (size_t)E * 4, s));
             d_bias = layer->st_bias;
         }
         d_logits = layer->st_logits;
+        d_x = layer->st_x;
+        d_y = layer->st_y;
+    }
+    if (forward && layer->padded) {
+        EK_TRY(ensure_io_staging(layer));
+        EK_TRY(rows_in(layer, layer->st_x, x, T, mem, s));
         d_x = layer->st_x;
         d_y = layer->st_y;
     }
@@ -1591,7 +1728,8 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
     ek_status st = EK_OK;
     if (forward) {
         EK_TRY(enqueue_forward(layer, d_x, layer->rt_ids, layer->rt_w, w_f32, T, d_y, s));
-        if (mem == EK_HOST && T > 0) EK_TRY(d2h(layer, y, layer->st_y, (size_t)T * H * 2, s));
+        if (layer->padded) EK_TRY(rows_out(layer, y, layer->st_y, T, mem, s));
+        else if (mem == EK_HOST && T > 0) EK_TRY(d2h(layer, y, layer->st_y, (size_t)T * H * 2, s));
         EK_TRY(copy_route_out(layer, route, P, mem, s));
         if (!stream) st = finish_blocking(layer, s);
         std::lock_guard<std::mutex> sl(layer->stats_mu);

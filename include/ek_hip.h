@@ -75,8 +75,12 @@ typedef enum ek_scale_kind {
 /* Stands for EKInstance{hidden, intermediate, backend} (ek-computation/src/x.rs:27-32)
  * plus the inference settings it is filled from (ek-base/src/config.rs:26-31). */
 typedef struct ek_cfg {
-    int64_t hidden;     /* H: a multiple of 64 (at least 128 with one-byte weights) */
-    int64_t inter;      /* I  (moe_intermediate_size): likewise */
+    int64_t hidden;     /* H: a positive multiple of 8.  The kernels take multiples of 64 (at least 128
+                           with one-byte weights); other sizes (the reference's toy models: ds-tiny has
+                           hidden 16, intermediate 8) are served zero-padded: the weights once at load,
+                           every call's rows through the layer's staging buffers, also for device
+                           memory.  Same results; such a layer cannot join a chain. */
+    int64_t inter;      /* I  (moe_intermediate_size): any positive size, padded likewise */
     int32_t n_experts;  /* E  experts owned by one layer object */
     int32_t top_k;      /* K  slots per token */
     int32_t act_dtype;  /* ek_dtype of x, y and the gate weights: EK_BF16 or EK_F16 */

@@ -35,13 +35,13 @@ def test_invalid_cfg_is_reported_not_fatal(ek):
     lib = ek.load()
     h = ctypes.c_void_p()
     bad = [
-        dict(hidden=100, inter=64),                 # not a multiple of 32
+        dict(hidden=100, inter=64),                 # rows are moved 16 bytes at a time
+        dict(hidden=0), dict(inter=0),
         dict(act_dtype=C.EK_F32),
         dict(w_dtype=C.EK_F16),                     # neither act dtype nor int8
         dict(n_experts=0), dict(n_experts=5000),
         dict(top_k=0), dict(top_k=99),
         dict(max_tokens=0), dict(max_tokens=1 << 40),
-        dict(hidden=96, w_dtype=C.EK_I8),           # int8 needs multiples of 64
     ]
     base = dict(hidden=128, inter=64, n_experts=8, top_k=2, act_dtype=C.EK_BF16, w_dtype=C.EK_BF16,
                 max_tokens=16, device_id=0, flags=0)

@@ -1,0 +1,176 @@
+"""Layers whose hidden / intermediate sizes the kernels do not take as they are.
+
+The reference's toy checkpoints are this small (ds-tiny: hidden 16, intermediate 8); the library
+keeps such a layer zero-padded to the kernels' sizes and moves the caller's rows through its
+staging buffers.  Bars: those of test_gpu_parity.py against the oracle at the caller's sizes
+(zero weights and zero activations add nothing to any sum, so no bar is loosened), bit-equal
+results between host- and device-memory calls, and the caller's sizes in every shape query.
+"""
+import pytest
+import torch
+
+from ek_hip import _capi as C
+from ek_hip import workloads as wl
+from test_gpu_block_scaled import KINDS, make_expert as make_block_expert, ref_weights
+from test_gpu_parity import TOL, check_vs_rounded, ffn_gate, layer_gate, oracle_weights, ulp_of
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [(16, 8), (72, 100), (200, 24), (64, 1), (8, 300)]
+
+
+def gate(oracle, got, x, wu, wg, wd, name):
+    """test_gpu_parity's one-expert gate.  Below 64 intermediate channels an output is the sum of so
+    few terms that one of them can be most of it, and the reference's own storage roundings of that
+    term (up, gate, silu, their product: four, and a result that takes another summation order may
+    land one step of 2^-8 (bf16) / 2^-11 (fp16) away at each) are no longer small against the
+    output RMS: there the bound adds that budget, 4 steps * sum_j |h_j| |W_down[i, j]|."""
+    ref, h = oracle.ffn(x, wu, wg, wd, mode=2, return_h=True)
+    if wu.shape[0] >= 64:
+        ffn_gate(got, ref, name, small=2)
+        return ref
+    step = 2.0 ** (-8 if x.dtype == torch.bfloat16 else -11)
+    budget = 4 * step * (h.float().abs() @ wd.float().abs().T)
+    rms = float(ref.pow(2).mean().sqrt())
+    err = (got.float().cpu() - ref).abs()
+    print(f"{name}: max|err|/rms = {float(err.max()) / rms:.3e}, over 2e-2*rms: {float((err > TOL * rms).float().mean()):.2e}", flush=True)
+    assert bool((err <= TOL * rms + 0.5 * ulp_of(ref, got.dtype) * 1.0001 + budget).all())
+    assert float((err > TOL * rms).float().mean()) <= 1e-3
+    return ref
+
+
+@pytest.mark.parametrize("H,I", SHAPES)
+@pytest.mark.parametrize("dt,w8", [(torch.bfloat16, False), (torch.float16, False), (torch.bfloat16, True)])
+def test_one_expert(ek, oracle, cuda, H, I, dt, w8):
+    for n in (1, 5, 16, 33, 130, 300):
+        print(f"odd shape expert H={H} I={I} dt={dt} w8={w8} n={n}", flush=True)
+        w = wl.Workload("t", H, I, 1, 1, n, dt, w8=w8)
+        ew = wl.make_expert(w, 0)
+        if not w8:
+            ew = ek.ExpertWeight(ew.up_w * 16, ew.gate_w * 16, ew.down_w * 16)
+        ffn = ek.HipFFN.construct(ek.EKInstance(H, I), ew, act_dtype=dt, max_rows=512)
+        assert ffn.shape() == (H, I)
+        x = torch.randn(n, H, generator=torch.Generator().manual_seed(n)).to(dt)
+        wu, wg, wd = [t[0] for t in oracle_weights(oracle, {0: ew}, 1, dt)]
+        got = ffn.forward(x.to(cuda))
+        assert got.shape == (n, H)
+        ref = gate(oracle, got, x, wu, wg, wd, f"odd H={H} I={I} w8={w8} n={n}")
+        if I >= 64:
+            check_vs_rounded(got, ref, "odd")
+        assert torch.equal(got.cpu().view(torch.int16), ffn.forward(x).view(torch.int16))
+        ffn.close()
+
+
+@pytest.mark.parametrize("H,I", SHAPES[:3])
+@pytest.mark.parametrize("dt,w8", [(torch.bfloat16, False), (torch.float16, True)])
+def test_layer(ek, oracle, cuda, H, I, dt, w8):
+    E, K = 8, 2
+    for T in (1, 17, 200):
+        print(f"odd shape layer H={H} I={I} dt={dt} w8={w8} T={T}", flush=True)
+        w = wl.Workload("odd", H, I, E, K, T, dt, w8=w8)
+        ws = {e: wl.make_expert(w, e, std=0.08) for e in range(E)}
+        layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=torch.int8 if w8 else dt, max_tokens=256)
+        for e in range(E):
+            layer.set_expert(e, ws[e])
+        x = wl.make_x(w)
+        ids, gw = wl.make_routing(w)
+        y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
+        assert y.shape == (T, H)
+        wu, wg, wd = oracle_weights(oracle, ws, E, dt)
+        ref, counts, offsets, perm, inv, y3 = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=2, return_y3=True)
+        for a, b in zip((rt.counts, rt.offsets, rt.perm, rt.inv_perm), (counts, offsets, perm, inv)):
+            assert torch.equal(a.cpu(), b)
+        if I >= 64:
+            layer_gate(y, ref, y3, gw, f"odd layer H={H} I={I}", small=2)
+        else:       # gate()'s budget, pair by pair, on top of the layer gate's own quanta
+            step = 2.0 ** (-8 if dt == torch.bfloat16 else -11)
+            budget = torch.zeros(T, H)
+            for k in range(K):
+                for e in ids[:, k].unique().tolist():
+                    rows = ids[:, k] == e
+                    h = oracle.ffn(x[rows], wu[e], wg[e], wd[e], mode=2, return_h=True)[1]
+                    budget[rows] += gw[rows, k, None].float().abs() * (h.float().abs() @ wd[e].float().abs().T)
+            rms = float(ref.pow(2).mean().sqrt())
+            err = (y.float().cpu() - ref).abs()
+            quanta = ulp_of((gw.float().unsqueeze(-1) * y3.float()).abs().amax(dim=1), dt) + 0.5 * ulp_of(ref, dt) * 1.0001
+            print(f"odd layer H={H} I={I} T={T}: max|err|/rms = {float(err.max()) / rms:.3e}", flush=True)
+            assert bool((err <= TOL * rms + quanta + 4 * step * budget).all())
+            assert float((err > TOL * rms).float().mean()) <= 1e-3
+        assert torch.equal(layer.forward(x, ids, gw).view(torch.int16), y.cpu().view(torch.int16))
+        # the per-expert and batched calls of the same layer
+        xe = x[:min(T, 40)]
+        one = layer.expert_forward(3, xe.to(cuda))
+        gate(oracle, one, xe, wu[3], wg[3], wd[3], "odd layer expert")
+        many = layer.experts_forward([3, 5, 3], [xe.to(cuda), xe[:1].to(cuda), xe.to(cuda)])
+        assert torch.equal(many[0].view(torch.int16), one.view(torch.int16))
+        assert torch.equal(many[2].view(torch.int16), one.view(torch.int16))
+        gate(oracle, many[1], xe[:1], wu[5], wg[5], wd[5], "odd layer batch")
+        many_host = layer.experts_forward([3, 5], [xe, xe[:1]])
+        assert torch.equal(many_host[0].view(torch.int16), one.cpu().view(torch.int16))
+        # router in front: the same result as routing first and calling forward with its tables
+        lg = torch.randn(T, E, generator=torch.Generator().manual_seed(T))
+        yl, lids, lw = layer.forward_logits(x.to(cuda), lg.to(cuda), ek.RouterConfig(kind=0))
+        assert torch.equal(yl.view(torch.int16), layer.forward(x.to(cuda), lids, lw).view(torch.int16))
+        hy, hids, hw = layer.forward_logits(x, lg, ek.RouterConfig(kind=0))
+        assert torch.equal(hy.view(torch.int16), yl.cpu().view(torch.int16)) and torch.equal(hids, lids.cpu())
+        # the shared expert rides along, padded like the routed ones
+        layer.set_shared_expert(ws[1])
+        ysh = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda))
+        ref_sh = oracle.add_shared(ref.to(dt), x, wu[1], wg[1], wd[1], rounded=False)
+        err = (ysh.float().cpu() - ref_sh).abs()
+        rms = float(ref_sh.pow(2).mean().sqrt())
+        quanta = 0.5 * ulp_of(ref_sh, dt) * 1.0001 + ulp_of(ref, dt) + ulp_of(ref_sh - ref.to(dt).float(), dt)
+        assert bool((err <= TOL * rms + quanta).all()), float(err.max()) / rms
+        layer.remove_expert(C.EK_SHARED_EXPERT)
+        assert torch.equal(layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda)).view(torch.int16), y.view(torch.int16))
+        # gather hands the caller's rows back at the caller's width (host call: through the staging rows)
+        _, xph = layer.pack(ids, x)
+        assert torch.equal(xph.view(torch.int16), x[(perm // K).long()].view(torch.int16))
+        assert torch.equal(layer.forward(x, ids, gw).view(torch.int16), y.cpu().view(torch.int16))
+        _, xp = layer.pack(ids.to(cuda), x.to(cuda))
+        assert torch.equal(xp.cpu().view(torch.int16), x[(perm // K).long()].view(torch.int16))
+        layer.close()
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
+@pytest.mark.parametrize("H,I", [(40, 24), (200, 136), (264, 72)])
+def test_block_scaled(ek, oracle, cuda, H, I, kind):
+    """The scale grid is padded with the matrices: [ceil(I/128), ceil(H/128)] at the caller's sizes."""
+    dt = torch.bfloat16
+    layer = ek.HipLayer(H, I, 2, 1, act_dtype=dt, max_tokens=256, **KINDS[kind])
+    ew = make_block_expert(ek, H, I, 5, kind)
+    layer.set_expert(1, ew)
+    for n in (1, 16, 70, 200):
+        print(f"odd shape block-scaled {kind} H={H} I={I} n={n}", flush=True)
+        x = torch.randn(n, H, generator=torch.Generator().manual_seed(n)).to(dt)
+        got = layer.expert_forward(1, x.to(cuda))
+        gate(oracle, got, x, *ref_weights(oracle, ew, dt), f"odd block {kind} H={H} I={I} n={n}")
+    layer.close()
+
+
+def test_wire_and_shapes(ek, oracle, cuda):
+    """ds-tiny's expert over the wire shim: safetensors in and out at the model's own sizes."""
+    from safetensors.torch import load as st_load, save as st_save
+    H, I, E = 16, 8, 4
+    dt = torch.bfloat16
+    w = wl.Workload("ds-tiny", H, I, E, 2, 8, dt)
+    ws = {e: wl.make_expert(w, e, std=0.5) for e in range(E)}
+    layer = ek.HipLayer(H, I, E, 2, act_dtype=dt, w_dtype=dt, max_tokens=64)
+    for e in range(E):
+        layer.set_expert(e, ws[e])
+    x = wl.make_x(w)
+    wu, wg, wd = oracle_weights(oracle, ws, E, dt)
+    reply = st_load(layer.worker_forward("ds-tiny/l0-e2", st_save({"data": x})))["data"]
+    assert reply.shape == (8, H) and reply.dtype == dt
+    gate(oracle, reply, x, wu[2], wg[2], wd[2], "ds-tiny wire")
+    assert torch.equal(reply.view(torch.int16), layer.expert_forward(2, x).view(torch.int16))
+    # a chain wants the kernels' own sizes
+    with pytest.raises(ek.EKError) as ei:
+        ek.HipChain([layer])
+    assert ei.value.status == C.EK_INVALID_INPUT
+    # weights of the wrong size are refused by the caller's sizes
+    bad = wl.make_expert(wl.Workload("b", 64, 64, 1, 1, 1, dt), 0)
+    with pytest.raises(ek.EKError) as ei:
+        layer.set_expert(0, bad)
+    assert ei.value.status == C.EK_INVALID_INPUT
+    layer.close()
