@@ -174,3 +174,50 @@ def test_wire_and_shapes(ek, oracle, cuda):
         layer.set_expert(0, bad)
     assert ei.value.status == C.EK_INVALID_INPUT
     layer.close()
+
+
+def test_ds_tiny_layer_as_configured(ek, oracle, cuda):
+    """The MoE layer of the reference's ds-tiny model (ek-db/resources/ds-tiny/config.json: hidden 16,
+    moe_intermediate_size 8, 256 routed experts, 8 per token out of 4 of 8 groups, sigmoid scores with
+    a correction bias, scaling 2.5, one shared expert, float32 tensors) end to end: router, pack,
+    grouped FFN, combine, shared expert.  The checkpoint itself is a large-file pointer in the
+    reference's tree, so the weights here are random ones of its shapes and dtype."""
+    H, I, E, K, T = 16, 8, 256, 8, 96
+    dt = torch.bfloat16
+    g = torch.Generator().manual_seed(2024)
+    f32 = [ek.ExpertWeight(up_w=torch.randn(I, H, generator=g) * 0.4, gate_w=torch.randn(I, H, generator=g) * 0.4,
+                           down_w=torch.randn(H, I, generator=g) * 0.4) for _ in range(E + 1)]
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=dt, max_tokens=128)
+    for e in range(E):
+        layer.set_expert(e, f32[e])                 # float32 sources are rounded to the layer's dtype at load
+    layer.set_shared_expert(f32[E])
+    wu, wg, wd = ([w.up_w.to(dt) for w in f32], [w.gate_w.to(dt) for w in f32], [w.down_w.to(dt) for w in f32])
+    x = torch.randn(T, H, generator=g).to(dt)
+    lg = torch.randn(T, E, generator=g)
+    bias = torch.randn(E, generator=g) * 0.1
+    r = ek.RouterConfig(kind=4, renorm=True, n_group=8, topk_group=4, routed_scaling=2.5, w_dtype=torch.float32, bias=bias)
+    y, ids, w = layer.forward_logits(x.to(cuda), lg.to(cuda), r)
+    o_ids, o_w = oracle.route(4, lg, K, True, w_dtype=torch.float32, bias=bias, n_group=8, topk_group=4, routed_scaling=2.5)
+    assert torch.equal(ids.cpu(), o_ids)
+    assert torch.allclose(w.cpu(), o_w, rtol=2e-6, atol=0)
+    ref_r, _, _, _, _, y3 = oracle.layer_forward(x, o_ids, w.cpu(), wu[:E], wg[:E], wd[:E], mode=2, return_y3=True)
+    ref = oracle.add_shared(ref_r.to(dt), x, wu[E], wg[E], wd[E], rounded=False)
+    step = 2.0 ** -8
+    budget = torch.zeros(T, H)
+    for k in range(K):
+        for t in range(T):
+            e = int(o_ids[t, k])
+            h = oracle.ffn(x[t:t + 1], wu[e], wg[e], wd[e], mode=2, return_h=True)[1]
+            budget[t] += float(w[t, k]) * (h.float().abs() @ wd[e].float().abs().T)[0]
+    h = oracle.ffn(x, wu[E], wg[E], wd[E], mode=2, return_h=True)[1]
+    budget += h.float().abs() @ wd[E].float().abs().T
+    rms = float(ref.pow(2).mean().sqrt())
+    err = (y.float().cpu() - ref).abs()
+    quanta = (ulp_of((w.cpu().unsqueeze(-1) * y3.float()).abs().amax(dim=1), dt) + 0.5 * ulp_of(ref, dt) * 1.0001
+              + ulp_of(ref_r, dt) + ulp_of(ref - ref_r.to(dt).float(), dt))
+    print(f"ds-tiny layer: max|err|/rms = {float(err.max()) / rms:.3e}, over 2e-2*rms: {float((err > TOL * rms).float().mean()):.2e}", flush=True)
+    assert bool((err <= TOL * rms + quanta + 4 * step * budget).all())
+    assert float((err > TOL * rms).float().mean()) <= 2e-3
+    hy, hids, hw = layer.forward_logits(x, lg, r)
+    assert torch.equal(hids, ids.cpu()) and torch.equal(hy.view(torch.int16), y.cpu().view(torch.int16))
+    layer.close()
