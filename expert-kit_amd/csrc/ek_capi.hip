@@ -769,16 +769,21 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
         return EK_OK;
     }
     // Two independent chains: the weight-streaming kernel (items of <= 16 rows) and the
-    // MFMA tile kernel (longer items) touch disjoint rows of h and out.  In the middle
-    // regime (a few to a few dozen rows per expert on average) both have real work of
-    // similar size and run side by side: the tile chain is forked to the side stream and
-    // joined before returning.  In the decode regime the tile lists are (nearly) empty and
-    // in the prefill regime the streaming list is short, and measured on MI355X the
-    // fork/join then costs more than it hides, so those run in order on s.
+    // MFMA tile kernel (longer items) touch disjoint rows of h and out, and run side by side:
+    // one chain is forked to the side stream and joined before returning.  The chain with
+    // most of the work stays on s; when that is the tile chain its kernel is launched first, so
+    // that its workgroups (one per CU, by their LDS) are resident before the streaming waves
+    // fill the register file around them.  Measured on MI355X against running both in order:
+    // Qwen3 fp16 (E 128, K 8) 512 / 1024 / 2048 / 4096 / 16384 tokens -7 / -11 / -2 / -1 / 0 %,
+    // the ragged 4-layer chain -4.8 %; DeepSeek-V3 int8 (E 128) -2 / -5 / -3 / 0 / 0 %; with
+    // its 16-bit weights (E 64) -7 / -4 / +3 / -1 / +1 %: with experts of that size, beyond 128
+    // pairs per expert, the long streaming kernel takes from the tiles what the overlap returns.  In the decode
+    // regime the tile lists are (nearly) empty and the fork/join costs more than it hides.
     const bool tiles_main = P > 16 * E;
     const bool have_stream = cap[ek::kListStream] > 0;
     const bool have_tiles = cap[ek::kListT32] + cap[ek::kListT64] + cap[ek::kListT128] > 0;
-    const bool fork = have_stream && have_tiles && P > 4 * E && P <= 64 * E;
+    const bool small_expert = 3 * H * I * (L->w8 ? 1 : 2) <= (16ll << 20);
+    const bool fork = have_stream && have_tiles && P > 4 * E && (P <= 128 * E || small_expert);
     hipStream_t s_stream = s, s_tiles = s;
     if (fork || shared_wide > 0) {
         EK_HIP(hipEventRecord(L->ev_fork, s));
@@ -787,6 +792,8 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
     if (fork) (tiles_main ? s_stream : s_tiles) = L->side_stream;
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
+        const bool tiles_first = fork && tiles_main;
+        if (tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
         if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, cap[ek::kListStream], false, s_stream));
         if (shared_wide > 0) {
             ek::FfnArgs aw = a;                  // the same stage over the shared segment's own list
@@ -794,7 +801,7 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
             aw.lists.count = L->wide_count;
             EK_HIP(ek::launch_ffn_stream(aw, stage, L->act, L->wmode, shared_wide, true, L->side_stream));
         }
-        if (have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
+        if (!tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
     }
     if (fork || shared_wide > 0) {
