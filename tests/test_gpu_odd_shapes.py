@@ -221,3 +221,25 @@ def test_ds_tiny_layer_as_configured(ek, oracle, cuda):
     hy, hids, hw = layer.forward_logits(x, lg, r)
     assert torch.equal(hids, ids.cpu()) and torch.equal(hy.view(torch.int16), y.cpu().view(torch.int16))
     layer.close()
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_block_scaled_dequantised_at_load(ek, oracle, cuda, kind, dt):
+    """A 16-bit layer fed block-scaled one-byte tensors (dequantised once, at load, with
+    w8a16_activate's arithmetic): the padded scale grid must line up with the padded matrix."""
+    H, I, n = 200, 136, 50
+    ew = make_block_expert(ek, H, I, 9, kind)
+    ffn = ek.HipFFN.construct(ek.EKInstance(H, I), ew, act_dtype=dt, max_rows=64)
+    x = torch.randn(n, H, generator=torch.Generator().manual_seed(3)).to(dt)
+    got = ffn.forward(x.to(cuda))
+    gate(oracle, got, x, *ref_weights(oracle, ew, dt), f"odd block-at-load {kind} {dt}")
+    ffn.close()
+    # from an ek-db blob with the checkpoint's tensor names
+    from safetensors.torch import save as st_save
+    blob = st_save({f"m.experts.0.{m}_proj.weight": getattr(ew, m + "_w") for m in ("up", "gate", "down")} |
+                   {f"m.experts.0.{m}_proj.weight_scale_inv": getattr(ew, m + "_scale") for m in ("up", "gate", "down")})
+    layer = ek.HipLayer(H, I, 1, 1, act_dtype=dt, w_dtype=dt, max_tokens=64)
+    layer.set_expert_safetensors(0, blob)
+    assert torch.equal(layer.expert_forward(0, x.to(cuda)).view(torch.int16), got.view(torch.int16))
+    layer.close()
