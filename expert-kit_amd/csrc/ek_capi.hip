@@ -156,6 +156,7 @@ struct ek_expert {
 struct ek_chain {
     std::vector<ek_layer *> layers;
     void *act[2] = {nullptr, nullptr};       // ping-pong activations [max_tokens, H]
+    void *act_in = nullptr;                  // hidden size padded: the caller's rows at the kernels' row size
     int32_t *d_err = nullptr;                // [L] per-layer routing error words, gathered
     int32_t *h_err = nullptr;                // pinned
     hipStream_t stream = nullptr;
@@ -1401,6 +1402,7 @@ static void free_chain(ek_chain *c)
     if (c->graph) (void)hipGraphDestroy(c->graph);
     if (c->act[0]) (void)hipFree(c->act[0]);
     if (c->act[1]) (void)hipFree(c->act[1]);
+    if (c->act_in) (void)hipFree(c->act_in);
     if (c->d_err) (void)hipFree(c->d_err);
     if (c->h_err) (void)hipHostFree(c->h_err);
     if (c->stream) (void)hipStreamDestroy(c->stream);
@@ -1416,11 +1418,9 @@ ek_status ek_chain_create(ek_layer *const *layers, int32_t n_layers, ek_chain **
             return fail(EK_INVALID_INPUT, "n_layers must be in [1, 1024]");
         for (int i = 0; i < n_layers; ++i) {
             if (!layers[i]) return fail(EK_INVALID_INPUT, "layer %d is NULL", i);
-            if (layers[i]->padded)
-                return fail(EK_INVALID_INPUT, "layer %d runs on padded copies of its rows (hidden or inter is not a "
-                            "multiple of 64): not in a chain", i);
             const ek_cfg &a = layers[0]->cfg, &b = layers[i]->cfg;
-            if (a.hidden != b.hidden || a.top_k != b.top_k || a.act_dtype != b.act_dtype ||
+            // (equal padded sizes too: layers with one-byte weights pad a small hidden size further)
+            if (a.hidden != b.hidden || layers[0]->user_hidden != layers[i]->user_hidden || a.top_k != b.top_k || a.act_dtype != b.act_dtype ||
                 a.device_id != b.device_id || a.max_tokens != b.max_tokens)
                 return fail(EK_INVALID_INPUT, "layer %d differs from layer 0 in hidden / top_k / "
                             "act_dtype / device / max_tokens", i);
@@ -1433,6 +1433,13 @@ ek_status ek_chain_create(ek_layer *const *layers, int32_t n_layers, ek_chain **
         const size_t act_bytes = (size_t)layers[0]->cfg.max_tokens * layers[0]->cfg.hidden * 2;
         ek_status st = dev_alloc(&c->act[0], act_bytes, "chain activations");
         if (st == EK_OK) st = dev_alloc(&c->act[1], act_bytes, "chain activations");
+        if (st == EK_OK && layers[0]->cfg.hidden != layers[0]->user_hidden) {
+            // the padding columns of the first layer's input are zero and stay so; every layer writes
+            // zeros into those of its output (its padded output channels have zero weights)
+            st = dev_alloc(&c->act_in, act_bytes, "chain input");
+            if (st == EK_OK && hipMemset(c->act_in, 0, act_bytes) != hipSuccess) st = fail(EK_HIP_ERROR, "hipMemset failed");
+            if (st == EK_OK && hipDeviceSynchronize() != hipSuccess) st = fail(EK_HIP_ERROR, "hipDeviceSynchronize failed");
+        }
         if (st == EK_OK) st = dev_alloc((void **)&c->d_err, sizeof(int32_t) * n_layers, "chain errors");
         if (st == EK_OK) {
             hipError_t e = hipHostMalloc((void **)&c->h_err, sizeof(int32_t) * n_layers, hipHostMallocDefault);
@@ -1458,8 +1465,12 @@ static ek_status enqueue_chain(ek_chain *c, const void *x, const int32_t *ids, c
     const int64_t K = c->layers[0]->cfg.top_k;
     const size_t w_es = w_f32 ? 4 : 2;
     const void *in = x;
+    if (c->act_in) {
+        EK_TRY(rows_in(c->layers[0], c->act_in, x, T, EK_DEVICE, s));
+        in = c->act_in;
+    }
     for (int l = 0; l < L; ++l) {
-        void *outp = l == L - 1 ? y : c->act[l & 1];
+        void *outp = l == L - 1 && !c->act_in ? y : c->act[l & 1];
         ek_layer *ly = c->layers[l];
         const bool prof = ly->profiling;
         ly->profiling = false;               // no event records inside a chain (capture-safe)
@@ -1471,6 +1482,7 @@ static ek_status enqueue_chain(ek_chain *c, const void *x, const int32_t *ids, c
         EK_HIP(hipMemcpyAsync(c->d_err + l, ly->err, sizeof(int32_t), hipMemcpyDeviceToDevice, s));
         in = outp;
     }
+    if (c->act_in) EK_TRY(rows_out(c->layers[0], y, in, T, EK_DEVICE, s));
     return EK_OK;
 }
 

@@ -79,7 +79,7 @@ typedef struct ek_cfg {
                            with one-byte weights); other sizes (the reference's toy models: ds-tiny has
                            hidden 16, intermediate 8) are served zero-padded: the weights once at load,
                            every call's rows through the layer's staging buffers, also for device
-                           memory.  Same results; such a layer cannot join a chain. */
+                           memory (a chain stages its first input and last output only).  Same results. */
     int64_t inter;      /* I  (moe_intermediate_size): any positive size, padded likewise */
     int32_t n_experts;  /* E  experts owned by one layer object */
     int32_t top_k;      /* K  slots per token */

@@ -164,10 +164,6 @@ def test_wire_and_shapes(ek, oracle, cuda):
     assert reply.shape == (8, H) and reply.dtype == dt
     gate(oracle, reply, x, wu[2], wg[2], wd[2], "ds-tiny wire")
     assert torch.equal(reply.view(torch.int16), layer.expert_forward(2, x).view(torch.int16))
-    # a chain wants the kernels' own sizes
-    with pytest.raises(ek.EKError) as ei:
-        ek.HipChain([layer])
-    assert ei.value.status == C.EK_INVALID_INPUT
     # weights of the wrong size are refused by the caller's sizes
     bad = wl.make_expert(wl.Workload("b", 64, 64, 1, 1, 1, dt), 0)
     with pytest.raises(ek.EKError) as ei:
@@ -243,3 +239,40 @@ def test_block_scaled_dequantised_at_load(ek, oracle, cuda, kind, dt):
     layer.set_expert_safetensors(0, blob)
     assert torch.equal(layer.expert_forward(0, x.to(cuda)).view(torch.int16), got.view(torch.int16))
     layer.close()
+
+
+@pytest.mark.parametrize("H,inters", [(16, (8, 8, 8)), (72, (100, 64, 24))])
+def test_chain_of_padded_layers(ek, cuda, H, inters):
+    """Layers of such sizes in a chain (one graph): the same bits as calling them one by one, on every
+    replay, with the caller's buffers at the caller's row size."""
+    E, K, T = 8, 2, 90
+    dt = torch.bfloat16
+    layers = []
+    for l, I in enumerate(inters):
+        w = wl.Workload("odd chain", H, I, E, K, T, dt)
+        layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=dt, max_tokens=128)
+        for e in range(E):
+            layer.set_expert(e, wl.make_expert(w, e, layer=l, std=0.2))
+        layers.append(layer)
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(T, H, generator=g).to(dt).to(cuda)
+    ids = torch.stack([torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]) for _ in inters]).to(torch.int32).to(cuda)
+    gw = (torch.rand(len(inters), T, K, generator=g) + 0.2).to(dt).to(cuda)
+    cur = x
+    for l, layer in enumerate(layers):
+        cur = layer.forward(cur, ids[l].contiguous(), gw[l].contiguous())
+    assert float(cur.float().abs().max()) > 0
+    chain = ek.HipChain(layers)
+    y = chain.forward(x, ids, gw, use_graph=False)
+    assert y.shape == (T, H) and torch.equal(y.view(torch.int16), cur.view(torch.int16))
+    for replay in range(3):
+        yg = chain.forward(x, ids, gw, use_graph=True)
+        assert torch.equal(yg.view(torch.int16), cur.view(torch.int16)), replay
+        layers[0].forward(x, ids[0].contiguous(), gw[0].contiguous())      # eager work between the replays
+        torch.cuda.synchronize()
+    # a layer of another hidden size does not join
+    other = ek.HipLayer(H + 8, 64, E, K, act_dtype=dt, w_dtype=dt, max_tokens=128)
+    with pytest.raises(ek.EKError) as ei:
+        ek.HipChain([layers[0], other])
+    assert ei.value.status == C.EK_INVALID_INPUT
+    chain.close()
