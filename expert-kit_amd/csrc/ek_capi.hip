@@ -110,7 +110,9 @@ struct ek_layer {
     // a list of its own for a shared expert's segment cut into wide streaming items
     ek::WorkItem *wide_items = nullptr;
     int32_t *wide_count = nullptr;           // [kNumLists], only [kListStream] is used
-    int32_t *h_err = nullptr;                // pinned
+    int32_t *h_err = nullptr;                // pinned: [0] the error word of a finished call; [1] the number of tile
+                                             // items the last pack cut, stored by its kernel (see enqueue_ffn)
+    int32_t *d_tile_items = nullptr;         // the device's address of h_err[1] (nullptr: the word stays 0)
     // host-built work lists (ek_layer_experts_forward): pinned image of the device lists,
     // reused once ev_items says the previous copy has been consumed
     uint8_t *h_items = nullptr;
@@ -312,6 +314,12 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         if (e == hipSuccess) e = hipMemset(L->lists.count, 0, sizeof(int32_t) * ek::kNumLists);
         if (e == hipSuccess) e = hipMemset(L->wide_count, 0, sizeof(int32_t) * ek::kNumLists);
         if (e == hipSuccess) e = hipHostMalloc((void **)&L->h_err, sizeof(int32_t) * 4, hipHostMallocDefault);
+        if (e == hipSuccess) {
+            memset(L->h_err, 0, sizeof(int32_t) * 4);
+            void *dp = nullptr;
+            if (hipHostGetDevicePointer(&dp, L->h_err + 1, 0) == hipSuccess) L->d_tile_items = (int32_t *)dp;
+            else (void)hipGetLastError();
+        }
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->load_stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->side_stream, hipStreamNonBlocking);
@@ -731,6 +739,7 @@ ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_lo
     a.row_token = L->row_token;
     a.err = L->err;
     a.activation = check_loaded ? L->d_activation : nullptr;
+    a.tile_items_host = check_loaded ? L->d_tile_items : nullptr;
     if (check_loaded) a.lists = L->lists;
     else a.lists = ek::WorkLists{{nullptr, nullptr, nullptr, nullptr}, nullptr};
     return a;
@@ -776,17 +785,26 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
     // takes a whole CU (registers and LDS), so its persistent workgroups claim as many CUs as
     // they have tiles at once and the streaming kernel runs on the others, instead of the tiles
     // waiting for streaming workgroups to drain (in that order Qwen3 fp16 decode at 256 tokens
-    // takes 0.235 ms, in this one 0.221 ms).  With tiles for all 256 CUs the two run in turn.  Measured on MI355X against running both in order:
-    // Qwen3 fp16 (E 128, K 8) 512 / 1024 / 2048 / 4096 / 16384 tokens -7 / -11 / -2 / -1 / 0 %,
-    // the ragged 4-layer chain -4.8 %; DeepSeek-V3 int8 (E 128) -2 / -5 / -3 / 0 / 0 %; with
-    // its 16-bit weights (E 64) -7 / -4 / +3 / -1 / +1 %: with experts of that size, beyond 128
-    // pairs per expert, the long streaming kernel takes from the tiles what the overlap returns.  In the decode
-    // regime the tile lists are (nearly) empty and the fork/join costs more than it hides.
+    // takes 0.235 ms, in this one 0.221 ms).  With tiles for all 256 CUs the two run in turn.
+    // Measured on MI355X against running both in order: Qwen3 fp16 (E 128, K 8) 512 / 1024 /
+    // 2048 / 4096 / 16384 tokens -7 / -11 / -2 / -1 / 0 %, the ragged 4-layer chain -4.8 %;
+    // DeepSeek-V3 int8 (E 128) -2 / -5 / -3 / 0 / 0 %; with its 16-bit weights (E 64) -7 / -4 /
+    // +3 / -1 / +1 %: with experts of that size, beyond 128 pairs per expert, the long streaming
+    // kernel takes from the tiles what the overlap returns.
+    // Up to 4 pairs per expert the tile lists are empty unless the routing is skewed: then a hot
+    // expert's 17+ rows are a tile that keeps a handful of CUs busy for a whole contraction, after
+    // the streaming kernel in the same stream (DeepSeek-V3 int8, 32 / 64 / 128 tokens, Zipf 1.0:
+    // 493 / 587 / 813 us in order, 391 / 521 / 748 us side by side), while with no tiles the
+    // fork/join costs 10-20 us for nothing.  Skew persists from one call to the next, so the last
+    // pack's tile count, which its kernel left in pinned memory, decides; it may be a call or two
+    // old, and either choice computes the same bits.
     const bool tiles_main = P > 16 * E;
     const bool have_stream = cap[ek::kListStream] > 0;
     const bool have_tiles = cap[ek::kListT32] + cap[ek::kListT64] + cap[ek::kListT128] > 0;
     const bool small_expert = 3 * H * I * (L->w8 ? 1 : 2) <= (16ll << 20);
-    const bool fork = have_stream && have_tiles && P > 4 * E && (P <= 128 * E || small_expert);
+    const bool tiles_lately = ((volatile int32_t *)L->h_err)[1] > 0;
+    const bool fork = have_stream && have_tiles &&
+                      (P > 4 * E ? P <= 128 * E || small_expert : tiles_lately);
     hipStream_t s_stream = s, s_tiles = s;
     if (fork || shared_wide > 0) {
         EK_HIP(hipEventRecord(L->ev_fork, s));

@@ -120,6 +120,7 @@ struct PackArgs {
     int32_t *row_token;       // [P]  perm[j] / K
     int32_t *err;             // bit 0: id out of range, bit 1: expert not loaded
     uint64_t *activation;     // [E] running sum of counts over calls, or nullptr
+    int32_t *tile_items_host; // pinned host word that receives the number of tile items cut, or nullptr
     WorkLists lists;
 };
 constexpr int kPackChunk = 4096;   // pairs per workgroup

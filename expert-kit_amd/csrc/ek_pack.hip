@@ -122,6 +122,7 @@ __global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
         a.lists.count[kListT64] = s64;
         a.lists.count[kListT32] = s32;
         a.lists.count[kListStream] = ss;
+        if (a.tile_items_host) *a.tile_items_host = s128 + s64 + s32;
     }
 }
 
@@ -309,6 +310,7 @@ __global__ __launch_bounds__(1024) void pack_fused_kernel(PackArgs a, int nbits)
             a.lists.count[kListT64] = s64;
             a.lists.count[kListT32] = s32;
             a.lists.count[kListStream] = ss;
+        if (a.tile_items_host) *a.tile_items_host = s128 + s64 + s32;
         }
     }
     __syncthreads();

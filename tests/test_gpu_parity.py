@@ -511,3 +511,29 @@ def test_block128_scaled_weights(ek, oracle, cuda, src, dt):
     be = ek.ExpertBackend.build(ek.EKInstance(H, I), named, act_dtype=dt, max_rows=64)
     assert torch.equal(be.forward(x.to(cuda)).cpu().view(torch.int16), got.cpu().view(torch.int16))
     ffn.close()
+
+
+def test_decode_with_skewed_routing_repeats_bitwise(ek, oracle, cuda):
+    """At decode sizes the library runs the tile chain beside the streaming chain only when the
+    previous call's routing produced tile items; both orders must give the same bits, call after
+    call, also when the skew comes and goes."""
+    w = wl.Workload("skew", 512, 256, 32, 4, 24, torch.bfloat16)
+    layer, ws = load_layer(ek, w, max_tokens=64)
+    wu, wg, wd = oracle_weights(oracle, ws, w.n_experts, w.act_dtype)
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(w.tokens, w.hidden, generator=g).to(w.act_dtype)
+    gw = (torch.rand(w.tokens, w.top_k, generator=g) + 0.1).to(w.act_dtype)
+    uniform = torch.stack([torch.randperm(w.n_experts, generator=g)[:w.top_k] for _ in range(w.tokens)]).to(torch.int32)
+    skewed = uniform.clone()
+    skewed[:, 0] = 5                           # every token also goes to expert 5: a 24-row segment, one tile
+    first = {}
+    for step, ids in enumerate([uniform, skewed, skewed, uniform, uniform, skewed]):
+        name = "skewed" if ids is skewed else "uniform"
+        y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
+        assert (int(rt.counts.max()) > 16) == (ids is skewed)        # a tile item exactly when skewed
+        if name not in first:
+            first[name] = y.clone()
+            ref, _, _, _, _, y3 = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=2, return_y3=True)
+            layer_gate(y, ref, y3, gw, f"decode {name}", small=2)
+        assert torch.equal(y.view(torch.int16), first[name].view(torch.int16)), (step, name)
+    layer.close()
