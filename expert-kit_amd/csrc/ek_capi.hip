@@ -755,9 +755,11 @@ ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_lo
 // shared segment cut into 16-row items).
 // shared_wide: L->wide_items holds that many streaming items of up to kWideRows rows (a shared
 // segment); they get launches of their own on the side stream, beside the others.
+// exact: the lists' lengths when the caller built them on the host (the grids then fit them,
+// an empty list gets no launch, and the two chains run side by side exactly when both have work).
 ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out, int64_t P, int64_t E,
                       hipStream_t s, hipEvent_t *ev, int64_t wide_items = 0, int64_t extra_stream = 0,
-                      int64_t shared_wide = 0)
+                      int64_t shared_wide = 0, const int64_t *exact = nullptr)
 {
     const int64_t H = L->cfg.hidden, I = L->cfg.inter;
     ek::FfnArgs a1;
@@ -769,6 +771,7 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
     int64_t cap[ek::kNumLists];
     for (int l = 0; l < ek::kNumLists; ++l) {
         cap[l] = ek::list_capacity(l, P, E) + (l == ek::kListStream ? extra_stream : 0);
+        if (exact) cap[l] = exact[l];          // the caller built the lists on the host
         if (cap[l] > L->list_cap[l]) cap[l] = L->list_cap[l];
         if (cap[l] < 0) cap[l] = 0;
     }
@@ -802,7 +805,7 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
     const bool have_stream = cap[ek::kListStream] > 0;
     const bool have_tiles = cap[ek::kListT32] + cap[ek::kListT64] + cap[ek::kListT128] > 0;
     const bool small_expert = 3 * H * I * (L->w8 ? 1 : 2) <= (16ll << 20);
-    const bool tiles_lately = ((volatile int32_t *)L->h_err)[1] > 0;
+    const bool tiles_lately = exact ? true : ((volatile int32_t *)L->h_err)[1] > 0;   // (exact: have_tiles says it)
     const bool fork = have_stream && have_tiles &&
                       (P > 4 * E ? P <= 128 * E || small_expert : tiles_lately);
     hipStream_t s_stream = s, s_tiles = s;
@@ -1223,12 +1226,22 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             // Work lists cut on the host exactly as the pack kernels cut them: a call is one
             // segment (ek_internal.h, "work lists").
             std::vector<ek::WorkItem> items[ek::kNumLists];
-            int64_t row0 = 0, tile_items = 0, wide_items = 0;
+            int64_t row0 = 0, tile_items = 0, wide_items = 0, short_items = 0;
             for (int i = 0; i < n_calls; ++i) {
                 tile_items += (rows[i] >> 7) + ((rows[i] & 127) > 16);
                 wide_items += (rows[i] + ek::kWideRows - 1) / ek::kWideRows;
+                short_items += (rows[i] & 127) > 0 && (rows[i] & 127) <= 16;
             }
-            const bool wide = ek::wide_cut_pays(tile_items, P, H, layer->cfg.inter, layer->w8 ? 1 : 2) &&
+            // The wide cut spares a batch the tile kernel's long, nearly empty launch.  When the batch
+            // also has many short requests, their streaming chain (one pass over an expert's weights
+            // each, ~6.5 TB/s) runs beside the tile chain and covers it, and the short items are
+            // served faster by the sliced streaming form than by the wide one (64 DeepSeek-V3 int8
+            // requests from host memory, 4 rows each but one of 40 / four of 100: 995 / 1500 us cut wide,
+            // 890 / 1325 us as tiles beside streams).
+            const int wb = layer->w8 ? 1 : 2;
+            const double cover_us = (double)short_items * 3.0 * (double)H * (double)layer->cfg.inter * wb / 6.5e6;
+            const double tiled_us = 15.0 + (double)(H + layer->cfg.inter) * (wb == 1 ? 0.025 : 0.0285);
+            const bool wide = ek::wide_cut_pays(tile_items, P, H, layer->cfg.inter, wb) && cover_us < 0.5 * tiled_us &&
                               wide_items <= layer->list_cap[ek::kListStream];
             for (int i = 0; i < n_calls; ++i) {
                 const int32_t n = (int32_t)rows[i], full = n >> 7, r = n & 127;
@@ -1303,7 +1316,10 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
                                           hipMemcpyDeviceToDevice, s));
                 row0 += rows[i];
             }
-            EK_TRY(enqueue_ffn(layer, layer->st_x, nullptr, layer->st_y, P, n_calls, s, nullptr, wide ? wide_items : 0));
+            int64_t exact[ek::kNumLists];
+            for (int l = 0; l < ek::kNumLists; ++l) exact[l] = (int64_t)items[l].size();
+            EK_TRY(enqueue_ffn(layer, layer->st_x, nullptr, layer->st_y, P, n_calls, s, nullptr, wide ? wide_items : 0, 0, 0,
+                               wide ? nullptr : exact));
             EK_HIP(hipGetLastError());
             row0 = 0;
             if (one_transfer) {
