@@ -117,6 +117,9 @@ struct ek_layer {
     // reused once ev_items says the previous copy has been consumed
     uint8_t *h_items = nullptr;
     hipEvent_t ev_items = nullptr;
+    ek::RowCopy *h_segs = nullptr;           // pinned: the row-copy tables of a batched device-memory call, in then out
+    ek::RowCopy *d_segs = nullptr;           // the device's address of h_segs
+    int64_t segs_cap = 0;                    // entries per table
 
     // staging for host-memory callers (allocated on first use)
     void *st_x = nullptr, *st_w = nullptr, *st_y = nullptr, *st_xp = nullptr;
@@ -210,6 +213,7 @@ void free_layer(ek_layer *L)
     if (L->pin_in) (void)hipHostFree(L->pin_in);
     if (L->pin_out) (void)hipHostFree(L->pin_out);
     if (L->ev_items) (void)hipEventDestroy(L->ev_items);
+    if (L->h_segs) (void)hipHostFree(L->h_segs);
     if (L->stream) (void)hipStreamDestroy(L->stream);
     if (L->load_stream) (void)hipStreamDestroy(L->load_stream);
     if (L->side_stream) (void)hipStreamDestroy(L->side_stream);
@@ -1305,8 +1309,35 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
                 layer->pin_in_used = all_bytes;
                 EK_HIP(hipMemcpyAsync(layer->st_x, layer->pin_in, all_bytes, hipMemcpyHostToDevice, s));
             }
+            // Device-memory requests: one copy kernel each way over a table of the requests' rows
+            // (64 requests: 128 asynchronous copies cost ~500 us of host time, more than the kernels).
+            bool table = mem == EK_DEVICE && n_calls > 1;
+            for (int i = 0; i < n_calls && table; ++i)
+                table = (((uintptr_t)xs[i] | (uintptr_t)outs[i]) & 15) == 0 || rows[i] == 0;
+            if (table && layer->segs_cap < n_calls) {
+                EK_HIP(hipEventSynchronize(layer->ev_items));      // (the previous tables have been read)
+                if (layer->h_segs) { (void)hipHostFree(layer->h_segs); layer->h_segs = nullptr; layer->segs_cap = 0; }
+                const int64_t cap_new = n_calls < 1024 ? 1024 : 2 * (int64_t)n_calls;
+                EK_HIP(hipHostMalloc((void **)&layer->h_segs, sizeof(ek::RowCopy) * 2 * (size_t)cap_new, hipHostMallocDefault));
+                void *dp = nullptr;
+                if (hipHostGetDevicePointer(&dp, layer->h_segs, 0) != hipSuccess) { (void)hipGetLastError(); table = false; }
+                layer->d_segs = (ek::RowCopy *)dp;
+                layer->segs_cap = table ? cap_new : 0;
+            }
+            if (table) {
+                const int64_t uw = layer->user_hidden * 2;          // bytes of a caller's row
+                row0 = 0;
+                for (int i = 0; i < n_calls; ++i) {
+                    layer->h_segs[i] = ek::RowCopy{(const uint8_t *)xs[i], (uint8_t *)layer->st_x + row0 * H * 2, uw, H * 2,
+                                                   (int32_t)rows[i], (int32_t)uw};
+                    layer->h_segs[layer->segs_cap + i] = ek::RowCopy{(const uint8_t *)layer->st_y + row0 * H * 2, (uint8_t *)outs[i],
+                                                                     H * 2, uw, (int32_t)rows[i], (int32_t)uw};
+                    row0 += rows[i];
+                }
+                ek::launch_rows_copy(layer->d_segs, n_calls, s);
+            }
             row0 = 0;
-            for (int i = 0; i < n_calls && !one_transfer; ++i) {
+            for (int i = 0; i < n_calls && !one_transfer && !table; ++i) {
                 if (layer->padded)
                     EK_TRY(rows_in(layer, (char *)layer->st_x + row0 * H * 2, xs[i], rows[i], mem, s));
                 else if (rows[i] && mem == EK_HOST)
@@ -1330,7 +1361,12 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
                     row0 += rows[i];
                 }
             }
-            for (int i = 0; i < n_calls && !one_transfer; ++i) {
+            if (table) {
+                ek::launch_rows_copy(layer->d_segs + layer->segs_cap, n_calls, s);
+                EK_HIP(hipGetLastError());
+                EK_HIP(hipEventRecord(layer->ev_items, s));         // the tables are free again after this
+            }
+            for (int i = 0; i < n_calls && !one_transfer && !table; ++i) {
                 if (layer->padded)
                     EK_TRY(rows_out(layer, outs[i], (char *)layer->st_y + row0 * H * 2, rows[i], mem, s));
                 else if (rows[i] && mem == EK_HOST)

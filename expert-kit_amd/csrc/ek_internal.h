@@ -178,6 +178,20 @@ struct CombineArgs {
 };
 void launch_combine(const CombineArgs &a, hipStream_t s);
 
+// ---- batched row copies -----------------------------------------------------
+// One launch moves the rows of many requests between the callers' buffers and a staging buffer
+// (instead of one asynchronous copy per request, ~4 us of host time each).
+struct RowCopy {
+    const uint8_t *src;
+    uint8_t *dst;
+    int64_t src_pitch, dst_pitch;   // bytes from one row to the next
+    int32_t rows;
+    int32_t row_bytes;              // a multiple of 16; src and dst are 16-byte aligned
+};
+// segs: n entries the device can read (device memory or pinned host memory), unchanged until the
+// kernel has run
+void launch_rows_copy(const RowCopy *segs, int n, hipStream_t s);
+
 // ---- weight ingestion -------------------------------------------------------
 // src [N, K] row-major of src_dtype (ek_dtype numbering) -> chunked layout at
 // dst, matrix m of an nmat-group.  dst_dtype: 0 bf16, 1 f16, 3 int8.  block_scale (16-bit

@@ -76,6 +76,25 @@ void launch_combine(const CombineArgs &a, hipStream_t s)
     }
 }
 
+// ---- batched row copies -------------------------------------------------------
+
+__global__ __launch_bounds__(256) void rows_copy_kernel(const RowCopy *segs)
+{
+    const RowCopy c = segs[blockIdx.x];
+    const int per_row = c.row_bytes >> 4;
+    const int64_t units = (int64_t)c.rows * per_row;
+    for (int64_t u = (int64_t)blockIdx.y * 256 + threadIdx.x; u < units; u += (int64_t)gridDim.y * 256) {
+        const int64_t r = u / per_row, k = u - r * per_row;
+        *(uint4 *)(c.dst + r * c.dst_pitch + k * 16) = *(const uint4 *)(c.src + r * c.src_pitch + k * 16);
+    }
+}
+
+void launch_rows_copy(const RowCopy *segs, int n, hipStream_t s)
+{
+    if (n <= 0) return;
+    hipLaunchKernelGGL(rows_copy_kernel, dim3((unsigned)n, 8), dim3(256), 0, s, segs);
+}
+
 // ---- weight ingestion ---------------------------------------------------------
 
 // OCP fp8 e4m3fn -> fp32 (no infinities; 0x7f / 0xff are NaN)

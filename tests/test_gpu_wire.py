@@ -71,7 +71,16 @@ def test_batch_equals_individual_calls(ek, dt, w8):
     dev = layer.experts_forward([e for e, _ in calls], [x.cuda() for x in xs])
     for out, d in zip(outs, dev):
         assert d.is_cuda and torch.equal(bits(out), bits(d))
-    assert layer.stats()["expert_forward_calls"] >= 3 * len(calls)
+    # device rows that do not start on a 16-byte boundary take the copy-by-copy route: same bits
+    shifted = []
+    for x in xs:
+        flat = torch.empty(x.numel() + 1, dtype=dt, device="cuda")
+        flat[1:] = x.reshape(-1).cuda()
+        shifted.append(flat[1:].view(x.shape))
+    assert any(t.data_ptr() % 16 for t in shifted if t.numel())
+    for out, d in zip(outs, layer.experts_forward([e for e, _ in calls], shifted)):
+        assert torch.equal(bits(out), bits(d))
+    assert layer.stats()["expert_forward_calls"] >= 4 * len(calls)
     # a batch with enough rows for the tile kernel: its long calls take the other kernel family than
     # they take alone, so the results agree as two evaluations of the same product do, not bit for bit
     big = [(2, 128), (4, 300), (1, 200), (3, 9)]
