@@ -127,7 +127,8 @@ constexpr int kPackChunk = 4096;   // pairs per workgroup
 constexpr int kPackThreads = 256;
 constexpr int kMaxExperts = 1024;
 
-// clears *err itself (with a fill kernel, never a memset node: graph-capture safe)
+// writes *err itself (one kernel of every pack stores the call's word: nothing to clear first,
+// no memset node: graph-capture safe)
 void launch_pack(const PackArgs &a, hipStream_t s);
 // work lists for one segment [0, n) of expert e (per-expert forward)
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool wide, hipStream_t s);

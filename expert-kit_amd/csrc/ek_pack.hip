@@ -25,13 +25,11 @@ __global__ __launch_bounds__(kPackThreads) void pack_hist_kernel(PackArgs a)
     __syncthreads();
     const int64_t base = (int64_t)blockIdx.x * kPackChunk;
     const int64_t end = min(base + (int64_t)kPackChunk, a.P);
-    bool bad = false;
+    // (ids out of range are left out; the scan kernel sees that the counts do not add up to P)
     for (int64_t p = base + threadIdx.x; p < end; p += kPackThreads) {
         const int32_t id = a.ids[p];
         if ((uint32_t)id < (uint32_t)a.E) atomicAdd(&hist[id], 1);
-        else bad = true;
     }
-    if (bad) atomicOr(a.err, 1);
     __syncthreads();
     for (int i = threadIdx.x; i < a.E; i += kPackThreads)
         a.block_hist[(int64_t)blockIdx.x * a.E + i] = hist[i];
@@ -103,12 +101,17 @@ __global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
         }
         a.counts[e] = total;
         if (a.activation) a.activation[e] += (uint64_t)total;
-        if (total > 0 && a.slabs != nullptr && a.slabs[e].upgate == nullptr) atomicOr(a.err, 2);
     }
+    const bool unloaded = e < a.E && total > 0 && a.slabs != nullptr && a.slabs[e].upgate == nullptr;
+    const int any_unloaded = __syncthreads_or(unloaded);
     int32_t sum;
     const int32_t off = block_exclusive_scan(total, wave_tot, &sum);
     if (e < a.E) a.offsets[e] = off;
-    if (e == 0) a.offsets[a.E] = sum;
+    if (e == 0) {
+        a.offsets[a.E] = sum;
+        // the error word is written, not accumulated: every pair with an id in range was counted once
+        a.err[0] = ((int64_t)sum != a.P ? 1 : 0) | (any_unloaded ? 2 : 0);
+    }
     if (a.lists.count == nullptr) return;
     const SegmentCut c = cut_segment(total);
     int32_t s128, s64, s32, ss;
@@ -338,20 +341,13 @@ __global__ __launch_bounds__(1024) void pack_fused_kernel(PackArgs a, int nbits)
     }
 }
 
-__global__ void clear_err_kernel(int32_t *err) { err[0] = 0; }
-
-void launch_clear_err(int32_t *err, hipStream_t s)
-{
-    hipLaunchKernelGGL(clear_err_kernel, dim3(1), dim3(1), 0, s, err);
-}
-
 void launch_pack(const PackArgs &a, hipStream_t s)
 {
     if (a.P <= 0) {
         // offsets and counts must still be defined (all zero)
         PackArgs z = a;
         z.nblocks = 0;
-        launch_clear_err(a.err, s);
+        z.P = 0;
         hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(1024), 0, s, z);
         return;
     }
@@ -362,7 +358,6 @@ void launch_pack(const PackArgs &a, hipStream_t s)
         hipLaunchKernelGGL(pack_fused_kernel, dim3(1), dim3(1024), lds_bytes, s, a, nbits);
         return;
     }
-    launch_clear_err(a.err, s);
     hipLaunchKernelGGL(pack_hist_kernel, dim3(a.nblocks), dim3(kPackThreads), 0, s, a);
     hipLaunchKernelGGL(pack_scan_kernel, dim3(1), dim3(1024), 0, s, a);
     hipLaunchKernelGGL(pack_rank_kernel, dim3(a.nblocks), dim3(kPackThreads), 0, s, a, nbits);

@@ -473,6 +473,34 @@ def test_error_paths(ek, cuda):
     layer.close()                                               # idempotent
 
 
+def test_error_word_large_calls(ek, cuda):
+    """Calls too long for the single-workgroup pack (more than 4096 pairs): one bad pair among
+    thousands is reported, and the next good call is clean (the word is written per call)."""
+    from ek_hip import _capi as C
+    w = wl.Workload("t", 128, 64, 8, 2, 3000, torch.bfloat16)
+    layer, ws = load_layer(ek, w, experts=[0, 1, 2, 3])
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(w.tokens, 128, generator=g).to(torch.bfloat16).to(cuda)
+    gw = torch.full((w.tokens, 2), 0.5).to(torch.bfloat16).to(cuda)
+    ok_ids = torch.stack([torch.randperm(4, generator=g)[:2] for _ in range(w.tokens)]).to(torch.int32).to(cuda)
+    y0 = layer.forward(x, ok_ids, gw)
+    for bad, status in ((8, C.EK_INVALID_INPUT), (-1, C.EK_INVALID_INPUT), (7, C.EK_EXPERT_NOT_FOUND)):
+        ids = ok_ids.clone()
+        ids[2999, 1] = bad
+        with pytest.raises(ek.EKError) as ei:
+            layer.forward(x, ids, gw)
+        assert ei.value.status == status, bad
+        assert torch.equal(layer.forward(x, ok_ids, gw).view(torch.int16), y0.view(torch.int16))
+    ids = ok_ids.clone()
+    ids[0, 0] = 100                                             # routing tables alone: range check only
+    with pytest.raises(ek.EKError) as ei:
+        layer.pack(ids)
+    assert ei.value.status == C.EK_INVALID_INPUT
+    ids[0, 0] = 7
+    assert int(layer.pack(ids).counts[7]) == 1                  # loaded or not is no matter for pack
+    layer.close()
+
+
 # ------------------------------------------- block-scaled checkpoint weights
 
 @pytest.mark.parametrize("src", ["int8", "fp8"])
