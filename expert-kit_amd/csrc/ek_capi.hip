@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <memory>
 #include <new>
 #include <string>
 #include <vector>
@@ -82,6 +83,20 @@ int64_t elem_size(int dt)
 
 }  // namespace
 
+// Device memory one layer call works in besides its inputs and outputs: routing tables, work
+// lists and the two packed intermediates.  Every call writes what it reads (nothing has to start
+// at zero).  A layer owns one.
+struct Workspace {
+    int32_t *counts = nullptr, *offsets = nullptr, *perm = nullptr, *inv_perm = nullptr;
+    int32_t *row_token = nullptr, *block_hist = nullptr, *err = nullptr;
+    void *h = nullptr, *yp = nullptr;
+    ek::WorkLists lists{};                   // device work lists (see ek_internal.h)
+    int64_t list_cap[ek::kNumLists] = {0, 0, 0, 0};
+    // a list of its own for a shared expert's segment cut into wide streaming items
+    ek::WorkItem *wide_items = nullptr;
+    int32_t *wide_count = nullptr;           // [kNumLists], only [kListStream] is used
+};
+
 struct ek_layer {
     ek_cfg cfg{};             // as the kernels see it: hidden and inter rounded up to what they need
     // The caller's hidden and inter.  A layer whose sizes are not multiples of the kernels' 64
@@ -101,15 +116,12 @@ struct ek_layer {
     std::vector<ek::ExpertSlab> h_slabs;
     ek::ExpertSlab *d_slabs = nullptr;
 
-    // workspace
-    int32_t *counts = nullptr, *offsets = nullptr, *perm = nullptr, *inv_perm = nullptr;
-    int32_t *row_token = nullptr, *block_hist = nullptr, *err = nullptr;
-    void *h = nullptr, *yp = nullptr;
-    ek::WorkLists lists{};                   // device work lists (see ek_internal.h)
-    int64_t list_cap[ek::kNumLists] = {0, 0, 0, 0};
-    // a list of its own for a shared expert's segment cut into wide streaming items
-    ek::WorkItem *wide_items = nullptr;
-    int32_t *wide_count = nullptr;           // [kNumLists], only [kListStream] is used
+    Workspace ws;                            // the layer's own, allocated at creation
+    // Calls that only enqueue return, and drop `mu`, while their kernels still use the workspace
+    // (and the side stream with its fork / join events).  ev_ws marks the end of the last such
+    // call; the next user of the workspace, on whatever stream, waits for it on the device first.
+    hipEvent_t ev_ws = nullptr;
+    bool ws_busy = false;                    // ev_ws has been recorded and not been waited out by a host synchronisation
     int32_t *h_err = nullptr;                // pinned: [0] the error word of a finished call; [1] the number of tile
                                              // items the last pack cut, stored by its kernel (see enqueue_ffn)
     int32_t *d_tile_items = nullptr;         // the device's address of h_err[1] (nullptr: the word stays 0)
@@ -202,10 +214,10 @@ void free_layer(ek_layer *L)
     if (!L) return;
     (void)hipDeviceSynchronize();
     for (void *p : L->expert_mem) if (p) (void)hipFree(p);
-    void *bufs[] = {L->d_slabs, L->counts, L->offsets, L->perm, L->inv_perm, L->row_token,
-                    L->block_hist, L->err, L->h, L->yp, L->st_x, L->st_w, L->st_y, L->st_xp,
-                    L->d_activation, L->st_ids, L->st_raw, L->rt_ids, L->rt_w, L->st_logits, L->st_bias, L->lists.count, L->lists.items[0], L->lists.items[1],
-                    L->lists.items[2], L->lists.items[3], L->wide_items, L->wide_count};
+    void *bufs[] = {L->d_slabs, L->ws.counts, L->ws.offsets, L->ws.perm, L->ws.inv_perm, L->ws.row_token,
+                    L->ws.block_hist, L->ws.err, L->ws.h, L->ws.yp, L->st_x, L->st_w, L->st_y, L->st_xp,
+                    L->d_activation, L->st_ids, L->st_raw, L->rt_ids, L->rt_w, L->st_logits, L->st_bias, L->ws.lists.count, L->ws.lists.items[0], L->ws.lists.items[1],
+                    L->ws.lists.items[2], L->ws.lists.items[3], L->ws.wide_items, L->ws.wide_count};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
     if (L->h_err) (void)hipHostFree(L->h_err);
@@ -219,6 +231,7 @@ void free_layer(ek_layer *L)
     if (L->side_stream) (void)hipStreamDestroy(L->side_stream);
     if (L->ev_fork) (void)hipEventDestroy(L->ev_fork);
     if (L->ev_join) (void)hipEventDestroy(L->ev_join);
+    if (L->ev_ws) (void)hipEventDestroy(L->ev_ws);
     delete L;
 }
 
@@ -288,35 +301,35 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         if (st == EK_OK) st = dev_alloc(p, bytes, what);
     };
     A((void **)&L->d_slabs, sizeof(ek::ExpertSlab) * (E + 1), "slab table");
-    A((void **)&L->counts, sizeof(int32_t) * E, "counts");
-    A((void **)&L->offsets, sizeof(int32_t) * (E + 1), "offsets");
-    A((void **)&L->perm, sizeof(int32_t) * pmax, "perm");
-    A((void **)&L->inv_perm, sizeof(int32_t) * pmax, "inv_perm");
-    A((void **)&L->row_token, sizeof(int32_t) * rows_max, "row_token");
-    A((void **)&L->block_hist, sizeof(int32_t) * nblocks * E, "block_hist");
-    A((void **)&L->err, sizeof(int32_t) * 4, "err");
+    A((void **)&L->ws.counts, sizeof(int32_t) * E, "counts");
+    A((void **)&L->ws.offsets, sizeof(int32_t) * (E + 1), "offsets");
+    A((void **)&L->ws.perm, sizeof(int32_t) * pmax, "perm");
+    A((void **)&L->ws.inv_perm, sizeof(int32_t) * pmax, "inv_perm");
+    A((void **)&L->ws.row_token, sizeof(int32_t) * rows_max, "row_token");
+    A((void **)&L->ws.block_hist, sizeof(int32_t) * nblocks * E, "block_hist");
+    A((void **)&L->ws.err, sizeof(int32_t) * 4, "err");
     A((void **)&L->d_activation, sizeof(uint64_t) * E, "activation counters");
     L->h_activation.assign(E, 0);
     for (int i = 0; i < 10; ++i) L->forward_hist.le[i] = 4000.0 * i;   // the reference's buckets (metrics.rs:51)
-    A(&L->h, (size_t)rows_max * cfg->inter * 2, "h");
-    A(&L->yp, (size_t)rows_max * cfg->hidden * 2, "yp");
-    A((void **)&L->lists.count, sizeof(int32_t) * ek::kNumLists, "work list counts");
-    A((void **)&L->wide_items, sizeof(ek::WorkItem) * kSharedWideItems, "shared expert's work list");
-    A((void **)&L->wide_count, sizeof(int32_t) * ek::kNumLists, "shared expert's work list count");
+    A(&L->ws.h, (size_t)rows_max * cfg->inter * 2, "h");
+    A(&L->ws.yp, (size_t)rows_max * cfg->hidden * 2, "yp");
+    A((void **)&L->ws.lists.count, sizeof(int32_t) * ek::kNumLists, "work list counts");
+    A((void **)&L->ws.wide_items, sizeof(ek::WorkItem) * kSharedWideItems, "shared expert's work list");
+    A((void **)&L->ws.wide_count, sizeof(int32_t) * ek::kNumLists, "shared expert's work list count");
     for (int l = 0; l < ek::kNumLists; ++l) {
         // the per-expert entry point cuts one segment of up to pmax rows: capacity for E = 1 too
         // (and the wide cut, see wide_cut_pays: fewer than 128 tile items of at most 128 rows
         // become at most two streaming items each)
         const int64_t cap = ek::list_capacity(l, rows_max, E + 1) + (l == ek::kListStream ? 264 : 1);
-        L->list_cap[l] = cap;
-        A((void **)&L->lists.items[l], sizeof(ek::WorkItem) * cap, "work list");
+        L->ws.list_cap[l] = cap;
+        A((void **)&L->ws.lists.items[l], sizeof(ek::WorkItem) * cap, "work list");
     }
     if (st == EK_OK) {
         hipError_t e = hipMemset(L->d_slabs, 0, sizeof(ek::ExpertSlab) * (E + 1));
-        if (e == hipSuccess) e = hipMemset(L->err, 0, sizeof(int32_t) * 4);
+        if (e == hipSuccess) e = hipMemset(L->ws.err, 0, sizeof(int32_t) * 4);
         if (e == hipSuccess) e = hipMemset(L->d_activation, 0, sizeof(uint64_t) * E);
-        if (e == hipSuccess) e = hipMemset(L->lists.count, 0, sizeof(int32_t) * ek::kNumLists);
-        if (e == hipSuccess) e = hipMemset(L->wide_count, 0, sizeof(int32_t) * ek::kNumLists);
+        if (e == hipSuccess) e = hipMemset(L->ws.lists.count, 0, sizeof(int32_t) * ek::kNumLists);
+        if (e == hipSuccess) e = hipMemset(L->ws.wide_count, 0, sizeof(int32_t) * ek::kNumLists);
         if (e == hipSuccess) e = hipHostMalloc((void **)&L->h_err, sizeof(int32_t) * 4, hipHostMallocDefault);
         if (e == hipSuccess) {
             memset(L->h_err, 0, sizeof(int32_t) * 4);
@@ -329,6 +342,7 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->side_stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_fork, hipEventDisableTiming);
         if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_join, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_ws, hipEventDisableTiming);
         if (e != hipSuccess) st = hip_fail(e, "layer setup");
     }
     if (st != EK_OK) {
@@ -577,6 +591,39 @@ ek_status set_expert_padded(ek_layer *L, int32_t e, const ek_weight_desc *up, co
     return st;
 }
 
+// One use of a layer's workspace on stream s; the caller holds L->mu for the scope.
+// begin(): the stream waits (on the device) for the last enqueue-only call that used the
+// workspace.  At the end of the scope the stream's position is recorded as that call's end,
+// unless synced() says the host has waited for the stream, after which nothing is pending.
+// A stream under capture by the caller is left alone both ways (a captured wait on an event
+// recorded outside the capture is not allowed): replays of such a graph use the workspace like
+// the call they record, and ordering them against other calls on the layer is the caller's part.
+struct WorkspaceUse {
+    hipEvent_t ev;
+    bool *busy;
+    hipStream_t s;
+    bool capturing = false, host_synced = false;
+    WorkspaceUse(ek_layer *layer, hipStream_t stream) : ev(layer->ev_ws), busy(&layer->ws_busy), s(stream) {}
+    WorkspaceUse(hipEvent_t event, bool *busy_flag, hipStream_t stream) : ev(event), busy(busy_flag), s(stream) {}
+    ek_status begin()
+    {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cs) != hipSuccess) { (void)hipGetLastError(); cs = hipStreamCaptureStatusNone; }
+        capturing = cs != hipStreamCaptureStatusNone;
+        if (!capturing && *busy) EK_HIP(hipStreamWaitEvent(s, ev, 0));
+        return EK_OK;
+    }
+    void device_idle() { *busy = false; }          // after a hipDeviceSynchronize
+    void synced() { host_synced = true; }          // after a hipStreamSynchronize(s) that followed begin()
+    ~WorkspaceUse()
+    {
+        if (capturing) return;
+        if (host_synced) { *busy = false; return; }
+        if (hipEventRecord(ev, s) == hipSuccess) *busy = true;
+        else (void)hipGetLastError();
+    }
+};
+
 struct Timer {
     std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
     double us() const
@@ -710,7 +757,7 @@ ek_status err_to_status(int32_t err)
     return EK_OK;
 }
 
-ek_status copy_route_out(ek_layer *L, const ek_route_out *r, int64_t P, int mem, hipStream_t s)
+ek_status copy_route_out(ek_layer *L, const Workspace &W, const ek_route_out *r, int64_t P, int mem, hipStream_t s)
 {
     if (!r) return EK_OK;
     const int E = L->cfg.n_experts;
@@ -719,14 +766,14 @@ ek_status copy_route_out(ek_layer *L, const ek_route_out *r, int64_t P, int mem,
         EK_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s));
         return EK_OK;
     };
-    if (r->counts) EK_TRY(out(r->counts, L->counts, sizeof(int32_t) * E));
-    if (r->offsets) EK_TRY(out(r->offsets, L->offsets, sizeof(int32_t) * (E + 1)));
-    if (P > 0 && r->perm) EK_TRY(out(r->perm, L->perm, sizeof(int32_t) * P));
-    if (P > 0 && r->inv_perm) EK_TRY(out(r->inv_perm, L->inv_perm, sizeof(int32_t) * P));
+    if (r->counts) EK_TRY(out(r->counts, W.counts, sizeof(int32_t) * E));
+    if (r->offsets) EK_TRY(out(r->offsets, W.offsets, sizeof(int32_t) * (E + 1)));
+    if (P > 0 && r->perm) EK_TRY(out(r->perm, W.perm, sizeof(int32_t) * P));
+    if (P > 0 && r->inv_perm) EK_TRY(out(r->inv_perm, W.inv_perm, sizeof(int32_t) * P));
     return EK_OK;
 }
 
-ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_loaded)
+ek::PackArgs pack_args(ek_layer *L, const Workspace &W, const int32_t *ids, int64_t P, bool check_loaded)
 {
     ek::PackArgs a;
     a.ids = ids;
@@ -735,48 +782,48 @@ ek::PackArgs pack_args(ek_layer *L, const int32_t *ids, int64_t P, bool check_lo
     a.K = L->cfg.top_k;
     a.nblocks = (int32_t)((P + ek::kPackChunk - 1) / ek::kPackChunk);
     a.slabs = check_loaded ? L->d_slabs : nullptr;
-    a.block_hist = L->block_hist;
-    a.counts = L->counts;
-    a.offsets = L->offsets;
-    a.perm = L->perm;
-    a.inv_perm = L->inv_perm;
-    a.row_token = L->row_token;
-    a.err = L->err;
+    a.block_hist = W.block_hist;
+    a.counts = W.counts;
+    a.offsets = W.offsets;
+    a.perm = W.perm;
+    a.inv_perm = W.inv_perm;
+    a.row_token = W.row_token;
+    a.err = W.err;
     a.activation = check_loaded ? L->d_activation : nullptr;
     a.tile_items_host = check_loaded ? L->d_tile_items : nullptr;
-    if (check_loaded) a.lists = L->lists;
+    if (check_loaded) a.lists = W.lists;
     else a.lists = ek::WorkLists{{nullptr, nullptr, nullptr, nullptr}, nullptr};
     return a;
 }
 
-// Both FFN stages over the work lists in L->lists: x [*, H] (rows picked through
-// `rows`, or packed order when nullptr) -> L->h -> out [P, H].  P and E bound the
+// Both FFN stages over the work lists in W.lists: x [*, H] (rows picked through
+// `rows`, or packed order when nullptr) -> W.h -> out [P, H].  P and E bound the
 // list lengths (grid sizes); ev, if set, receives the stage boundary event.
 // wide_items > 0: the lists hold that many weight-streaming items of up to kWideRows rows and
 // nothing else (the per-expert entry points' cut for calls that would leave the tile kernel
 // most of the chip idle).
 // extra_stream: streaming items the lists hold beyond what P rows over E experts can give (a
 // shared segment cut into 16-row items).
-// shared_wide: L->wide_items holds that many streaming items of up to kWideRows rows (a shared
+// shared_wide: W.wide_items holds that many streaming items of up to kWideRows rows (a shared
 // segment); they get launches of their own on the side stream, beside the others.
 // exact: the lists' lengths when the caller built them on the host (the grids then fit them,
 // an empty list gets no launch, and the two chains run side by side exactly when both have work).
-ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out, int64_t P, int64_t E,
+ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int32_t *rows, void *out, int64_t P, int64_t E,
                       hipStream_t s, hipEvent_t *ev, int64_t wide_items = 0, int64_t extra_stream = 0,
                       int64_t shared_wide = 0, const int64_t *exact = nullptr)
 {
     const int64_t H = L->cfg.hidden, I = L->cfg.inter;
     ek::FfnArgs a1;
-    a1.x = x; a1.x_stride = H; a1.rows = rows; a1.slabs = L->d_slabs; a1.out = L->h; a1.out_stride = I;
-    a1.N = (int32_t)I; a1.Kdim = (int32_t)H; a1.lists = L->lists;
+    a1.x = x; a1.x_stride = H; a1.rows = rows; a1.slabs = L->d_slabs; a1.out = W.h; a1.out_stride = I;
+    a1.N = (int32_t)I; a1.Kdim = (int32_t)H; a1.lists = W.lists;
     ek::FfnArgs a2 = a1;
-    a2.x = L->h; a2.x_stride = I; a2.rows = nullptr; a2.out = out; a2.out_stride = H;
+    a2.x = W.h; a2.x_stride = I; a2.rows = nullptr; a2.out = out; a2.out_stride = H;
     a2.N = (int32_t)H; a2.Kdim = (int32_t)I;
     int64_t cap[ek::kNumLists];
     for (int l = 0; l < ek::kNumLists; ++l) {
         cap[l] = ek::list_capacity(l, P, E) + (l == ek::kListStream ? extra_stream : 0);
         if (exact) cap[l] = exact[l];          // the caller built the lists on the host
-        if (cap[l] > L->list_cap[l]) cap[l] = L->list_cap[l];
+        if (cap[l] > W.list_cap[l]) cap[l] = W.list_cap[l];
         if (cap[l] < 0) cap[l] = 0;
     }
     if (wide_items > 0) {
@@ -825,8 +872,8 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
         if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, cap[ek::kListStream], false, s_stream));
         if (shared_wide > 0) {
             ek::FfnArgs aw = a;                  // the same stage over the shared segment's own list
-            aw.lists.items[ek::kListStream] = L->wide_items;
-            aw.lists.count = L->wide_count;
+            aw.lists.items[ek::kListStream] = W.wide_items;
+            aw.lists.count = W.wide_count;
             EK_HIP(ek::launch_ffn_stream(aw, stage, L->act, L->wmode, shared_wide, true, L->side_stream));
         }
         if (!tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
@@ -840,7 +887,7 @@ ek_status enqueue_ffn(ek_layer *L, const void *x, const int32_t *rows, void *out
 }
 
 // pack -> stage 1 -> stage 2 -> combine on stream s; all pointers are device.
-ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const void *w, int w_f32,
+ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const int32_t *ids, const void *w, int w_f32,
                           int64_t T, void *y, hipStream_t s)
 {
     const int64_t H = L->cfg.hidden;
@@ -852,7 +899,7 @@ ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const 
         L->events_used += 5;
     }
     if (ev) EK_HIP(hipEventRecord(ev[0], s));
-    ek::launch_pack(pack_args(L, ids, P, true), s);
+    ek::launch_pack(pack_args(L, W, ids, P, true), s);
     // the shared expert is one more segment: every token once, rows P .. P+T-1 of the packed buffers
     const bool shared = L->expert_mem[E] != nullptr && T > 0;
     // As tiles a decode-sized shared segment would occupy 8 to 14 CUs for the length of the whole
@@ -863,24 +910,24 @@ ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const 
     const bool shared_streamed = shared && T <= kSharedStreamRows;
     const bool shared_wide = shared && !shared_streamed && T <= kSharedWideRows;
     if (shared_wide) {
-        ek::WorkLists own = L->lists;
-        own.items[ek::kListStream] = L->wide_items;
-        own.count = L->wide_count;
-        ek::launch_append_segment(own, E, (int32_t)P, (int32_t)T, L->row_token, 2, s);
+        ek::WorkLists own = W.lists;
+        own.items[ek::kListStream] = W.wide_items;
+        own.count = W.wide_count;
+        ek::launch_append_segment(own, E, (int32_t)P, (int32_t)T, W.row_token, 2, s);
     } else if (shared) {
-        ek::launch_append_segment(L->lists, E, (int32_t)P, (int32_t)T, L->row_token, shared_streamed ? 1 : 0, s);
+        ek::launch_append_segment(W.lists, E, (int32_t)P, (int32_t)T, W.row_token, shared_streamed ? 1 : 0, s);
     }
     if (ev) EK_HIP(hipEventRecord(ev[1], s));
     if (P > 0) {
         const bool in_lists = shared && !shared_wide;   // the shared segment's items sit in the routed pairs' lists
-        EK_TRY(enqueue_ffn(L, x, L->row_token, L->yp, in_lists ? P + T : P, in_lists ? E + 1 : E, s, ev, 0,
+        EK_TRY(enqueue_ffn(L, W, x, W.row_token, W.yp, in_lists ? P + T : P, in_lists ? E + 1 : E, s, ev, 0,
                            shared_streamed ? (T + 15) / 16 : 0,
                            shared_wide ? (T + ek::kWideRows - 1) / ek::kWideRows : 0));
         if (ev) EK_HIP(hipEventRecord(ev[3], s));
         ek::CombineArgs c;
-        c.yp = L->yp; c.inv_perm = L->inv_perm; c.w = w; c.y = y; c.T = T; c.K = K; c.H = H;
+        c.yp = W.yp; c.inv_perm = W.inv_perm; c.w = w; c.y = y; c.T = T; c.K = K; c.H = H;
         c.act = L->act; c.w_f32 = w_f32;
-        c.shared = shared ? (const char *)L->yp + (size_t)P * H * 2 : nullptr;
+        c.shared = shared ? (const char *)W.yp + (size_t)P * H * 2 : nullptr;
         ek::launch_combine(c, s);
     } else if (ev) {
         EK_HIP(hipEventRecord(ev[2], s));
@@ -891,9 +938,9 @@ ek_status enqueue_forward(ek_layer *L, const void *x, const int32_t *ids, const 
     return EK_OK;
 }
 
-ek_status finish_blocking(ek_layer *L, hipStream_t s)
+ek_status finish_blocking(ek_layer *L, const Workspace &W, hipStream_t s)
 {
-    EK_HIP(hipMemcpyAsync(L->h_err, L->err, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    EK_HIP(hipMemcpyAsync(L->h_err, W.err, sizeof(int32_t), hipMemcpyDeviceToHost, s));
     EK_HIP(hipStreamSynchronize(s));
     bounce_flush(L);
     return err_to_status(L->h_err[0]);
@@ -1029,9 +1076,11 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
         const int w_f32 = w_dtype == EK_F32;
         std::lock_guard<std::mutex> lk(layer->mu);
         hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+        WorkspaceUse use(layer, s);
+        EK_TRY(use.begin());
         ek_status st = EK_OK;
         // a blocking call on device buffers sees everything submitted before it
-        if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
+        if (mem == EK_DEVICE && !stream) { EK_HIP(hipDeviceSynchronize()); use.device_idle(); }
         if (layer->padded) {
             EK_TRY(ensure_io_staging(layer));
             const int32_t *d_ids = ids;
@@ -1043,14 +1092,14 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
                 d_w = layer->st_w;
             }
             EK_TRY(rows_in(layer, layer->st_x, x, T, mem, s));
-            EK_TRY(enqueue_forward(layer, layer->st_x, d_ids, d_w, w_f32, T, layer->st_y, s));
+            EK_TRY(enqueue_forward(layer, layer->ws, layer->st_x, d_ids, d_w, w_f32, T, layer->st_y, s));
             EK_TRY(rows_out(layer, y, layer->st_y, T, mem, s));
-            EK_TRY(copy_route_out(layer, route, P, mem, s));
-            if (!stream) st = finish_blocking(layer, s);
+            EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
+            if (!stream) { st = finish_blocking(layer, layer->ws, s); use.synced(); }
         } else if (mem == EK_DEVICE) {
-            EK_TRY(enqueue_forward(layer, x, ids, w, w_f32, T, y, s));
-            EK_TRY(copy_route_out(layer, route, P, mem, s));
-            if (!stream) st = finish_blocking(layer, s);
+            EK_TRY(enqueue_forward(layer, layer->ws, x, ids, w, w_f32, T, y, s));
+            EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
+            if (!stream) { st = finish_blocking(layer, layer->ws, s); use.synced(); }
         } else {
             EK_TRY(ensure_io_staging(layer));
             EK_TRY(bounce_begin(layer, s, (size_t)T * H * 2 + (size_t)P * 8));
@@ -1059,11 +1108,12 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
                 EK_TRY(h2d(layer, layer->st_ids, ids, (size_t)P * 4, s));
                 EK_TRY(h2d(layer, layer->st_w, w, (size_t)P * (w_f32 ? 4 : 2), s));
             }
-            EK_TRY(enqueue_forward(layer, layer->st_x, layer->st_ids, layer->st_w, w_f32, T,
+            EK_TRY(enqueue_forward(layer, layer->ws, layer->st_x, layer->st_ids, layer->st_w, w_f32, T,
                                    layer->st_y, s));
             if (T > 0) EK_TRY(d2h(layer, y, layer->st_y, (size_t)T * H * 2, s));
-            EK_TRY(copy_route_out(layer, route, P, mem, s));
-            st = finish_blocking(layer, s);
+            EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
+            st = finish_blocking(layer, layer->ws, s);
+            use.synced();
         }
         {
             std::lock_guard<std::mutex> sl(layer->stats_mu);
@@ -1094,7 +1144,9 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
         const int64_t H = layer->user_hidden, K = layer->cfg.top_k, P = T * K;   // rows are gathered as the caller has them
         std::lock_guard<std::mutex> lk(layer->mu);
         hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
-        if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
+        WorkspaceUse use(layer, s);
+        EK_TRY(use.begin());
+        if (mem == EK_DEVICE && !stream) { EK_HIP(hipDeviceSynchronize()); use.device_idle(); }
         const int32_t *d_ids = ids;
         const void *d_x = x;
         void *d_xp = xp;
@@ -1106,17 +1158,17 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
             if (xp && T > 0) {
                 EK_TRY(h2d(layer, layer->st_x, x, (size_t)T * H * 2, s));
                 d_x = layer->st_x;
-                d_xp = layer->yp;   // [Pmax, H] scratch of the right size
+                d_xp = layer->ws.yp;   // [Pmax, H] scratch of the right size
             }
         }
-        ek::launch_pack(pack_args(layer, d_ids, P, false), s);
-        if (xp) ek::launch_gather(d_x, layer->row_token, P, H * 2, d_xp, s);
+        ek::launch_pack(pack_args(layer, layer->ws, d_ids, P, false), s);
+        if (xp) ek::launch_gather(d_x, layer->ws.row_token, P, H * 2, d_xp, s);
         EK_HIP(hipGetLastError());
         if (mem == EK_HOST && xp && P > 0) EK_TRY(d2h(layer, xp, d_xp, (size_t)P * H * 2, s));
         // the rows went into the staging buffer back to back: give a padded layer its zero columns back
         if (layer->padded && mem == EK_HOST && xp && T > 0) EK_HIP(hipMemsetAsync(layer->st_x, 0, (size_t)T * H * 2, s));
-        EK_TRY(copy_route_out(layer, route, P, mem, s));
-        if (!stream) return finish_blocking(layer, s);
+        EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
+        if (!stream) { use.synced(); return finish_blocking(layer, layer->ws, s); }
         return EK_OK;
     )
 }
@@ -1143,7 +1195,9 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
         if (!layer->expert_mem[expert])
             return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", expert);
         hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
-        if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
+        WorkspaceUse use(layer, s);
+        EK_TRY(use.begin());
+        if (mem == EK_DEVICE && !stream) { EK_HIP(hipDeviceSynchronize()); use.device_idle(); }
         if (n > 0) {
             const void *d_x = x;
             void *d_out = out;
@@ -1162,14 +1216,15 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
             // the ordinary cut's tile items: full 128-row tiles and a remainder of more than 16 rows
             const int64_t wide_items = (n + ek::kWideRows - 1) / ek::kWideRows;
             const bool wide = ek::wide_cut_pays((n >> 7) + ((n & 127) > 16), n, H, layer->cfg.inter, layer->w8 ? 1 : 2) &&
-                              wide_items <= layer->list_cap[ek::kListStream];
-            ek::launch_single_lists(layer->lists, expert, (int32_t)n, wide, s);
-            EK_TRY(enqueue_ffn(layer, d_x, nullptr, d_out, n, 1, s, nullptr, wide ? wide_items : 0));
+                              wide_items <= layer->ws.list_cap[ek::kListStream];
+            ek::launch_single_lists(layer->ws.lists, expert, (int32_t)n, wide, s);
+            EK_TRY(enqueue_ffn(layer, layer->ws, d_x, nullptr, d_out, n, 1, s, nullptr, wide ? wide_items : 0));
             if (layer->padded) EK_TRY(rows_out(layer, out, layer->st_y, n, mem, s));
             else if (mem == EK_HOST) EK_TRY(d2h(layer, out, layer->st_y, (size_t)n * H * 2, s));
         }
         if (!stream) {
             EK_HIP(hipStreamSynchronize(s));
+            use.synced();
             bounce_flush(layer);
         }
         {
@@ -1225,7 +1280,9 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             if (!layer->expert_mem[experts[i]])
                 return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", experts[i]);
         hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
-        if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
+        WorkspaceUse use(layer, s);
+        EK_TRY(use.begin());
+        if (mem == EK_DEVICE && !stream) { EK_HIP(hipDeviceSynchronize()); use.device_idle(); }
         if (P > 0) {
             // Work lists cut on the host exactly as the pack kernels cut them: a call is one
             // segment (ek_internal.h, "work lists").
@@ -1246,7 +1303,7 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             const double cover_us = (double)short_items * 3.0 * (double)H * (double)layer->cfg.inter * wb / 6.5e6;
             const double tiled_us = 15.0 + (double)(H + layer->cfg.inter) * (wb == 1 ? 0.025 : 0.0285);
             const bool wide = ek::wide_cut_pays(tile_items, P, H, layer->cfg.inter, wb) && cover_us < 0.5 * tiled_us &&
-                              wide_items <= layer->list_cap[ek::kListStream];
+                              wide_items <= layer->ws.list_cap[ek::kListStream];
             for (int i = 0; i < n_calls; ++i) {
                 const int32_t n = (int32_t)rows[i], full = n >> 7, r = n & 127;
                 if (wide) {
@@ -1268,10 +1325,10 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             size_t off[ek::kNumLists + 1];
             off[0] = 16;
             for (int l = 0; l < ek::kNumLists; ++l) {
-                if ((int64_t)items[l].size() > layer->list_cap[l])
+                if ((int64_t)items[l].size() > layer->ws.list_cap[l])
                     return fail(EK_INVALID_INPUT, "too many calls for one launch (work list %d holds %lld items)", l,
-                                (long long)layer->list_cap[l]);
-                off[l + 1] = off[l] + sizeof(ek::WorkItem) * (size_t)layer->list_cap[l];
+                                (long long)layer->ws.list_cap[l]);
+                off[l + 1] = off[l] + sizeof(ek::WorkItem) * (size_t)layer->ws.list_cap[l];
             }
             if (!layer->h_items) {
                 EK_HIP(hipHostMalloc((void **)&layer->h_items, off[ek::kNumLists], hipHostMallocDefault));
@@ -1284,11 +1341,11 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
                 cnt[l] = (int32_t)items[l].size();
                 if (cnt[l]) {
                     memcpy(layer->h_items + off[l], items[l].data(), sizeof(ek::WorkItem) * items[l].size());
-                    EK_HIP(hipMemcpyAsync(layer->lists.items[l], layer->h_items + off[l],
+                    EK_HIP(hipMemcpyAsync(layer->ws.lists.items[l], layer->h_items + off[l],
                                           sizeof(ek::WorkItem) * items[l].size(), hipMemcpyHostToDevice, s));
                 }
             }
-            EK_HIP(hipMemcpyAsync(layer->lists.count, cnt, sizeof(int32_t) * ek::kNumLists, hipMemcpyHostToDevice, s));
+            EK_HIP(hipMemcpyAsync(layer->ws.lists.count, cnt, sizeof(int32_t) * ek::kNumLists, hipMemcpyHostToDevice, s));
             EK_HIP(hipEventRecord(layer->ev_items, s));
             EK_TRY(ensure_io_staging(layer));
             // Many small host requests: their rows are gathered in pinned memory and cross the
@@ -1349,7 +1406,7 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             }
             int64_t exact[ek::kNumLists];
             for (int l = 0; l < ek::kNumLists; ++l) exact[l] = (int64_t)items[l].size();
-            EK_TRY(enqueue_ffn(layer, layer->st_x, nullptr, layer->st_y, P, n_calls, s, nullptr, wide ? wide_items : 0, 0, 0,
+            EK_TRY(enqueue_ffn(layer, layer->ws, layer->st_x, nullptr, layer->st_y, P, n_calls, s, nullptr, wide ? wide_items : 0, 0, 0,
                                wide ? nullptr : exact));
             EK_HIP(hipGetLastError());
             row0 = 0;
@@ -1379,6 +1436,7 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
         }
         if (!stream) {
             EK_HIP(hipStreamSynchronize(s));
+            use.synced();
             bounce_flush(layer);
         }
         {
@@ -1546,12 +1604,12 @@ static ek_status enqueue_chain(ek_chain *c, const void *x, const int32_t *ids, c
         ek_layer *ly = c->layers[l];
         const bool prof = ly->profiling;
         ly->profiling = false;               // no event records inside a chain (capture-safe)
-        ek_status st = enqueue_forward(ly, in, ids + (size_t)l * T * K,
+        ek_status st = enqueue_forward(ly, ly->ws, in, ids + (size_t)l * T * K,
                                        (const char *)w + (size_t)l * T * K * w_es, w_f32, T, outp, s);
         ly->profiling = prof;
         EK_TRY(st);
         // collect the layer's error word with a copy kernel-free D2D memcpy node
-        EK_HIP(hipMemcpyAsync(c->d_err + l, ly->err, sizeof(int32_t), hipMemcpyDeviceToDevice, s));
+        EK_HIP(hipMemcpyAsync(c->d_err + l, ly->ws.err, sizeof(int32_t), hipMemcpyDeviceToDevice, s));
         in = outp;
     }
     if (c->act_in) EK_TRY(rows_out(c->layers[0], y, in, T, EK_DEVICE, s));
@@ -1581,9 +1639,15 @@ ek_status ek_chain_forward(ek_chain *chain, const void *x, const int32_t *ids, c
         std::vector<std::unique_lock<std::mutex>> locks;
         for (ek_layer *ly : order) locks.emplace_back(ly->mu);
         hipStream_t s = stream ? (hipStream_t)stream : chain->stream;
+        // every layer's workspace is used on s: eagerly, or by the replay of the graph
+        std::vector<std::unique_ptr<WorkspaceUse>> uses;
+        for (ek_layer *ly : order) {
+            uses.emplace_back(new WorkspaceUse(ly, s));
+            EK_TRY(uses.back()->begin());
+        }
         const int w_f32 = w_dtype == EK_F32;
         const int L = (int)chain->layers.size();
-        if (!stream) EK_HIP(hipDeviceSynchronize());
+        if (!stream) { EK_HIP(hipDeviceSynchronize()); for (auto &u : uses) u->device_idle(); }
         if (!use_graph) {
             EK_TRY(enqueue_chain(chain, x, ids, w, w_f32, T, y, s));
         } else {
@@ -1620,6 +1684,7 @@ ek_status ek_chain_forward(ek_chain *chain, const void *x, const int32_t *ids, c
         if (!stream) {
             EK_HIP(hipMemcpyAsync(chain->h_err, chain->d_err, sizeof(int32_t) * L, hipMemcpyDeviceToHost, s));
             EK_HIP(hipStreamSynchronize(s));
+            for (auto &u : uses) u->synced();
             int32_t err = 0;
             for (int l = 0; l < L; ++l) err |= chain->h_err[l];
             return err_to_status(err);
@@ -1782,7 +1847,9 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
     const size_t l_bytes = (size_t)T * E * (rcfg->logits_dtype == EK_F32 ? 4 : 2);
     std::lock_guard<std::mutex> lk(layer->mu);
     hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
-    if (mem == EK_DEVICE && !stream) EK_HIP(hipDeviceSynchronize());
+    WorkspaceUse use(layer, s);
+    EK_TRY(use.begin());
+    if (mem == EK_DEVICE && !stream) { EK_HIP(hipDeviceSynchronize()); use.device_idle(); }
     EK_TRY(ensure_router_ws(layer, mem == EK_HOST));
     const void *d_logits = logits, *d_x = x;
     const float *d_bias = (const float *)rcfg->bias;
@@ -1818,11 +1885,11 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
     if (P > 0 && w_out) EK_TRY(give(w_out, layer->rt_w, w_bytes));
     ek_status st = EK_OK;
     if (forward) {
-        EK_TRY(enqueue_forward(layer, d_x, layer->rt_ids, layer->rt_w, w_f32, T, d_y, s));
+        EK_TRY(enqueue_forward(layer, layer->ws, d_x, layer->rt_ids, layer->rt_w, w_f32, T, d_y, s));
         if (layer->padded) EK_TRY(rows_out(layer, y, layer->st_y, T, mem, s));
         else if (mem == EK_HOST && T > 0) EK_TRY(d2h(layer, y, layer->st_y, (size_t)T * H * 2, s));
-        EK_TRY(copy_route_out(layer, route, P, mem, s));
-        if (!stream) st = finish_blocking(layer, s);
+        EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
+        if (!stream) { st = finish_blocking(layer, layer->ws, s); use.synced(); }
         std::lock_guard<std::mutex> sl(layer->stats_mu);
         layer->stats.forward_calls += 1;
         layer->stats.tokens += T;
@@ -1830,6 +1897,7 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
         if (!stream) { layer->stats.last_forward_us = tm.us(); observe_forward(layer, layer->stats.last_forward_us); }
     } else if (!stream) {
         EK_HIP(hipStreamSynchronize(s));
+        use.synced();
         bounce_flush(layer);
     }
     return st;

@@ -21,8 +21,16 @@
  *  - `stream` is a hipStream_t passed as void*.  NULL means "run on the
  *    library's own stream and return after the work has completed".  With a
  *    non-NULL stream and device pointers the call only enqueues work;
- *  - all entry points may be called from any thread.  Calls that use the same
- *    layer's workspace are serialised internally.
+ *  - all entry points may be called from any thread.  A layer has one
+ *    workspace (routing tables, work lists, packed intermediates).  Host code
+ *    that uses it runs under the layer's lock; on the device, every call makes
+ *    its stream wait for the end of the last enqueue-only call on the layer
+ *    (an event recorded when that call returned), so calls on different
+ *    streams run one after another in the order they were made and never
+ *    overlap in the workspace.  Exception: a call made while `stream` is under
+ *    capture by the caller neither waits for nor records that event; replays
+ *    of the captured graph use the workspace like the call they record, and
+ *    ordering them against other work on the same layer is the caller's part.
  */
 #ifndef EK_HIP_H
 #define EK_HIP_H

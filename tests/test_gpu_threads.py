@@ -114,3 +114,67 @@ def test_concurrent_layers_do_not_interfere(ek, cuda):
     assert not errors, errors[:3]
     for f in ffns:
         f.close()
+
+
+def test_enqueue_only_calls_on_two_streams(ek, cuda):
+    """Calls that only enqueue (device pointers and a caller's stream) return while their kernels
+    still use the layer's one workspace.  Two host threads, each with a stream of its own, keep
+    enqueuing calls with different inputs on the same layer while a third makes blocking calls on
+    host tensors (the library's own stream): every result must be bit-equal to the answer the
+    same call gives alone.  Without an ordering between the streams the routing tables and
+    intermediates of one call would be overwritten under the kernels of another."""
+    H, I, E, K = 1024, 512, 16, 4
+    dt = torch.bfloat16
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, max_tokens=700)
+    work = wl.Workload("streams", H, I, E, K, 1, dt)
+    for e in range(E):
+        layer.set_expert(e, wl.make_expert(work, e, std=0.05))
+    iters = 12
+
+    def inputs(t):
+        g = torch.Generator().manual_seed(900 + t)
+        n = [650, 37, 300][t]                      # tiles and streaming items; a decode-sized call; in between
+        x = torch.randn(n, H, generator=g).to(dt)
+        ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(n)]).to(torch.int32)
+        w = torch.rand(n, K, generator=g).to(dt)
+        return x, ids, w
+
+    ins = [inputs(t) for t in range(3)]
+    want = [layer.forward(*i) for i in ins]                      # serial answers (blocking, host tensors)
+    errors = []
+
+    def enqueuer(t):
+        try:
+            stream = torch.cuda.Stream()
+            x, ids, w = (v.to(cuda) for v in ins[t])
+            outs = [torch.zeros_like(x) for _ in range(iters)]
+            torch.cuda.synchronize()
+            for i in range(iters):
+                layer.forward(x, ids, w, stream=stream, out=outs[i])
+                if i % 4 == 3:
+                    layer.expert_forward(t, x[:20].contiguous(), stream=stream)   # another user of the workspace
+            stream.synchronize()
+            for i in range(iters):
+                if not torch.equal(outs[i].cpu().view(torch.int16), want[t].view(torch.int16)):
+                    raise AssertionError(f"stream {t}, call {i}: differs from the serial answer")
+        except Exception as ex:                 # noqa: BLE001 - reported by the main thread
+            errors.append(ex)
+
+    def blocker():
+        try:
+            for i in range(iters):
+                y = layer.forward(*ins[2])
+                if not torch.equal(y.view(torch.int16), want[2].view(torch.int16)):
+                    raise AssertionError(f"blocking host call {i}: differs from the serial answer")
+        except Exception as ex:                 # noqa: BLE001
+            errors.append(ex)
+
+    threads = [threading.Thread(target=enqueuer, args=(0,)), threading.Thread(target=enqueuer, args=(1,)),
+               threading.Thread(target=blocker)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(timeout=100)
+    assert not any(th.is_alive() for th in threads)
+    assert not errors, errors[:3]
+    layer.close()
