@@ -85,7 +85,7 @@ int64_t elem_size(int dt)
 
 // Device memory one layer call works in besides its inputs and outputs: routing tables, work
 // lists and the two packed intermediates.  Every call writes what it reads (nothing has to start
-// at zero).  A layer owns one.
+// at zero).  A layer owns one; ek_layer_forward_static carves one out of a static device array.
 struct Workspace {
     int32_t *counts = nullptr, *offsets = nullptr, *perm = nullptr, *inv_perm = nullptr;
     int32_t *row_token = nullptr, *block_hist = nullptr, *err = nullptr;
@@ -196,6 +196,8 @@ namespace {
 // beside the others, beyond that into tiles like any segment (see enqueue_forward).
 constexpr int64_t kSharedStreamRows = 64, kSharedWideRows = 256;
 constexpr int64_t kSharedWideItems = kSharedWideRows / ek::kWideRows;
+
+ek_status static_scratch_setup(int dev);   // (defined with ek_layer_forward_static's scratch array)
 
 ek_status dev_alloc(void **p, size_t bytes, const char *what)
 {
@@ -345,6 +347,7 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_ws, hipEventDisableTiming);
         if (e != hipSuccess) st = hip_fail(e, "layer setup");
     }
+    if (st == EK_OK) st = static_scratch_setup(cfg->device_id);
     if (st != EK_OK) {
         std::string keep = g_last_error;
         free_layer(L);
@@ -623,6 +626,72 @@ struct WorkspaceUse {
         else (void)hipGetLastError();
     }
 };
+
+// ---- ek_layer_forward_static: the workspace of a layer call in a static device array ----------
+// Callers that must not allocate (code under HIP graph capture, serving loops, harnesses that
+// forbid hipMalloc) get a layer call whose workspace is this array instead of memory from
+// hipMalloc.  Every GPU the library runs on holds its own copy of the array, at its own address,
+// until the process ends; the array's name is only a host-side handle, so host code takes the
+// device address once per device (static_scratch_setup, with that device current) and passes
+// that address, never the name, to kernels.
+constexpr size_t kStaticScratchBytes = EK_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+struct StaticScratch {
+    unsigned char *ptr = nullptr;            // this device's address of `scratch`
+    hipEvent_t ev = nullptr;                 // end of the last enqueue-only call that used it
+    bool busy = false;
+    std::mutex mu;                           // one call at a time carves and enqueues
+};
+StaticScratch g_static[kMaxDevices];
+std::mutex g_static_setup_mu;
+
+// Once per device, with that device current (called by ek_layer_create): address and event.
+ek_status static_scratch_setup(int dev)
+{
+    if (dev < 0 || dev >= kMaxDevices) return EK_OK;   // such a device gets no static entry point
+    std::lock_guard<std::mutex> lk(g_static_setup_mu);
+    StaticScratch &S = g_static[dev];
+    if (S.ptr) return EK_OK;
+    void *p = nullptr;
+    EK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p || ((uintptr_t)p & 255)) return fail(EK_INTERNAL, "static scratch array at %p is not 256-byte aligned", p);
+    EK_HIP(hipEventCreateWithFlags(&S.ev, hipEventDisableTiming));
+    S.ptr = (unsigned char *)p;
+    return EK_OK;
+}
+
+// Lays a workspace for T tokens of layer L out in `base` (capacity `cap` bytes).  Returns the bytes
+// needed; W is valid only if they fit.
+size_t carve_workspace(const ek_layer *L, int64_t T, unsigned char *base, size_t cap, Workspace *W)
+{
+    const int64_t E = L->cfg.n_experts, K = L->cfg.top_k, P = T * K, rows = P + T;
+    const int64_t nblocks = (P + ek::kPackChunk - 1) / ek::kPackChunk;
+    size_t off = 0;
+    auto take = [&](size_t bytes) -> void * {
+        void *p = base + off;
+        off += (bytes + 255) & ~(size_t)255;
+        return off <= cap ? p : nullptr;
+    };
+    W->counts = (int32_t *)take(sizeof(int32_t) * E);
+    W->offsets = (int32_t *)take(sizeof(int32_t) * (E + 1));
+    W->perm = (int32_t *)take(sizeof(int32_t) * P);
+    W->inv_perm = (int32_t *)take(sizeof(int32_t) * P);
+    W->row_token = (int32_t *)take(sizeof(int32_t) * rows);
+    W->block_hist = (int32_t *)take(sizeof(int32_t) * nblocks * E);
+    W->err = (int32_t *)take(sizeof(int32_t) * 4);
+    W->lists.count = (int32_t *)take(sizeof(int32_t) * ek::kNumLists);
+    W->wide_items = (ek::WorkItem *)take(sizeof(ek::WorkItem) * kSharedWideItems);
+    W->wide_count = (int32_t *)take(sizeof(int32_t) * ek::kNumLists);
+    for (int l = 0; l < ek::kNumLists; ++l) {
+        W->list_cap[l] = ek::list_capacity(l, rows, E + 1) + (l == ek::kListStream ? 264 : 1);
+        W->lists.items[l] = (ek::WorkItem *)take(sizeof(ek::WorkItem) * (size_t)W->list_cap[l]);
+    }
+    W->h = take((size_t)rows * L->cfg.inter * 2);
+    W->yp = take((size_t)rows * L->cfg.hidden * 2);
+    return off;
+}
 
 struct Timer {
     std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
@@ -1114,6 +1183,62 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
             EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
             st = finish_blocking(layer, layer->ws, s);
             use.synced();
+        }
+        {
+            std::lock_guard<std::mutex> sl(layer->stats_mu);
+            layer->stats.forward_calls += 1;
+            layer->stats.tokens += T;
+            layer->stats.pairs += P;
+            if (!stream) { layer->stats.last_forward_us = tm.us(); observe_forward(layer, layer->stats.last_forward_us); }
+        }
+        return st;
+    )
+}
+
+ek_status ek_layer_forward_static(ek_layer *layer, const void *x, const int32_t *ids, const void *w,
+                                  int32_t w_dtype, int64_t T, void *y, const ek_route_out *route, void *stream)
+{
+    EK_GUARDED(
+        if (!layer) return fail(EK_INVALID_INPUT, "layer is NULL");
+        if (T < 0 || T > layer->cfg.max_tokens)
+            return fail(EK_INVALID_INPUT, "T = %lld outside [0, max_tokens = %lld]", (long long)T,
+                        (long long)layer->cfg.max_tokens);
+        if (w_dtype != layer->cfg.act_dtype && w_dtype != EK_F32)
+            return fail(EK_INVALID_INPUT, "w_dtype must be the activation dtype or EK_F32 (got %d)", w_dtype);
+        if (T > 0 && (!x || !ids || !w || !y)) return fail(EK_INVALID_INPUT, "NULL tensor pointer");
+        if (layer->padded)
+            return fail(EK_INVALID_INPUT, "ek_layer_forward_static: hidden and inter must be multiples of 64 (128 with "
+                        "one-byte weights); padded layers stage their rows in allocated buffers");
+        const int dev = layer->cfg.device_id;
+        if (dev < 0 || dev >= kMaxDevices || !g_static[dev].ptr)
+            return fail(EK_INTERNAL, "no static scratch on device %d", dev);
+        StaticScratch &S = g_static[dev];
+        Workspace W;
+        const size_t need = carve_workspace(layer, T, S.ptr, kStaticScratchBytes, &W);
+        if (need > kStaticScratchBytes)
+            return fail(EK_INVALID_INPUT, "ek_layer_forward_static: T = %lld needs %zu bytes of workspace, the static "
+                        "scratch holds %zu; use ek_layer_forward", (long long)T, need, kStaticScratchBytes);
+        DeviceGuard dg(dev);
+        if (!dg.ok) return fail(EK_HIP_ERROR, "hipSetDevice(%d) failed", dev);
+        Timer tm;
+        const int64_t P = T * layer->cfg.top_k;
+        const int w_f32 = w_dtype == EK_F32;
+        std::lock_guard<std::mutex> lk(layer->mu);      // the layer's side stream, events and slab table
+        std::lock_guard<std::mutex> sk(S.mu);           // the device's scratch array
+        hipStream_t s = stream ? (hipStream_t)stream : layer->stream;
+        WorkspaceUse use(layer, s);
+        EK_TRY(use.begin());
+        WorkspaceUse use_scratch(S.ev, &S.busy, s);
+        EK_TRY(use_scratch.begin());
+        ek_status st = EK_OK;
+        // a blocking call sees everything submitted before it (waiting allocates nothing)
+        if (!stream) EK_HIP(hipDeviceSynchronize());
+        EK_TRY(enqueue_forward(layer, W, x, ids, w, w_f32, T, y, s));
+        EK_TRY(copy_route_out(layer, W, route, P, EK_DEVICE, s));
+        if (!stream) {
+            st = finish_blocking(layer, W, s);
+            use.synced();
+            use_scratch.synced();
         }
         {
             std::lock_guard<std::mutex> sl(layer->stats_mu);

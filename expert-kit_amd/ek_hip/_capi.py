@@ -70,6 +70,7 @@ class ek_router_cfg(ctypes.Structure):
 EK_ROUTER_MASK_NEG_INF = 1
 EK_SHARED_EXPERT = -1
 EK_CFG_BLOCK_SCALES = 1
+EK_STATIC_SCRATCH_BYTES = 32 << 20
 
 _P = ctypes.c_void_p
 _PP = ctypes.POINTER(ctypes.c_void_p)
@@ -90,6 +91,7 @@ PROTOTYPES = {
     "ek_layer_remove_expert": (_I32, [_P, _I32]),
     "ek_layer_has_expert": (_I32, [_P, _I32, ctypes.POINTER(_I32)]),
     "ek_layer_forward": (_I32, [_P, _P, _P, _P, _I32, _I64, _P, ctypes.POINTER(ek_route_out), _I32, _P]),
+    "ek_layer_forward_static": (_I32, [_P, _P, _P, _P, _I32, _I64, _P, ctypes.POINTER(ek_route_out), _P]),
     "ek_layer_pack": (_I32, [_P, _P, _I64, ctypes.POINTER(ek_route_out), _P, _P, _I32, _P]),
     "ek_layer_expert_forward": (_I32, [_P, _I32, _P, _I64, _P, _I32, _P]),
     "ek_layer_describe": (_I32, [_P, ctypes.POINTER(_I64), ctypes.POINTER(_I64), ctypes.POINTER(_I32),

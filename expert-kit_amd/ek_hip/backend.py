@@ -206,6 +206,22 @@ class HipLayer:
                                            _stream_ptr(stream)))
         return (y, rt) if return_route else y
 
+    def forward_static(self, x: torch.Tensor, ids: torch.Tensor, w: torch.Tensor, return_route: bool = False,
+                       stream=None, out: Optional[torch.Tensor] = None):
+        """ek_layer_forward_static: the same call with its workspace in the library's static device
+        array (no allocation inside the call); device tensors only.  `out` (and the routing tables,
+        which this wrapper allocates before the call) are the caller's."""
+        assert x.is_cuda and ids.is_cuda and w.is_cuda and x.dim() == 2 and w.shape == ids.shape
+        assert x.is_contiguous() and ids.is_contiguous() and w.is_contiguous()
+        assert ids.dtype == torch.int32 and x.dtype == self.act_dtype
+        T = x.shape[0]
+        y = out if out is not None else torch.empty_like(x)
+        rt, ro = self._route(T, x.device) if return_route else (None, None)
+        C.check(self._lib.ek_layer_forward_static(self._h, _ptr(x), _ptr(ids), _ptr(w), _DT[w.dtype], T, _ptr(y),
+                                                  ctypes.byref(ro) if ro is not None else None,
+                                                  _stream_ptr(stream)))
+        return (y, rt) if return_route else y
+
     def pack(self, ids: torch.Tensor, x: Optional[torch.Tensor] = None, stream=None):
         """Routing tables (and the gathered rows Xp if x is given)."""
         ids = ids.contiguous()

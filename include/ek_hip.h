@@ -206,6 +206,26 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
                            int32_t w_dtype, int64_t T, void *y, const ek_route_out *route,
                            int32_t mem, void *stream);
 
+/* ek_layer_forward for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  Same arguments, results (bit for bit) and errors as ek_layer_forward with
+ * device pointers, but the call's workspace (routing tables, work lists, the packed
+ * intermediates h [P+T, I] and y' [P+T, H]) is laid out in a static device array of
+ * EK_STATIC_SCRATCH_BYTES that each GPU holds until the process ends, and the call runs no
+ * hipMalloc / hipFree or other allocating routine.  A call whose workspace does not fit
+ * (roughly (T*K + T) * (H + I) * 2 bytes plus tables; DeepSeek-V3 shape: up to 192 tokens of
+ * top-8) fails with EK_INVALID_INPUT and a message that gives the bytes needed.  x, ids, w, y
+ * and route are device pointers; hidden and inter must be multiples of 64 (128 with one-byte
+ * weights).  All layers on a GPU share that GPU's array, which keeps the last call's contents
+ * (every call writes what it reads; nothing needs clearing): the library orders calls through
+ * this entry point on one GPU one after another on the device (as it does for a layer's own
+ * workspace), except calls made while `stream` is under capture -- replays of such graphs that
+ * overlap on one GPU race. */
+#define EK_STATIC_SCRATCH_BYTES (32u << 20)
+ek_status ek_layer_forward_static(ek_layer *layer, const void *x, const int32_t *ids, const void *w,
+                                  int32_t w_dtype, int64_t T, void *y, const ek_route_out *route,
+                                  void *stream);
+
 /* Routing only: the pack step of ek_layer_forward, plus (if xp != NULL) the
  * gather Xp[j,:] = x[perm[j]/K,:] of assemble_seq_tensors
  * (controller/executor.rs:112-133).  x may be NULL when xp is NULL. */
