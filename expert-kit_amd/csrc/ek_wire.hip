@@ -69,9 +69,13 @@ struct Cursor {
         v = *s == '-' ? -acc : acc;
         return true;
     }
-    // skips any JSON value
-    bool skip()
+    // skips any JSON value.  Wire bytes are untrusted: nesting beyond kMaxDepth is refused (the
+    // recursion would otherwise be as deep as the header is long; a safetensors header nests
+    // three levels, and the reference's parser rejects a __metadata__ that is not flat)
+    static constexpr int kMaxDepth = 32;
+    bool skip(int depth = 0)
     {
+        if (depth > kMaxDepth) return false;
         ws();
         if (p >= end) return false;
         if (*p == '"') { std::string t; return string(t); }
@@ -81,7 +85,7 @@ struct Cursor {
             if (eat(close)) return true;
             while (true) {
                 if (open == '{') { std::string k; if (!string(k) || !eat(':')) return false; }
-                if (!skip()) return false;
+                if (!skip(depth + 1)) return false;
                 if (eat(',')) continue;
                 return eat(close);
             }

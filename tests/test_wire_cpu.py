@@ -187,3 +187,33 @@ def test_parser_survives_mutated_blobs():
         else:
             bad += 1
     assert bad > 3000 and ok > 0
+
+
+def _blob_with_header(header: bytes, payload: bytes) -> bytes:
+    return struct.pack("<Q", len(header)) + header + payload
+
+
+def test_deeply_nested_header_is_refused_not_recursed_into():
+    """An unknown key (or a __metadata__) whose value nests a million levels deep must come back
+    as EK_INVALID_INPUT: the value skipper recurses once per level, and wire bytes are untrusted
+    (an unbounded recursion would overflow the worker thread's stack).  Nesting of a few levels,
+    which a real header can hold, still parses."""
+    lib = C.load()
+    data = bytes(64)
+    entry = b'"data":{"dtype":"BF16","shape":[4,8],"data_offsets":[0,64]}'
+    view = C.ek_tensor_view()
+    for depth, want in ((3, C.EK_OK), (20, C.EK_OK), (64, C.EK_INVALID_INPUT), (1_000_000, C.EK_INVALID_INPUT)):
+        for opener, closer in ((b"[", b"]"), (b'{"k":', b"}")):
+            nested = opener * depth + b"1" + closer * depth
+            # as the __metadata__ value, and as an unknown field inside a tensor's entry
+            for head in (b'{"__metadata__":' + nested + b",",
+                         b'{"other":{"dtype":"BF16","shape":[0],"data_offsets":[0,0],"extra":' + nested + b"},"):
+                key = head[:16]
+                blob = _blob_with_header(head + entry + b"}", data)
+                st = lib.ek_safetensors_find(blob, len(blob), b"data", ctypes.byref(view))
+                assert st == want, (depth, opener, key, st)
+                if want == C.EK_OK:
+                    assert view.nbytes == 64 and list(view.shape[:2]) == [4, 8]
+        # unbalanced: only openers
+        blob = _blob_with_header(b'{"x":' + b"[" * depth, data)
+        assert lib.ek_safetensors_find(blob, len(blob), b"data", ctypes.byref(view)) == C.EK_INVALID_INPUT
