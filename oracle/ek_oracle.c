@@ -452,10 +452,15 @@ static inline double silu_d(double v) { return v / (1.0 + exp(-v)); }
  * the output distribution is up to 3.5e-2 x RMS, so a max-norm gate against
  * the rounded output would be decided by 1-ulp coin flips of the last
  * rounding; this mode gives the value those flips are taken around.
+ * mode 3 ("reference-rounded, fp32 accumulation in index order"): as mode 0, but
+ * each dot product is accumulated in fp32, one term after the other, the way a
+ * scalar fp32 backend would: a second legitimate evaluation order of the same
+ * reference ops, used by the tests to show how far two faithful evaluations
+ * of the reference lie apart.
  *
  * x [n,H] (dt), w_* 16-bit of type dt (or fp32 if dt==EKO_F32).
- * out: dt in mode 0, fp32 in modes 1 and 2.  h_out (optional, may be NULL):
- * [n,I], dt in modes 0 and 2, fp32 in mode 1.
+ * out: dt in modes 0 and 3, fp32 in modes 1 and 2.  h_out (optional, may be NULL):
+ * [n,I], dt in modes 0, 2 and 3, fp32 in mode 1.
  */
 void eko_ffn(const void *x, int64_t n, int64_t H, int64_t I, const void *w_up, const void *w_gate,
              const void *w_down, int dt, int mode, void *out, void *h_out)
@@ -469,9 +474,19 @@ void eko_ffn(const void *x, int64_t n, int64_t H, int64_t I, const void *w_up, c
         for (int64_t r = 0; r < n; ++r) {
             double au = 0.0, ag = 0.0;
             const float *xr = xf + r * H;
-            for (int64_t k = 0; k < H; ++k) {
-                au += (double)xr[k] * (double)load_act(w_up, c * H + k, dt);
-                ag += (double)xr[k] * (double)load_act(w_gate, c * H + k, dt);
+            if (mode == 3) {
+                float fu = 0.0f, fg = 0.0f;
+                for (int64_t k = 0; k < H; ++k) {
+                    fu += xr[k] * load_act(w_up, c * H + k, dt);
+                    fg += xr[k] * load_act(w_gate, c * H + k, dt);
+                }
+                au = (double)fu;
+                ag = (double)fg;
+            } else {
+                for (int64_t k = 0; k < H; ++k) {
+                    au += (double)xr[k] * (double)load_act(w_up, c * H + k, dt);
+                    ag += (double)xr[k] * (double)load_act(w_gate, c * H + k, dt);
+                }
             }
             if (mode != 1) {
                 float up = round_act((float)au, dt);
@@ -494,8 +509,14 @@ void eko_ffn(const void *x, int64_t n, int64_t H, int64_t I, const void *w_up, c
         for (int64_t r = 0; r < n; ++r) {
             double a = 0.0;
             const double *hr = h + r * I;
-            for (int64_t k = 0; k < I; ++k) a += hr[k] * (double)load_act(w_down, c * I + k, dt);
-            if (mode == 0) store_act(out, r * H + c, (float)a, dt);
+            if (mode == 3) {
+                float fa = 0.0f;
+                for (int64_t k = 0; k < I; ++k) fa += (float)hr[k] * load_act(w_down, c * I + k, dt);
+                a = (double)fa;
+            } else {
+                for (int64_t k = 0; k < I; ++k) a += hr[k] * (double)load_act(w_down, c * I + k, dt);
+            }
+            if (mode == 0 || mode == 3) store_act(out, r * H + c, (float)a, dt);
             else ((float *)out)[r * H + c] = (float)a;
         }
     }
@@ -545,7 +566,7 @@ void eko_combine(const void *y3, const void *w, int64_t T, int K, int64_t H, int
  *
  * weights: arrays of E pointers (NULL allowed for experts that receive no
  * pair); mode as in eko_ffn.  In mode 1 the combine is done in double and y is
- * written as fp32 [T,H]; in mode 0 y has dtype dt; in mode 2 every tensor of
+ * written as fp32 [T,H]; in modes 0 and 3 y has dtype dt; in mode 2 every tensor of
  * the reference is rounded as in mode 0 except y itself, written as fp32.
  * route outputs (counts, offsets, perm, inv_perm) may each be NULL.
  * y3_o (may be NULL): the [T,K,H] tensor the controller hands back before the
@@ -567,8 +588,8 @@ int eko_layer_forward(const void *x, const int32_t *ids, const void *w, int64_t 
     int rc = eko_pack(ids, P, E, counts, offsets, perm, inv);
     if (rc) { free(counts); free(offsets); free(perm); free(inv); return rc; }
 
-    int ffn_mode = mode == 1 ? 1 : 0;
-    int oes = ffn_mode == 0 ? es : 4;
+    int ffn_mode = mode == 1 ? 1 : (mode == 3 ? 3 : 0);
+    int oes = ffn_mode == 1 ? 4 : es;
     char *xp = (char *)malloc((size_t)(P * H + 1) * (size_t)es);
     char *yp = (char *)malloc((size_t)(P * H + 1) * (size_t)oes);
     char *y3 = (char *)malloc((size_t)(P * H + 1) * (size_t)oes);
@@ -583,7 +604,7 @@ int eko_layer_forward(const void *x, const int32_t *ids, const void *w, int64_t 
     if (rc == 0) {
         eko_scatter(yp, H, oes, perm, P, y3);
         if (mode != 1) {
-            eko_combine(y3, w, T, K, H, dt, w_dt, mode == 0, y);
+            eko_combine(y3, w, T, K, H, dt, w_dt, mode == 0 || mode == 3, y);
         } else {
             for (int64_t t = 0; t < T; ++t)
                 for (int64_t c = 0; c < H; ++c) {

@@ -182,6 +182,7 @@ def ffn(x, w_up, w_gate, w_down, mode: int = 0, return_h: bool = False):
     mode 0: reference rounding points, result in x.dtype.
     mode 1: ideal (double, unrounded), result fp32.
     mode 2: as mode 0 with the last storage rounding left out, result fp32.
+    mode 3: as mode 0 with every dot product accumulated in fp32 in index order.
     """
     dt = _DT[x.dtype]
     assert w_up.dtype == x.dtype and w_gate.dtype == x.dtype and w_down.dtype == x.dtype
@@ -189,7 +190,7 @@ def ffn(x, w_up, w_gate, w_down, mode: int = 0, return_h: bool = False):
     n, H = x.shape
     I = w_up.shape[0]
     assert tuple(w_up.shape) == (I, H) and tuple(w_gate.shape) == (I, H) and tuple(w_down.shape) == (H, I)
-    out = torch.empty(n, H, dtype=x.dtype if mode == 0 else torch.float32)
+    out = torch.empty(n, H, dtype=x.dtype if mode in (0, 3) else torch.float32)
     h = torch.empty(n, I, dtype=torch.float32 if mode == 1 else x.dtype) if return_h else None
     lib().eko_ffn(_p(x), _i64(n), _i64(H), _i64(I), _p(w_up.contiguous()), _p(w_gate.contiguous()),
                   _p(w_down.contiguous()), dt, mode, _p(out), _p(h))
@@ -211,8 +212,9 @@ def combine(y3: torch.Tensor, w: torch.Tensor, round_out: bool = True) -> torch.
 def layer_forward(x, ids, w, w_up, w_gate, w_down, mode: int = 0, return_y3: bool = False):
     """Whole layer, Expert Kit form.  w_* are lists of E tensors (None allowed).
 
-    Returns (y, counts, offsets, perm, inv_perm); y is x.dtype (mode 0) or fp32
-    (mode 1 ideal; mode 2 reference-rounded except for y's own storage rounding).
+    Returns (y, counts, offsets, perm, inv_perm); y is x.dtype (mode 0; mode 3, the same with
+    fp32 accumulation in index order) or fp32 (mode 1 ideal; mode 2 reference-rounded except
+    for y's own storage rounding).
     With return_y3 the [T,K,H] tensor before the weighted sum is appended.
     """
     x = x.contiguous()
@@ -223,7 +225,7 @@ def layer_forward(x, ids, w, w_up, w_gate, w_down, mode: int = 0, return_y3: boo
     ids = ids.to(torch.int32).contiguous()
     w = w.contiguous()
     P = T * K
-    y = torch.empty(T, H, dtype=x.dtype if mode == 0 else torch.float32)
+    y = torch.empty(T, H, dtype=x.dtype if mode in (0, 3) else torch.float32)
     counts = torch.empty(E, dtype=torch.int32)
     offsets = torch.empty(E + 1, dtype=torch.int32)
     perm = torch.empty(P, dtype=torch.int32)

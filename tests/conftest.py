@@ -34,3 +34,11 @@ def cuda(ek):
     assert torch.cuda.is_available(), "gpu-marked test started without a GPU"
     assert ek.load().ek_device_count() >= 1
     return torch.device("cuda:0")
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The parity gates' plain figures (`-q` drops test output, not this)."""
+    import parity_report
+    for line in parity_report.summary_lines():
+        terminalreporter.write_line(line)
+    parity_report.dump_if_asked()

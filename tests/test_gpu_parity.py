@@ -1,24 +1,29 @@
 """Parity of the HIP path against the CPU oracle, through the C ABI.
 
-Bars: routing tables and the gather are bit-exact; FFN / layer outputs satisfy
-|y - y_ref| <= 2e-2 * rms(y_ref) + q, where q is the storage quantum of the
-16-bit output type.  y_ref is the oracle's reference-rounded form
-(fp32-equivalent accumulation, storage rounding after every op) taken *before
-its last storage rounding* (oracle mode 2).  Why q: the output is stored in
-bf16 / fp16, so even the exactly computed value sits up to half an ulp from
-y_ref; a bf16 ulp is 2^-7..2^-8 of the value, i.e. up to 3.5e-2 x RMS at 4.5
-sigma, so without q the gate would be decided by the last storage rounding and
-by how far the tail of the distribution reaches, not by the arithmetic.  Every
-test also asserts that the plain bound 2e-2 * rms holds for all but 1e-4 of the
-elements and prints the plain max|err| / rms.
+Bars: routing tables and the gather are bit-exact.  FFN / layer outputs: the stated tolerance
+max|y - y_ref| <= 2e-2 * rms(y_ref) is asserted as it stands by every gate call, except those that
+say plain=False next to their measured figure.  y_ref is the oracle's reference-rounded form
+(fp32-equivalent accumulation, storage rounding after every op) taken *before its last storage
+rounding* (oracle mode 2).  The exceptions assert |y - y_ref| <= 2e-2 * rms + q with q the storage
+quanta of the 16-bit tensors involved (half an ulp of y; for a layer also one ulp of the largest
+gate-weighted term), and the plain bound for all but 1e-4 of the elements: a bf16 ulp is 2^-7..2^-8
+of the value, so beyond 5 sigma the last storage rounding alone moves an output by more than
+2e-2 * rms.  tests/test_oracle_tolerance.py shows on the CPU that the reference's own arithmetic
+(libtorch, and the oracle in two accumulation orders) leaves the plain bound by exactly those
+quanta.  Every gate's plain figure, asserted or not, reaches the run's summary
+(tests/parity_report.py), next to what y_ref itself scores once rounded to the output type.
 """
+import os
+
 import pytest
 import torch
 
+import parity_report
 from ek_hip import workloads as wl
 
 pytestmark = pytest.mark.gpu
 TOL = 2e-2
+NO_PLAIN = bool(os.environ.get("EK_PARITY_NO_PLAIN"))   # survey run: record the plain figures, assert only the wide gates
 
 
 def rel_err(got: torch.Tensor, ref: torch.Tensor) -> float:
@@ -33,17 +38,30 @@ def ulp_of(v: torch.Tensor, dtype) -> torch.Tensor:
     return torch.exp2(torch.floor(torch.log2(v.float().abs().clamp_min(1e-30))) - bits)
 
 
-def ffn_gate(got: torch.Tensor, ref32: torch.Tensor, name: str, small: int = 0) -> float:
-    """One expert's gate: 2e-2 * rms plus half an output ulp (the output's own storage rounding).
-    small: outputs of a few thousand elements cannot resolve a fraction of 1e-4; that many
-    elements may then exceed the plain bound (never the full one)."""
+def rounding_floor(ref32: torch.Tensor, dtype) -> float:
+    """max|rne(y_ref) - y_ref| / rms(y_ref): what an implementation that computes y_ref exactly and
+    stores it in the 16-bit output type scores; no implementation can be held to less."""
+    rms = float(ref32.pow(2).mean().sqrt())
+    return float((ref32.to(dtype).float() - ref32).abs().max()) / max(rms, 1e-30)
+
+
+def ffn_gate(got: torch.Tensor, ref32: torch.Tensor, name: str, small: int = 0, plain: bool = True) -> float:
+    """One expert's gate.  plain (the default): the stated tolerance as it stands, every element
+    within 2e-2 * rms(y_ref).  plain=False, only where the comment at the call gives the measured
+    figure and the reason: 2e-2 * rms plus half an output ulp (the output's own storage
+    rounding), and the plain bound for all but 1e-4 of the elements (small: outputs of a few
+    thousand elements cannot resolve a fraction of 1e-4; that many elements may exceed it)."""
     rms = float(ref32.pow(2).mean().sqrt())
     err = (got.float().cpu() - ref32).abs()
     strict_viol = float((err > TOL * rms).float().mean())
     worst = float(err.max()) / rms
+    parity_report.record(name, worst, strict_viol, err.numel(), plain and not NO_PLAIN, rounding_floor(ref32, got.dtype))
     print(f"{name}: max|err|/rms = {worst:.3e}, elements over 2e-2*rms: {strict_viol:.2e}", flush=True)
     assert bool((err <= TOL * rms + 0.5 * ulp_of(ref32, got.dtype) * 1.0001).all()), worst
-    assert strict_viol <= 1e-4 or int((err > TOL * rms).sum()) <= small
+    if plain and not NO_PLAIN:
+        assert worst <= TOL, f"{name}: max|err|/rms = {worst:.3e} exceeds the plain bound"
+    else:
+        assert strict_viol <= 1e-4 or int((err > TOL * rms).sum()) <= small
     return worst
 
 
@@ -61,18 +79,19 @@ def check_vs_rounded(got: torch.Tensor, ref32: torch.Tensor, name: str = ""):
 
 
 def layer_gate(y: torch.Tensor, ref32: torch.Tensor, y3: torch.Tensor, gw: torch.Tensor, name: str,
-               small: int = 0) -> float:
+               small: int = 0, plain: bool = True) -> float:
     """The layer's parity gate.
 
-    strict : max|y - y_ref| <= 2e-2 * rms(y_ref) -- must hold for all but 1e-4 of the
-             elements, and is reported;
-    always : every element is within the strict bound plus the storage quanta of the
-             16-bit tensors involved: half an ulp of y itself (its own storage
-             rounding) and ONE ulp flip of a stored intermediate,
-             ulp(max_k |w[t,k] * Y[t,k,c]|).  The reference materialises Y[T,K,H] and
-             w*Y in the 16-bit type; fp32 accumulation order alone decides on which
-             side of a rounding boundary such a stored value falls, and for K <= 2
-             (gate weight near 1) one such flip at 3-4 sigma already exceeds 2e-2 * RMS.
+    plain  : max|y - y_ref| <= 2e-2 * rms(y_ref), the stated tolerance as it stands -- asserted
+             by default;
+    plain=False (only where the comment at the call gives the measured figure and the reason):
+             the plain bound for all but 1e-4 of the elements, and every element within the
+             plain bound plus the storage quanta of the 16-bit tensors involved: half an ulp of
+             y itself (its own storage rounding) and ONE ulp flip of a stored intermediate,
+             ulp(max_k |w[t,k] * Y[t,k,c]|).  The reference materialises Y[T,K,H] and w*Y in the
+             16-bit type; fp32 accumulation order alone decides on which side of a rounding
+             boundary such a stored value falls (tests/test_oracle_tolerance.py shows the
+             reference's own arithmetic on libtorch needing both terms).
     """
     y = y.float().cpu()
     rms = float(ref32.pow(2).mean().sqrt())
@@ -81,9 +100,16 @@ def layer_gate(y: torch.Tensor, ref32: torch.Tensor, y3: torch.Tensor, gw: torch
         + 0.5 * ulp_of(ref32, y3.dtype) * 1.0001
     strict_viol = float((err > TOL * rms).float().mean())
     worst = float(err.max()) / rms
+    parity_report.record(name, worst, strict_viol, err.numel(), plain and not NO_PLAIN, rounding_floor(ref32, y3.dtype))
+    if os.environ.get("EK_PARITY_NO_PLAIN"):
+        half_only = bool((err <= TOL * rms + 0.5 * ulp_of(ref32, y3.dtype) * 1.0001).all())
+        parity_report.RECORDS[-1]["needs_flip_term"] = not half_only
     print(f"{name}: max|err|/rms = {worst:.3e}, elements over 2e-2*rms: {strict_viol:.2e}", flush=True)
     assert bool((err <= TOL * rms + flip).all()), worst
-    assert strict_viol <= 1e-4 or int((err > TOL * rms).sum()) <= small      # see ffn_gate
+    if plain and not NO_PLAIN:
+        assert worst <= TOL, f"{name}: max|err|/rms = {worst:.3e} exceeds the plain bound"
+    else:
+        assert strict_viol <= 1e-4 or int((err > TOL * rms).sum()) <= small      # see ffn_gate
     return worst
 
 
@@ -213,7 +239,9 @@ def test_expert_forward(ek, oracle, cuda, dt, w8, n):
     ref = oracle.ffn(x, wu, wg, wd, mode=2)
     got_dev = ffn.forward(x.to(cuda))
     got_host = ffn.forward(x)
-    ffn_gate(got_dev, ref, f"expert_forward dt={dt} w8={w8} n={n}")
+    # (bf16, int8 weights, 300 rows: 2.16e-2, 1.3e-5 of the 76800 outputs beyond the plain bound; the rounding of
+    # a 7-sigma output to bf16 alone is 1.9e-2)
+    ffn_gate(got_dev, ref, f"expert_forward dt={dt} w8={w8} n={n}", plain=not (dt == torch.bfloat16 and w8 and n == 300))
     same = check_vs_rounded(got_dev, ref, f"expert_forward dt={dt} w8={w8} n={n}")
     assert same > 0.9   # same weights bit for bit (int8 ones after dequantisation): only accumulation order differs
     assert torch.equal(got_dev.cpu().view(torch.int16), got_host.view(torch.int16))
@@ -257,7 +285,9 @@ def test_tile_route_shortest_contractions(ek, oracle, cuda, H, I, w8):
     wu, wg, wd = [t[0] for t in oracle_weights(oracle, ws, 1, dt)]
     ref = oracle.ffn(x, wu, wg, wd, mode=2)
     got = layer.forward(x.to(cuda), torch.zeros(n, 1, dtype=torch.int32, device=cuda), torch.ones(n, 1, dtype=dt, device=cuda))
-    ffn_gate(got, ref, f"shortest contractions H={H} I={I} w8={w8}")
+    # 0.3 to 1.3 million outputs of 64- to 256-term contractions reach 7 sigma, where half a bf16 ulp is
+    # 2.7e-2 * rms: measured 1.6e-2 .. 2.9e-2, 3e-6 of the elements beyond the plain bound
+    ffn_gate(got, ref, f"shortest contractions H={H} I={I} w8={w8}", plain=False)
     assert check_vs_rounded(got, ref) > 0.9
     layer.close()
 
@@ -303,7 +333,7 @@ def test_expert_forward_special_cases(ek, cuda):
 
 # ------------------------------------------------------------ whole layer
 
-def run_layer_parity(ek, oracle, cuda, w, w_f32=False):
+def run_layer_parity(ek, oracle, cuda, w, w_f32=False, plain=True):
     w = wl.resolve(w)
     layer, ws = load_layer(ek, w)
     x = wl.make_x(w)
@@ -315,7 +345,7 @@ def run_layer_parity(ek, oracle, cuda, w, w_f32=False):
     ref, counts, offsets, perm, inv, y3 = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=2, return_y3=True)
     for a, b in zip((rt.counts, rt.offsets, rt.perm, rt.inv_perm), (counts, offsets, perm, inv)):
         assert torch.equal(a.cpu(), b)
-    err = layer_gate(y, ref, y3, gw, w.name)
+    err = layer_gate(y, ref, y3, gw, w.name, plain=plain)
     check_vs_rounded(y, ref, w.name)
     y_host = layer.forward(x, ids, gw)
     assert torch.equal(y_host.view(torch.int16), y.cpu().view(torch.int16))
@@ -344,7 +374,9 @@ def test_layer_small_w8(ek, oracle, cuda):
 def test_layer_ragged_lengths(ek, oracle, cuda):
     """Segment lengths from 0 to a few hundred in one call (hot expert + empty experts)."""
     w = wl.Workload("ragged", 256, 128, 24, 2, 400, torch.bfloat16, zipf_s=2.0)
-    run_layer_parity(ek, oracle, cuda, w)
+    # 2.33e-2: the distance of the correctly rounded reference output itself from y_ref on this input
+    # (tests/test_oracle_tolerance.py::test_last_storage_rounding_alone_exceeds_the_plain_bound)
+    run_layer_parity(ek, oracle, cuda, w, plain=False)
 
 
 def test_layer_c3_sampled(ek, oracle, cuda):
@@ -381,6 +413,7 @@ def test_layer_full_size_sampled_tokens(ek, oracle, cuda, name):
     between them sit in the longest segment, in a segment short enough for the streaming
     kernel, in segments whose remainder is cut into a 128-, 64- and 32-row tile (prefill), and
     four tokens drawn at random."""
+    from oracle import sampled
     w = wl.resolve(wl.CONFIGS[name])
     print(f"{name} full size: building {w.n_experts} experts on the GPU", flush=True)
     layer, ws = load_layer(ek, w, device="cuda")
@@ -389,20 +422,11 @@ def test_layer_full_size_sampled_tokens(ek, oracle, cuda, name):
     counts = torch.bincount(ids.flatten().long(), minlength=w.n_experts)
     y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
     assert torch.equal(rt.counts.cpu().long(), counts)
-    rem = counts % 128
-    classes = [counts == counts.max(), (counts > 0) & (counts <= 16), (counts > 128) & (rem > 64),
-               (counts > 128) & (rem > 32) & (rem <= 64), (counts > 128) & (rem > 16) & (rem <= 32)]
-    tokens = torch.randint(0, w.tokens, (4,), generator=torch.Generator().manual_seed(5)).tolist()
-    for c in classes:                     # the last token routed there: it sits in the segment's remainder
-        if bool(c.any()):
-            e = int(torch.where(c)[0][0])
-            tokens.append(int(torch.where((ids == e).any(dim=1))[0][-1]))
-    tokens = sorted(set(tokens))
-    need = sorted(set(ids[tokens].flatten().tolist()))
-    print(f"{name} full size: tokens {tokens}, {len(need)} experts recomputed by the oracle", flush=True)
-    wu, wg, wd = oracle_weights(oracle, {e: ws[e] for e in need}, w.n_experts, w.act_dtype)
-    ref, _, _, _, _, y3 = oracle.layer_forward(x[tokens], ids[tokens], gw[tokens], wu, wg, wd, mode=2, return_y3=True)
-    layer_gate(y[tokens], ref, y3, gw[tokens], f"{name} full size, sampled tokens")
+    tokens = sampled.choose_tokens(ids, w.n_experts)
+    print(f"{name} full size: tokens {tokens}", flush=True)
+    r = sampled.check(y[tokens], x[tokens], ids[tokens], gw[tokens], w.n_experts, lambda e: ws[e])
+    # c3: 2.72e-2 on 3 of the 43008 sampled outputs (rounding floor of the reference's own output: see the summary)
+    layer_gate(y[tokens], r["ref"], r["y3"], gw[tokens], f"{name} full size, sampled tokens", plain=name != "c3")
     assert layer.stats()["pairs"] == w.pairs
     layer.close()
 

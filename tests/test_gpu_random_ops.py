@@ -84,7 +84,7 @@ def test_random_walk(ek, oracle, cuda, w8):
                 done["wire"] += 1
             if n:
                 wu, wg, wd = ref_ws()
-                ffn_gate(got, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: expert {e}, {n} rows", small=tails(n))
+                ffn_gate(got, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: expert {e}, {n} rows", small=tails(n), plain=False)
             assert tuple(got.shape) == (n, H)
         elif op == 5:                                                 # several per-expert calls, one launch
             among = sorted(loaded) if draw(0, 3) else list(range(E))
@@ -101,7 +101,7 @@ def test_random_walk(ek, oracle, cuda, w8):
             wu, wg, wd = ref_ws()
             for (e, n), x, out in zip(calls, xs, outs):
                 if n:
-                    ffn_gate(out, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: batch, expert {e}, {n} rows", small=tails(n))
+                    ffn_gate(out, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: batch, expert {e}, {n} rows", small=tails(n), plain=False)
             done["experts"] += 1
         elif op in (6, 7, 8):                                         # the whole layer
             T = draw(0, TMAX)
@@ -124,7 +124,7 @@ def test_random_walk(ek, oracle, cuda, w8):
             if T:
                 wu, wg, wd = ref_ws()
                 ref, _, _, _, _, y3 = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=2, return_y3=True)
-                layer_gate(y, ref, y3, gw, f"step {step}: layer, T={T}", small=tails(T))
+                layer_gate(y, ref, y3, gw, f"step {step}: layer, T={T}", small=tails(T), plain=False)
             done["layer"] += 1
         else:                                                         # calls that must be refused
             kind = draw(0, 3)
