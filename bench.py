@@ -4,11 +4,15 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c1|c2]
 
 One "step" is one ek_layer_forward over one synthetic batch whose inputs and
-weights are already resident in HBM.  Prints ONE JSON line: whole-job
-token-expert pairs/s, the roofline of the dominant kernel (per-phase HIP events
-recorded on the launch stream inside the timed region) and, beside it, the
-reference-equivalent CPU backend timed on this box's host cores on a bounded
-sample of the same workload.
+weights are already resident in HBM, enqueued on a non-default stream.  Prints
+ONE JSON line: whole-job token-expert pairs/s of the decode configuration the
+metric is quoted on (c3), the roofline of its dominant kernel (per-phase HIP
+events recorded on the launch stream inside the timed region), `parity` (the
+CPU oracle's output gate on the timed input, sampled tokens), `prefill` (the
+8192-token configuration c4 measured on the same experts in the same run, with
+its MFMA roofline), `peaks` (copy / non-temporal read / MFMA ceilings measured by
+the library's microkernels) and `cpu_baseline` (the reference-equivalent CPU
+backend timed on this box's host cores on a bounded sample of the workload).
 """
 import argparse
 import json
@@ -106,7 +110,7 @@ def bench_chain(args, w, dev):
     xd = wl.make_x(w).to(dev)
     y = torch.empty_like(xd)
     chain = ek_hip.HipChain(layers)
-    stream = torch.cuda.current_stream()
+    stream = torch.cuda.Stream()          # enqueue-only calls on a stream of the caller's
     y_eager = chain.forward(xd, ids, gw, use_graph=False).clone()
     calibration_copy(args, dev)
     res = {}
@@ -120,6 +124,7 @@ def bench_chain(args, w, dev):
         for _ in range(args.steps):
             chain.forward(xd, ids, gw, use_graph=use_graph, stream=stream, out=y)
         ev1.record(stream)
+        stream.synchronize()
         torch.cuda.synchronize()
         res[mode] = max(time.perf_counter() - t0, ev0.elapsed_time(ev1) * 1e-3) / args.steps
         assert torch.equal(y.view(torch.int16), y_eager.view(torch.int16)), f"{mode} chain output changed"
@@ -147,84 +152,83 @@ def bench_chain(args, w, dev):
     print(json.dumps(out))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
-    ap.add_argument("--weights", choices=["config", "fp8"], default="config",
-                    help="fp8: the c3 / c4 layer with fp8 e4m3fn weights and 128x128 block scales kept as a "
-                         "DeepSeek-V3 checkpoint stores them, instead of the configuration's int8 per channel")
-    ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
-    ap.add_argument("--calib-copy-mib", type=int, default=0,
-                    help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
-                         "used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
-        sys.exit(2)
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
+
+def parity_on_timed_input(w, xd, ids, gw, y, x):
+    """The output gate on the very input that is timed: sampled tokens recomputed by the CPU oracle
+    (test infrastructure, outside every timed region).  Returns the plain figures; raises if an
+    output lies outside 2e-2 * rms plus the storage quanta of the 16-bit tensors."""
     import torch
-    import ek_hip
     from ek_hip import workloads as wl
+    from oracle import sampled
+    tokens = sampled.choose_tokens(ids, w.n_experts)
+    r = sampled.check(y[tokens], x[tokens], ids[tokens], gw[tokens], w.n_experts,
+                      lambda e: wl.make_expert(w, e, device="cuda"))      # (the generator gives the loaded weights again)
+    ref, y3 = r.pop("ref"), r.pop("y3")
+    bits = 7 if w.act_dtype == torch.bfloat16 else 10
+    ulp = lambda v: torch.exp2(torch.floor(torch.log2(v.float().abs().clamp_min(1e-30))) - bits)
+    rms = float(ref.pow(2).mean().sqrt())
+    quanta = 0.5 * ulp(ref) * 1.0001 + ulp((gw[tokens].float().unsqueeze(-1) * y3.float()).abs().amax(dim=1))
+    assert bool(((y[tokens].float().cpu() - ref).abs() <= 2e-2 * rms + quanta).all()), f"output parity failed: {r}"
+    r["tokens"] = tokens
+    r["y_ref"] = "CPU oracle, reference-rounded form before its last storage rounding"
+    return r
 
-    ek_hip.load()
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    dev = torch.device("cuda:0")
-    w = wl.resolve(wl.CONFIGS[args.workload])
-    if args.weights == "fp8":
-        assert w.w8, "--weights fp8 applies to the W8A16 configurations (c3, c4)"
-        from dataclasses import replace
-        w = replace(w, fp8_block=True)
-    if w.n_layers > 1:
-        return bench_chain(args, w, dev)
-    w_dtype = torch.float8_e4m3fn if w.fp8_block else torch.int8 if w.w8 else w.act_dtype
-    layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype, w_dtype=w_dtype,
-                            max_tokens=w.tokens)
+
+def time_layer(layer, w, args, dev, stream):
+    """Parity gates on the workload's input, then warm-up and K timed enqueue-only layer calls on
+    `stream` (a stream of the caller's, not the default one).  Returns the measurements."""
+    import torch
+    from ek_hip import workloads as wl
     ids, gw = wl.make_routing(w)
     counts = torch.bincount(ids.reshape(-1).long(), minlength=w.n_experts)
-    order = torch.argsort(counts, descending=True, stable=True).tolist()
-    sample_ids = sorted(order[:: max(1, w.n_experts // max(args.cpu_experts, 1))][: args.cpu_experts]) if args.cpu_experts else []
-    ws_sample = {}
-    for e in range(w.n_experts):
-        ew = wl.make_expert(w, e, device="cuda")
-        layer.set_expert(e, ew)
-        if e in sample_ids:
-            ws_sample[e] = ek_hip.ExpertWeight(*[None if t is None else t.cpu() for t in
-                                                 (ew.up_w, ew.gate_w, ew.down_w, ew.up_scale, ew.gate_scale, ew.down_scale)])
-        del ew
     x = wl.make_x(w)
     xd, idd, gwd = x.to(dev), ids.to(dev), gw.to(dev)
     y = torch.empty_like(xd)
-    stream = torch.cuda.current_stream()
 
-    # parity gate on this very input: routing tables vs a CPU stable sort
-    _, rt = layer.forward(xd, idd, gwd, return_route=True)
+    # parity gates on this very input: routing tables vs a CPU stable sort, outputs vs the oracle
+    y0, rt = layer.forward(xd, idd, gwd, return_route=True)
     ref_perm = torch.argsort(ids.reshape(-1).long(), stable=True).to(torch.int32)
     assert torch.equal(rt.perm.cpu(), ref_perm), "routing permutation mismatch"
+    parity = parity_on_timed_input(w, xd, ids, gw, y0, x) if args.parity else None
 
-    calibration_copy(args, dev)
+    torch.cuda.synchronize()
     for _ in range(args.warmup):
         layer.forward(xd, idd, gwd, stream=stream, out=y)
+    stream.synchronize()
     torch.cuda.synchronize()
     layer.profile(True)
-    t0 = time.perf_counter()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
     ev0.record(stream)
     for _ in range(args.steps):
         layer.forward(xd, idd, gwd, stream=stream, out=y)
     ev1.record(stream)
+    stream.synchronize()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     dev_s = ev0.elapsed_time(ev1) * 1e-3
     st = layer.stats()
     layer.profile(False)
+    assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), "timed calls changed the output"
     step_s = max(wall, dev_s) / args.steps
-    value = w.pairs / step_s
-
     n_prof = max(st["profiled_calls"], 1)
-    k_us = [v / n_prof for v in st["kernel_us"]]
+    return {"w": w, "x": x, "ids": ids, "gw": gw, "counts": counts, "step_s": step_s, "dev_s": dev_s / args.steps,
+            "k_us": [v / n_prof for v in st["kernel_us"]], "parity": parity}
+
+
+def roofline_of(m):
+    """Roofline of the dominant kernel of one measured workload, and the layer-level figures."""
+    w, counts, step_s, k_us = m["w"], m["counts"], m["step_s"], m["k_us"]
+    from ek_hip import workloads as wl
     active = int((counts > 0).sum())
     wsz = 1 if w.w8 else 2
     a = 2
@@ -253,28 +257,118 @@ def main():
     roof.update({"kernel": dom_name, "kernel_us": k_us[dom], "algorithmic_bytes": dom_bytes,
                  "algorithmic_flops": dom_flops})
     roof["traffic"] = measured_traffic(w.name, dom, decode=hbm_frac >= mfma_frac)
+    roof["traffic_source"] = ("profiles/pmc_traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, "
+                              "committed; not measured in this run") if roof["traffic"] is not None else None
+    layer = {"algorithmic_bytes": b_layer, "algorithmic_flops": f_layer, "hbm_frac": hbm_frac, "mfma_frac": mfma_frac,
+             "phase_us": {"pack": k_us[0], "ffn_up_gate": k_us[1], "ffn_down": k_us[2], "combine": k_us[3]},
+             "device_ms_per_step": m["dev_s"] * 1e3}
+    config = {"workload": w.name, "hidden": w.hidden, "moe_intermediate": w.inter, "experts": w.n_experts,
+              "top_k": w.top_k, "tokens": w.tokens, "pairs": w.pairs, "active_experts": active, "zipf_s": w.zipf_s,
+              "weights": "fp8 e4m3fn, 128x128 block scales" if w.fp8_block else "int8 per-channel" if w.w8 else "16-bit"}
+    return roof, layer, config
 
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--weights", choices=["config", "fp8"], default="config",
+                    help="fp8: the c3 / c4 layer with fp8 e4m3fn weights and 128x128 block scales kept as a "
+                         "DeepSeek-V3 checkpoint stores them, instead of the configuration's int8 per channel")
+    ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--no-prefill", dest="prefill", action="store_false",
+                    help="with --workload c3: do not also measure the c4 prefill call on the same experts")
+    ap.add_argument("--no-parity", dest="parity", action="store_false", help="skip the oracle's output gate before timing")
+    ap.add_argument("--no-peaks", dest="peaks", action="store_false", help="skip the copy / read / MFMA microbenchmarks")
+    ap.add_argument("--calib-copy-mib", type=int, default=0,
+                    help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
+                         "used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import ek_hip
+    from ek_hip import workloads as wl
+
+    ek_hip.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    w = wl.resolve(wl.CONFIGS[args.workload])
+    if args.weights == "fp8":
+        assert w.w8, "--weights fp8 applies to the W8A16 configurations (c3, c4)"
+        from dataclasses import replace
+        w = replace(w, fp8_block=True)
+    if w.n_layers > 1:
+        return bench_chain(args, w, dev)
+    # the decode configuration the metric is quoted on and the prefill configuration hold the same
+    # 256 experts: the default run measures both on one layer object, decode first
+    also = None
+    if args.workload == "c3" and args.prefill:
+        from dataclasses import replace
+        also = replace(wl.C4, fp8_block=w.fp8_block)
+    w_dtype = torch.float8_e4m3fn if w.fp8_block else torch.int8 if w.w8 else w.act_dtype
+    layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype, w_dtype=w_dtype,
+                            max_tokens=max(w.tokens, also.tokens if also else 0))
+    ids, gw = wl.make_routing(w)
+    counts = torch.bincount(ids.reshape(-1).long(), minlength=w.n_experts)
+    order = torch.argsort(counts, descending=True, stable=True).tolist()
+    sample_ids = sorted(order[:: max(1, w.n_experts // max(args.cpu_experts, 1))][: args.cpu_experts]) if args.cpu_experts else []
+    ws_sample = {}
+    for e in range(w.n_experts):
+        ew = wl.make_expert(w, e, device="cuda")
+        layer.set_expert(e, ew)
+        if e in sample_ids:
+            ws_sample[e] = ek_hip.ExpertWeight(*[None if t is None else t.cpu() for t in
+                                                 (ew.up_w, ew.gate_w, ew.down_w, ew.up_scale, ew.gate_scale, ew.down_scale)])
+        del ew
+    stream = torch.cuda.Stream()          # the calls are enqueue-only on a stream of the caller's
+    calibration_copy(args, dev)
+    m = time_layer(layer, w, args, dev, stream)
+    roof, layer_fig, config = roofline_of(m)
     out = {
         "metric": "token-expert pairs/s on 1 MI355X (DSv3 W8A16 layer); % HBM / MFMA roofline",
-        "value": value, "unit": "pairs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": step_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": w.pairs / m["step_s"], "unit": "pairs/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": m["step_s"] * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         # the type the MFMAs multiply in (int8 weights are dequantised to it in registers); fp32 accumulation
         "dtype": {"bfloat16": "bf16", "float16": "f16"}[str(w.act_dtype).replace("torch.", "")],
         "data": "synthetic",
-        "config": {"workload": w.name, "hidden": w.hidden, "moe_intermediate": w.inter, "experts": w.n_experts,
-                   "top_k": w.top_k, "tokens": w.tokens, "pairs": w.pairs, "active_experts": active,
-                   "zipf_s": w.zipf_s, "weights": "fp8 e4m3fn, 128x128 block scales" if w.fp8_block else "int8 per-channel" if w.w8 else "16-bit"},
+        "config": config,
+        "timed": "enqueue-only ek_layer_forward calls (device pointers) on a non-default stream; HIP events on that stream",
         "roofline": roof,
-        "layer": {"algorithmic_bytes": b_layer, "algorithmic_flops": f_layer, "hbm_frac": hbm_frac,
-                  "mfma_frac": mfma_frac,
-                  "phase_us": {"pack": k_us[0], "ffn_up_gate": k_us[1], "ffn_down": k_us[2], "combine": k_us[3]},
-                  "device_ms_per_step": dev_s / args.steps * 1e3},
+        "layer": layer_fig,
     }
+    if m["parity"] is not None:
+        out["parity"] = m["parity"]
+    if also is not None:
+        mp = time_layer(layer, also, args, dev, stream)
+        roof_p, layer_p, config_p = roofline_of(mp)
+        out["prefill"] = {"config": config_p, "value": also.pairs / mp["step_s"], "unit": "pairs/s",
+                          "ms_per_step": mp["step_s"] * 1e3, "steps": args.steps, "warmup": args.warmup,
+                          "roofline": roof_p, "layer": layer_p}
+        # the north-star figure of the prefill regime: the whole call's FLOPs against the bf16 dense peak
+        out["prefill"]["roofline_whole_call"] = {"bound": "mfma", "achieved": layer_p["algorithmic_flops"] / mp["step_s"] / 1e12,
+                                                 "peak": MFMA_PEAK_16 / 1e12, "unit": "TFLOP/s", "frac": layer_p["mfma_frac"]}
+        if mp["parity"] is not None:
+            out["prefill"]["parity"] = mp["parity"]
+    if args.peaks:
+        from ek_hip import _capi as C
+        import ctypes
+        pk = C.ek_peaks()
+        C.check(C.load().ek_measure_peaks(0, ctypes.byref(pk)))
+        out["peaks"] = {"copy_GBps": pk.copy_gbps, "nontemporal_read_GBps": pk.read_nt_gbps,
+                        "mfma_bf16_TFLOPs": pk.mfma_bf16_tflops,
+                        "source": "in-library microkernels (csrc/ek_peaks.hip), measured in this run",
+                        "published": {"hbm_GBps": HBM_PEAK / 1e9, "mfma_bf16_TFLOPs": MFMA_PEAK_16 / 1e12}}
     if args.cpu_experts:
         cores = os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"])
         torch.set_num_threads(cores)
-        v, pairs, iters = cpu_baseline(w, ws_sample, x, ids, gw)
+        v, pairs, iters = cpu_baseline(w, ws_sample, m["x"], m["ids"], m["gw"])
         out["cpu_baseline"] = {"value": v, "unit": "pairs/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "cpu_model": cpu_model(),
                                "sample": f"pairs routed to {len(ws_sample)} of {w.n_experts} experts ({pairs} pairs), "
                                          f"median of {iters} runs, libtorch CPU ops, weights pre-cast to "
                                          f"{str(w.act_dtype).replace('torch.', '')}"}

@@ -59,6 +59,10 @@ class ek_batcher_stats(ctypes.Structure):
     _fields_ = [("calls", ctypes.c_int64), ("batches", ctypes.c_int64), ("largest_batch", ctypes.c_int64)]
 
 
+class ek_peaks(ctypes.Structure):
+    _fields_ = [("copy_gbps", ctypes.c_double), ("read_nt_gbps", ctypes.c_double), ("mfma_bf16_tflops", ctypes.c_double)]
+
+
 class ek_router_cfg(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int32), ("renorm", ctypes.c_int32), ("n_group", ctypes.c_int32),
                 ("topk_group", ctypes.c_int32), ("routed_scaling", ctypes.c_float), ("flags", ctypes.c_int32),
@@ -119,6 +123,7 @@ PROTOTYPES = {
     "ek_layer_get_forward_histogram": (_I32, [_P, ctypes.POINTER(ek_histogram)]),
     "ek_layer_profile": (_I32, [_P, _I32]),
     "ek_layer_get_stats": (_I32, [_P, ctypes.POINTER(ek_stats)]),
+    "ek_measure_peaks": (_I32, [_I32, ctypes.POINTER(ek_peaks)]),
     "ek_chain_create": (_I32, [_PP, _I32, _PP]),
     "ek_chain_forward": (_I32, [_P, _P, _P, _P, _I32, _I64, _P, _I32, _P]),
     "ek_chain_destroy": (_I32, [_P]),

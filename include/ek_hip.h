@@ -360,6 +360,19 @@ typedef struct ek_histogram {
 } ek_histogram;
 ek_status ek_layer_get_forward_histogram(ek_layer *layer, ek_histogram *out);
 
+/* Ceilings measured on the device itself, for roofline lines next to the published peaks: a
+ * plain device copy (bytes read + written per second), a read-only stream with non-temporal
+ * loads (how the weight-streaming kernel reads expert weights) and a register-only bf16 MFMA
+ * loop.  No counterpart in the reference (its ek-benchmark times whole calls only,
+ * ek-benchmark/src/bench.rs:36-52).  Allocates 8 GiB for the duration of the call; takes about a
+ * second. */
+typedef struct ek_peaks {
+    double copy_gbps;        /* GB/s, read + write */
+    double read_nt_gbps;     /* GB/s */
+    double mfma_bf16_tflops; /* TFLOP/s, dense, fp32 accumulate */
+} ek_peaks;
+ek_status ek_measure_peaks(int32_t device_id, ek_peaks *out);
+
 /* Snapshot of the layer's counters (waits for recorded events to complete). */
 ek_status ek_layer_get_stats(ek_layer *layer, ek_stats *out);
 
