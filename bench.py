@@ -274,9 +274,10 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
-    ap.add_argument("--weights", choices=["config", "fp8"], default="config",
+    ap.add_argument("--weights", choices=["config", "fp8", "bf16"], default="config",
                     help="fp8: the c3 / c4 layer with fp8 e4m3fn weights and 128x128 block scales kept as a "
-                         "DeepSeek-V3 checkpoint stores them, instead of the configuration's int8 per channel")
+                         "DeepSeek-V3 checkpoint stores them, instead of the configuration's int8 per channel; "
+                         "bf16: the same layer with 16-bit weights")
     ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--no-prefill", dest="prefill", action="store_false",
                     help="with --workload c3: do not also measure the c4 prefill call on the same experts")
@@ -302,6 +303,10 @@ def main():
         assert w.w8, "--weights fp8 applies to the W8A16 configurations (c3, c4)"
         from dataclasses import replace
         w = replace(w, fp8_block=True)
+    if args.weights == "bf16":
+        assert w.w8, "--weights bf16 applies to the W8A16 configurations (c3, c4)"
+        from dataclasses import replace
+        w = replace(w, w8=False)
     if w.n_layers > 1:
         return bench_chain(args, w, dev)
     # the decode configuration the metric is quoted on and the prefill configuration hold the same
@@ -309,7 +314,7 @@ def main():
     also = None
     if args.workload == "c3" and args.prefill:
         from dataclasses import replace
-        also = replace(wl.C4, fp8_block=w.fp8_block)
+        also = replace(wl.C4, fp8_block=w.fp8_block, w8=w.w8)
     w_dtype = torch.float8_e4m3fn if w.fp8_block else torch.int8 if w.w8 else w.act_dtype
     layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype, w_dtype=w_dtype,
                             max_tokens=max(w.tokens, also.tokens if also else 0))

@@ -6,6 +6,7 @@
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <memory>
@@ -151,6 +152,14 @@ struct ek_layer {
     // the two FFN kernel families work on disjoint items, so their chains run side by side
     hipStream_t side_stream = nullptr;
     hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+    // Streams that share a hardware queue run their kernels one after the other (the runtime
+    // spreads streams over a few queues in turn), which would undo the fork: the side stream
+    // comes from a pool, and for every caller's stream the library finds once, by timing an idle
+    // kernel alone and beside itself, a pool member whose kernels do run beside that stream's.
+    static constexpr int kSidePool = 3;
+    hipStream_t side_pool[kSidePool] = {nullptr, nullptr, nullptr};
+    hipEvent_t ev_probe[4] = {nullptr, nullptr, nullptr, nullptr};
+    std::vector<std::pair<hipStream_t, hipStream_t>> side_for;   // caller's stream -> pool member
 
     ek_stats stats{};
     std::mutex stats_mu;
@@ -233,6 +242,8 @@ void free_layer(ek_layer *L)
     if (L->side_stream) (void)hipStreamDestroy(L->side_stream);
     if (L->ev_fork) (void)hipEventDestroy(L->ev_fork);
     if (L->ev_join) (void)hipEventDestroy(L->ev_join);
+    for (hipStream_t ps : L->side_pool) if (ps && ps != L->side_stream) (void)hipStreamDestroy(ps);
+    for (hipEvent_t ev : L->ev_probe) if (ev) (void)hipEventDestroy(ev);
     if (L->ev_ws) (void)hipEventDestroy(L->ev_ws);
     delete L;
 }
@@ -344,6 +355,10 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->side_stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_fork, hipEventDisableTiming);
         if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_join, hipEventDisableTiming);
+        L->side_pool[0] = L->side_stream;
+        for (int i = 1; i < ek_layer::kSidePool && e == hipSuccess; ++i)
+            e = hipStreamCreateWithFlags(&L->side_pool[i], hipStreamNonBlocking);
+        for (int i = 0; i < 4 && e == hipSuccess; ++i) e = hipEventCreate(&L->ev_probe[i]);
         if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_ws, hipEventDisableTiming);
         if (e != hipSuccess) st = hip_fail(e, "layer setup");
     }
@@ -865,6 +880,43 @@ ek::PackArgs pack_args(ek_layer *L, const Workspace &W, const int32_t *ids, int6
     return a;
 }
 
+// The side stream to fork to from stream s (the caller holds L->mu).  Decided once per caller's
+// stream: an idle kernel of ~100 us is timed alone on s, then on s and on a pool member at once;
+// the first member beside which the pair takes clearly less than twice the time runs its kernels
+// beside s's.  This first use waits for s on the host (a few hundred microseconds).  A stream under
+// capture is not probed (a graph's branches are not bound to the streams they were recorded on).
+hipStream_t pick_side_stream(ek_layer *L, hipStream_t s)
+{
+    for (const auto &p : L->side_for) if (p.first == s) return p.second;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cs) != hipSuccess) { (void)hipGetLastError(); return L->side_stream; }
+    if (cs != hipStreamCaptureStatusNone) return L->side_stream;
+    hipStream_t chosen = L->side_stream;
+    constexpr int kIters = 200;            // ~200k cycles: far above launch jitter
+    hipEvent_t *ev = L->ev_probe;
+    bool ok = hipEventRecord(ev[0], s) == hipSuccess;
+    if (ok) { ek::launch_idle(kIters, s); ok = hipEventRecord(ev[1], s) == hipSuccess; }
+    float alone = 0.f;
+    if (ok) ok = hipEventSynchronize(ev[1]) == hipSuccess && hipEventElapsedTime(&alone, ev[0], ev[1]) == hipSuccess;
+    for (int i = 0; i < ek_layer::kSidePool && ok; ++i) {
+        hipStream_t c = L->side_pool[i];
+        if (c == s) continue;
+        ok = hipEventRecord(ev[0], s) == hipSuccess && hipStreamWaitEvent(c, ev[0], 0) == hipSuccess;
+        if (!ok) break;
+        ek::launch_idle(kIters, s);
+        ek::launch_idle(kIters, c);
+        ok = hipEventRecord(ev[2], c) == hipSuccess && hipStreamWaitEvent(s, ev[2], 0) == hipSuccess &&
+             hipEventRecord(ev[3], s) == hipSuccess && hipEventSynchronize(ev[3]) == hipSuccess;
+        float both = 0.f;
+        if (ok) ok = hipEventElapsedTime(&both, ev[0], ev[3]) == hipSuccess;
+        if (ok && both < 1.6f * alone) { chosen = c; break; }
+    }
+    if (!ok) (void)hipGetLastError();
+    if (L->side_for.size() >= 64) L->side_for.erase(L->side_for.begin());   // (streams come and go)
+    L->side_for.emplace_back(s, chosen);
+    return chosen;
+}
+
 // Both FFN stages over the work lists in W.lists: x [*, H] (rows picked through
 // `rows`, or packed order when nullptr) -> W.h -> out [P, H].  P and E bound the
 // list lengths (grid sizes); ev, if set, receives the stage boundary event.
@@ -929,11 +981,13 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
     const bool fork = have_stream && have_tiles &&
                       (P > 4 * E ? P <= 128 * E || small_expert : tiles_lately);
     hipStream_t s_stream = s, s_tiles = s;
+    hipStream_t side = nullptr;
     if (fork || shared_wide > 0) {
+        side = pick_side_stream(L, s);
         EK_HIP(hipEventRecord(L->ev_fork, s));
-        EK_HIP(hipStreamWaitEvent(L->side_stream, L->ev_fork, 0));
+        EK_HIP(hipStreamWaitEvent(side, L->ev_fork, 0));
     }
-    if (fork) (tiles_main ? s_stream : s_tiles) = L->side_stream;
+    if (fork) (tiles_main ? s_stream : s_tiles) = side;
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
         const bool tiles_first = fork;
@@ -943,13 +997,13 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
             ek::FfnArgs aw = a;                  // the same stage over the shared segment's own list
             aw.lists.items[ek::kListStream] = W.wide_items;
             aw.lists.count = W.wide_count;
-            EK_HIP(ek::launch_ffn_stream(aw, stage, L->act, L->wmode, shared_wide, true, L->side_stream));
+            EK_HIP(ek::launch_ffn_stream(aw, stage, L->act, L->wmode, shared_wide, true, side));
         }
         if (!tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
     }
     if (fork || shared_wide > 0) {
-        EK_HIP(hipEventRecord(L->ev_join, L->side_stream));
+        EK_HIP(hipEventRecord(L->ev_join, side));
         EK_HIP(hipStreamWaitEvent(s, L->ev_join, 0));
     }
     return EK_OK;

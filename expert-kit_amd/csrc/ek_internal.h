@@ -193,6 +193,9 @@ struct RowCopy {
 // kernel has run
 void launch_rows_copy(const RowCopy *segs, int n, hipStream_t s);
 
+// one wave idling for iters x ~1000 cycles (see pick_side_stream in ek_capi.hip)
+void launch_idle(int iters, hipStream_t s);
+
 // ---- weight ingestion -------------------------------------------------------
 // src [N, K] row-major of src_dtype (ek_dtype numbering) -> chunked layout at
 // dst, matrix m of an nmat-group.  dst_dtype: 0 bf16, 1 f16, 3 int8.  block_scale (16-bit

@@ -191,4 +191,17 @@ void launch_scales_to_f32(const void *src, int src_dtype, int64_t n, float *dst,
                        n, dst);
 }
 
+// A kernel that does nothing for a fixed time (one wave, `iters` sleeps of about 1000 cycles):
+// the host times it alone and beside a copy of itself on another stream to learn whether the two
+// streams can run kernels side by side (streams that share a hardware queue cannot).
+__global__ void idle_kernel(int iters)
+{
+    for (int i = 0; i < iters; ++i) __builtin_amdgcn_s_sleep(16);
+}
+
+void launch_idle(int iters, hipStream_t s)
+{
+    hipLaunchKernelGGL(idle_kernel, dim3(1), dim3(64), 0, s, iters);
+}
+
 }  // namespace ek
