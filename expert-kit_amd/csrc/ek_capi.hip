@@ -955,12 +955,15 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
     }
     // Two independent chains: the weight-streaming kernel (items of <= 16 rows) and the
     // MFMA tile kernel (longer items) touch disjoint rows of h and out, and run side by side:
-    // one chain is forked to the side stream and joined before returning.  The chain with
-    // most of the work stays on s, and the tile kernel is launched first: a tile workgroup
-    // takes a whole CU (registers and LDS), so its persistent workgroups claim as many CUs as
-    // they have tiles at once and the streaming kernel runs on the others, instead of the tiles
-    // waiting for streaming workgroups to drain (in that order Qwen3 fp16 decode at 256 tokens
-    // takes 0.235 ms, in this one 0.221 ms).  With tiles for all 256 CUs the two run in turn.
+    // the streaming chain is forked to the side stream and joined before returning.  The tile
+    // chain stays on s: a tile workgroup takes a whole CU (registers and LDS), so its persistent
+    // workgroups should claim as many CUs as they have tiles at once and leave the others to the
+    // streaming kernel, instead of waiting for streaming workgroups to drain CU by CU.  Which kernel
+    // the device starts first is decided by the queues, not by the order of the launches: the
+    // kernel on s follows the pack kernel in its own queue at once, the one on the side stream
+    // only when the fork's event has crossed to the other queue, ~6 us later (Qwen3 fp16 decode at
+    // 256 tokens, enqueue-only calls: tile kernel second 128 us and 0.216 ms per call, first 88 us
+    // and 0.201 ms).  With tiles for all 256 CUs the two run in turn.
     // Measured on MI355X against running both in order: Qwen3 fp16 (E 128, K 8) 512 / 1024 /
     // 2048 / 4096 / 16384 tokens -7 / -11 / -2 / -1 / 0 %, the ragged 4-layer chain -4.8 %;
     // DeepSeek-V3 int8 (E 128) -2 / -5 / -3 / 0 / 0 %; with its 16-bit weights (E 64) -7 / -4 /
@@ -973,7 +976,6 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
     // fork/join costs 10-20 us for nothing.  Skew persists from one call to the next, so the last
     // pack's tile count, which its kernel left in pinned memory, decides; it may be a call or two
     // old, and either choice computes the same bits.
-    const bool tiles_main = P > 16 * E;
     const bool have_stream = cap[ek::kListStream] > 0;
     const bool have_tiles = cap[ek::kListT32] + cap[ek::kListT64] + cap[ek::kListT128] > 0;
     const bool small_expert = 3 * H * I * (L->w8 ? 1 : 2) <= (16ll << 20);
@@ -987,7 +989,7 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
         EK_HIP(hipEventRecord(L->ev_fork, s));
         EK_HIP(hipStreamWaitEvent(side, L->ev_fork, 0));
     }
-    if (fork) (tiles_main ? s_stream : s_tiles) = side;
+    if (fork) s_stream = side;
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
         const bool tiles_first = fork;
