@@ -205,7 +205,10 @@ def time_layer(layer, w, args, dev, stream):
         layer.forward(xd, idd, gwd, stream=stream, out=y)
     stream.synchronize()
     torch.cuda.synchronize()
-    layer.profile(True)
+    # per-phase events on every fourth timed call: five event records cost a decode-sized call ~15 us
+    # of gaps on the device, which is measurement, not the library
+    every = 4 if args.steps >= 8 else 1
+    layer.profile(every)
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     ev0.record(stream)
@@ -222,7 +225,7 @@ def time_layer(layer, w, args, dev, stream):
     step_s = max(wall, dev_s) / args.steps
     n_prof = max(st["profiled_calls"], 1)
     return {"w": w, "x": x, "ids": ids, "gw": gw, "counts": counts, "step_s": step_s, "dev_s": dev_s / args.steps,
-            "k_us": [v / n_prof for v in st["kernel_us"]], "parity": parity}
+            "k_us": [v / n_prof for v in st["kernel_us"]], "parity": parity, "phase_calls": st["profiled_calls"]}
 
 
 def roofline_of(m):
@@ -261,6 +264,7 @@ def roofline_of(m):
                               "committed; not measured in this run") if roof["traffic"] is not None else None
     layer = {"algorithmic_bytes": b_layer, "algorithmic_flops": f_layer, "hbm_frac": hbm_frac, "mfma_frac": mfma_frac,
              "phase_us": {"pack": k_us[0], "ffn_up_gate": k_us[1], "ffn_down": k_us[2], "combine": k_us[3]},
+             "phase_events": f"HIP events around the four phases on {m['phase_calls']} of the timed calls (every fourth)",
              "device_ms_per_step": m["dev_s"] * 1e3}
     config = {"workload": w.name, "hidden": w.hidden, "moe_intermediate": w.inter, "experts": w.n_experts,
               "top_k": w.top_k, "tokens": w.tokens, "pairs": w.pairs, "active_experts": active, "zipf_s": w.zipf_s,

@@ -171,6 +171,8 @@ struct ek_layer {
 
     // per-phase event timing (ek_layer_profile)
     bool profiling = false;
+    int profile_every = 1;                   // record the events of every n-th call only
+    int64_t profile_tick = 0;
     std::vector<hipEvent_t> events;          // 5 per recorded call
     size_t events_used = 0;
 };
@@ -1019,7 +1021,7 @@ ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const 
     const int E = L->cfg.n_experts, K = L->cfg.top_k;
     const int64_t P = T * K;
     hipEvent_t *ev = nullptr;
-    if (L->profiling && L->events_used + 5 <= L->events.size()) {
+    if (L->profiling && L->profile_tick++ % L->profile_every == 0 && L->events_used + 5 <= L->events.size()) {
         ev = L->events.data() + L->events_used;
         L->events_used += 5;
     }
@@ -1675,6 +1677,8 @@ ek_status ek_layer_profile(ek_layer *layer, int32_t enable)
         if (layer->events_used) EK_HIP(hipEventSynchronize(layer->events[layer->events_used - 1]));
         layer->events_used = 0;
         layer->profiling = enable != 0;
+        layer->profile_every = enable > 1 ? enable : 1;
+        layer->profile_tick = 0;
         std::lock_guard<std::mutex> sl(layer->stats_mu);
         for (double &v : layer->stats.kernel_us) v = 0.0;
         layer->stats.profiled_calls = 0;

@@ -330,7 +330,8 @@ class HipLayer:
         C.check(self._lib.ek_layer_get_forward_histogram(self._h, ctypes.byref(h)))
         return {"le": list(h.le), "cumulative": list(h.cumulative), "sum": h.sum, "count": h.count}
 
-    def profile(self, enable: bool) -> None:
+    def profile(self, enable) -> None:
+        """True / 1: per-phase events on every call; n > 1: on every n-th call; False / 0: off."""
         C.check(self._lib.ek_layer_profile(self._h, int(enable)))
 
     def stats(self) -> dict:

@@ -336,7 +336,9 @@ ek_status ek_batcher_forward(ek_batcher *batcher, const char *expert_id, const v
 ek_status ek_batcher_get_stats(ek_batcher *batcher, ek_batcher_stats *out);
 ek_status ek_batcher_destroy(ek_batcher *batcher);
 
-/* Turns per-phase HIP-event timing of ek_layer_forward on (1) or off (0) and
+/* Turns per-phase HIP-event timing of ek_layer_forward on (1: every call; n > 1: every n-th
+ * call, the first included -- five event records cost a decode-sized call ~15 us of gaps on
+ * the device, sampling keeps a timed loop close to its unobserved speed) or off (0) and
  * clears the accumulated kernel_us.  Stands for the PerfTimer checkpoints of
  * the reference (ek-base/src/utils.rs:4-45; controller/executor.rs:136,201,228).
  * At most 1024 calls are recorded between two ek_layer_get_stats calls. */
