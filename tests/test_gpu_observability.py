@@ -95,3 +95,34 @@ def test_chain_counts_every_layer(ek, cuda):
     chain.close()
     for layer in layers:
         layer.close()
+
+
+def test_phase_timing_every_call_and_sampled(ek, cuda):
+    """ek_layer_profile(1) records the four phases of every fused call, ek_layer_profile(n) of every
+    n-th call beginning with the first (the PerfTimer checkpoints of the reference stand behind it:
+    ek-base/src/utils.rs:4-45); turning it off or on again clears what was accumulated; results
+    do not depend on it."""
+    H, I, E, K, T = 256, 128, 8, 2, 64
+    dt = torch.bfloat16
+    layer = ek.HipLayer(H, I, E, K, act_dtype=dt, max_tokens=T)
+    work = wl.Workload("phases", H, I, E, K, T, dt)
+    for e in range(E):
+        layer.set_expert(e, wl.make_expert(work, e, std=0.05))
+    x = wl.make_x(work).to(cuda)
+    ids, gw = wl.make_routing(work)
+    ids, gw = ids.to(cuda), gw.to(cuda)
+    y0 = layer.forward(x, ids, gw)
+    assert layer.stats()["profiled_calls"] == 0
+    stream = torch.cuda.Stream()
+    for every, calls, want in ((1, 6, 6), (4, 10, 3), (3, 3, 1), (True, 2, 2)):
+        layer.profile(every)
+        for i in range(calls):
+            y = layer.forward(x, ids, gw, stream=stream if i % 2 else None)
+            stream.synchronize()
+            assert torch.equal(y.view(torch.int16), y0.view(torch.int16))
+        st = layer.stats()
+        assert st["profiled_calls"] == want, (every, st["profiled_calls"])
+        assert all(v > 0 for v in st["kernel_us"]) and sum(st["kernel_us"]) < 1e6 * want
+        layer.profile(False)
+        assert layer.stats()["profiled_calls"] == 0 and sum(layer.stats()["kernel_us"]) == 0
+    layer.close()
