@@ -68,6 +68,19 @@ __device__ __forceinline__ void block_barrier()
     asm volatile("s_barrier" : : : "memory");
 }
 
+// Timing-only builds (`make ablation ABL=...`, WRONG RESULTS, never the shipped library): the
+// tile kernel with one part of its step left out, to measure what that part costs in cycles
+// and in clock under the chip's power limit.
+//   EK_ABL_NO_DMA      no LDS-DMA after a workgroup's first loads (tiles compute on stale data)
+//   EK_ABL_NO_MFMA     no MFMA in the step loop;  EK_ABL_HALF_MFMA  every second row block's only
+//   EK_ABL_NO_DEQUANT  one-byte weights are fed to the MFMAs as they are stored
+#if defined(EK_ABL_HALF_MFMA)
+#define EK_ABL_MFMA(rb) ((rb) < (RB + 1) / 2)
+#elif defined(EK_ABL_NO_MFMA)
+#define EK_ABL_MFMA(rb) ((rb) < 0)
+#else
+#define EK_ABL_MFMA(rb) true
+#endif
 constexpr int kTileThreads = 512;
 constexpr int kTileWaves = 8;
 constexpr int kCusPerXcd = 32;   // MI355X: 8 XCDs x 32 CUs
@@ -295,11 +308,13 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                                // previous step is free again
             if (step == fstep) tn = fetch(tc + stride, nxt, cur.sslot ^ 1);
             const int ring2 = ring + AHEAD >= NS ? ring + AHEAD - NS : ring + AHEAD;   // (ring + AHEAD) % NS
+#ifndef EK_ABL_NO_DMA
             if (step + AHEAD < nsteps) {
                 EK_ISSUE(cur, step + AHEAD, ring2);
             } else if (tn >= 0) {
                 EK_ISSUE(nxt, step + AHEAD - nsteps, ring2);
             }
+#endif
 
             const uint8_t *stage = lds + ring * G::STAGE;
             const uint8_t *wreg = stage + w_off;
@@ -317,6 +332,9 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                     sblk[cb] = sc_area[cur.sslot * kScaleSlotFloats + cb * kTileScaleBlocks + (step >> 1)];
             }
             auto dq = [&](uint32_t w, int cb) -> u32x2 {
+#ifdef EK_ABL_NO_DEQUANT
+                return u32x2{w, w ^ (uint32_t)cb};
+#endif
                 if constexpr (WM == kWF8Block) return dequant_f8x4<T>(w, sblk[cb]);
                 else if constexpr (WM == kWI8Block) return dequant_u8x4<T>(w, sblk[cb], -128.f * sblk[cb]);
                 else return dequant_u8x4<T>(w, cur.as[cb], cur.ac[cb]);
@@ -331,7 +349,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             // the conversion of that step's first k-group, which nothing else could overlap.
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
-                if (step > 0) {
+                if (step > 0 && EK_ABL_MFMA(rb)) {
 #pragma unroll
                     for (int cb = 0; cb < CB; ++cb)
                         acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[1][cb]), bf[1][rb], acc[rb][cb]);
@@ -359,9 +377,11 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
                     bf[ng][rb] = *(const V8 *)(stage + boff[grp + 1] + rb * kRowBlockBytes);
+                    if (EK_ABL_MFMA(rb)) {
 #pragma unroll
-                    for (int cb = 0; cb < CB; ++cb)
-                        acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cg][cb]), bf[cg][rb], acc[rb][cb]);
+                        for (int cb = 0; cb < CB; ++cb)
+                            acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cg][cb]), bf[cg][rb], acc[rb][cb]);
+                    }
                     if constexpr (W8) {
                         // next group's A operands: 4 dwords (2 per column block) spread over the row blocks
                         constexpr int DW = 4 / RB;
