@@ -49,7 +49,8 @@ def check(y_rows: torch.Tensor, x_rows: torch.Tensor, ids_rows: torch.Tensor, gw
     """y_rows: the call's output for the sampled tokens; x_rows / ids_rows / gw_rows: their inputs
     (CPU tensors); weights_of(e) -> the ExpertWeight loaded as expert e.  Returns the plain figures
     against the oracle's reference-rounded form (mode 2) and its fp32-accumulate ideal form (mode 1),
-    and the tensors the tests' gates need."""
+    what the reference's own ops evaluated by libtorch score against the same y_ref on the same
+    tokens, and the tensors the tests' gates need."""
     dt = x_rows.dtype
     need = sorted(set(ids_rows.flatten().tolist()))
     wu, wg, wd = [None] * n_experts, [None] * n_experts, [None] * n_experts
@@ -57,6 +58,8 @@ def check(y_rows: torch.Tensor, x_rows: torch.Tensor, ids_rows: torch.Tensor, gw
         wu[e], wg[e], wd[e] = reference_weights(weights_of(e), dt)
     ref, _, _, _, _, y3 = oracle.layer_forward(x_rows, ids_rows, gw_rows, wu, wg, wd, mode=2, return_y3=True)
     ideal = oracle.layer_forward(x_rows, ids_rows, gw_rows, wu, wg, wd, mode=1)[0]
+    # the reference's own op sequence on libtorch (the library the reference calls), same tokens
+    twin, _ = oracle.torch_layer_forward(x_rows, ids_rows, gw_rows, wu, wg, wd)
     y = y_rows.float().cpu()
     rms = float(ref.pow(2).mean().sqrt())
     err = (y - ref).abs()
@@ -65,4 +68,5 @@ def check(y_rows: torch.Tensor, x_rows: torch.Tensor, ids_rows: torch.Tensor, gw
             "max_err_over_rms_vs_fp32_ideal": float(err_i.max()) / float(ideal.pow(2).mean().sqrt()),
             "over_frac_vs_fp32_ideal": float((err_i > tol * rms).float().mean()),
             "y_ref_rounded_to_output_type": float((ref.to(dt).float() - ref).abs().max()) / rms,
+            "reference_ops_on_libtorch_max_err_over_rms": float((twin.float() - ref).abs().max()) / rms,
             "elements": int(err.numel()), "experts_recomputed": len(need), "ref": ref, "y3": y3}
