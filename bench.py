@@ -221,7 +221,8 @@ def time_layer(layer, w, args, dev, stream):
     dev_s = ev0.elapsed_time(ev1) * 1e-3
     st = layer.stats()
     layer.profile(False)
-    assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), "timed calls changed the output"
+    if args.repeat_check:
+        assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), "timed calls changed the output"
     step_s = max(wall, dev_s) / args.steps
     n_prof = max(st["profiled_calls"], 1)
     return {"w": w, "x": x, "ids": ids, "gw": gw, "counts": counts, "step_s": step_s, "dev_s": dev_s / args.steps,
@@ -287,6 +288,9 @@ def main():
                     help="with --workload c3: do not also measure the c4 prefill call on the same experts")
     ap.add_argument("--no-parity", dest="parity", action="store_false", help="skip the oracle's output gate before timing")
     ap.add_argument("--no-peaks", dest="peaks", action="store_false", help="skip the copy / read / MFMA microbenchmarks")
+    ap.add_argument("--no-repeat-check", dest="repeat_check", action="store_false",
+                    help="do not require the timed calls to reproduce the first call's output bit for bit (only for "
+                         "the timing-only ablation builds of the library, whose results are wrong by construction)")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
                          "used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -370,6 +374,8 @@ def main():
         C.check(C.load().ek_measure_peaks(0, ctypes.byref(pk)))
         out["peaks"] = {"copy_GBps": pk.copy_gbps, "nontemporal_read_GBps": pk.read_nt_gbps,
                         "mfma_bf16_TFLOPs": pk.mfma_bf16_tflops,
+                        "mfma_bf16_random_operands_TFLOPs": pk.mfma_bf16_random_tflops,
+                        "mfma_bf16_with_int8_dequant_TFLOPs": pk.mfma_bf16_dequant_tflops,
                         "source": "in-library microkernels (csrc/ek_peaks.hip), measured in this run",
                         "published": {"hbm_GBps": HBM_PEAK / 1e9, "mfma_bf16_TFLOPs": MFMA_PEAK_16 / 1e12}}
     if args.cpu_experts:

@@ -74,12 +74,26 @@ __device__ __forceinline__ void block_barrier()
 //   EK_ABL_NO_DMA      no LDS-DMA after a workgroup's first loads (tiles compute on stale data)
 //   EK_ABL_NO_MFMA     no MFMA in the step loop;  EK_ABL_HALF_MFMA  every second row block's only
 //   EK_ABL_NO_DEQUANT  one-byte weights are fed to the MFMAs as they are stored
+//   EK_ABL_NO_BARRIER  no workgroup barrier per step
+//   EK_ABL_NO_VMWAIT   a step does not wait for its own LDS-DMA (one-byte weights)
+//   EK_ABL_NO_WDMA / EK_ABL_NO_XDMA  no LDS-DMA of the weights / of the activation tile at all
+// Several can be combined by giving the compiler more than one -DEK_ABL_... flag.
 #if defined(EK_ABL_HALF_MFMA)
 #define EK_ABL_MFMA(rb) ((rb) < (RB + 1) / 2)
 #elif defined(EK_ABL_NO_MFMA)
 #define EK_ABL_MFMA(rb) ((rb) < 0)
 #else
 #define EK_ABL_MFMA(rb) true
+#endif
+#if defined(EK_ABL_NO_WDMA)
+#define EK_ABL_WDMA false
+#else
+#define EK_ABL_WDMA true
+#endif
+#if defined(EK_ABL_NO_XDMA)
+#define EK_ABL_XDMA false
+#else
+#define EK_ABL_XDMA true
 #endif
 constexpr int kTileThreads = 512;
 constexpr int kTileWaves = 8;
@@ -255,9 +269,11 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
         _Pragma("unroll") for (int nr = 0; nr < NR; ++nr)                                       \
         _Pragma("unroll") for (int m = 0; m < NMAT; ++m)                                        \
         _Pragma("unroll") for (int kc = 0; kc < KC; ++kc)                                       \
+            if (EK_ABL_WDMA)                                                                    \
             dma16((ctx).wp[nr] + (int64_t)(((step) * KC + kc) * NMAT + m) * kChunkBytes,        \
                   st_ + w_off + ((nr * NMAT + m) * KC + kc) * kChunkBytes);                     \
-        _Pragma("unroll") for (int i = 0; i < LX; ++i) dma16((ctx).xsrc[i] + (step) * BK, st_ + xdst[i]); \
+        _Pragma("unroll") for (int i = 0; i < LX; ++i)                                          \
+            if (EK_ABL_XDMA) dma16((ctx).xsrc[i] + (step) * BK, st_ + xdst[i]);                 \
     }
 
     Ctx cur, nxt;
@@ -293,8 +309,10 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             // the next tile) and than the previous epilogue's stores: wait until only those remain
             if constexpr (AHEAD == 2) {
                 if (step + 1 < nsteps || tn >= 0) {
+#ifndef EK_ABL_NO_VMWAIT
                     if (step < 2 && pend_st) wait_vmcnt_dyn(LOADS + pend_st);
                     else wait_vmcnt<LOADS>();
+#endif
                 } else {
                     wait_vmcnt<0>();
                 }
@@ -304,8 +322,10 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                 if (step == 0 && pend_st) wait_vmcnt_dyn(pend_st);
                 else wait_vmcnt<0>();
             }
+#ifndef EK_ABL_NO_BARRIER
             block_barrier();   // this step's tile is visible to all waves; the stage of the
                                // previous step is free again
+#endif
             if (step == fstep) tn = fetch(tc + stride, nxt, cur.sslot ^ 1);
             const int ring2 = ring + AHEAD >= NS ? ring + AHEAD - NS : ring + AHEAD;   // (ring + AHEAD) % NS
 #ifndef EK_ABL_NO_DMA

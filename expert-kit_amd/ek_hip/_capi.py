@@ -60,7 +60,8 @@ class ek_batcher_stats(ctypes.Structure):
 
 
 class ek_peaks(ctypes.Structure):
-    _fields_ = [("copy_gbps", ctypes.c_double), ("read_nt_gbps", ctypes.c_double), ("mfma_bf16_tflops", ctypes.c_double)]
+    _fields_ = [("copy_gbps", ctypes.c_double), ("read_nt_gbps", ctypes.c_double), ("mfma_bf16_tflops", ctypes.c_double),
+                ("mfma_bf16_random_tflops", ctypes.c_double), ("mfma_bf16_dequant_tflops", ctypes.c_double)]
 
 
 class ek_router_cfg(ctypes.Structure):

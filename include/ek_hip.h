@@ -365,13 +365,19 @@ ek_status ek_layer_get_forward_histogram(ek_layer *layer, ek_histogram *out);
 /* Ceilings measured on the device itself, for roofline lines next to the published peaks: a
  * plain device copy (bytes read + written per second), a read-only stream with non-temporal
  * loads (how the weight-streaming kernel reads expert weights) and a register-only bf16 MFMA
- * loop.  No counterpart in the reference (its ek-benchmark times whole calls only,
+ * loop, once on constant operands and once on operands with random signs, exponents and
+ * mantissas that change from one MFMA to the next (the clock under the chip's power limit, and
+ * with it the rate a matrix product of real data can reach, depends on the bits that toggle).
+ * No counterpart in the reference (its ek-benchmark times whole calls only,
  * ek-benchmark/src/bench.rs:36-52).  Allocates 8 GiB for the duration of the call; takes about a
  * second. */
 typedef struct ek_peaks {
     double copy_gbps;        /* GB/s, read + write */
     double read_nt_gbps;     /* GB/s */
-    double mfma_bf16_tflops; /* TFLOP/s, dense, fp32 accumulate */
+    double mfma_bf16_tflops; /* TFLOP/s, dense, fp32 accumulate, constant operands */
+    double mfma_bf16_random_tflops; /* the same loop on random operands */
+    double mfma_bf16_dequant_tflops; /* ... with the W8A16 tile path's conversions beside every MFMA
+                                        (5 vector instructions per MFMA, operands in registers) */
 } ek_peaks;
 ek_status ek_measure_peaks(int32_t device_id, ek_peaks *out);
 

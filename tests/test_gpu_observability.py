@@ -126,3 +126,17 @@ def test_phase_timing_every_call_and_sampled(ek, cuda):
         layer.profile(False)
         assert layer.stats()["profiled_calls"] == 0 and sum(layer.stats()["kernel_us"]) == 0
     layer.close()
+
+
+def test_measured_peaks_are_ordered_and_below_the_published_ones(ek, cuda):
+    """ek_measure_peaks: the device's own ceilings.  Each is below the published peak, the MFMA loop
+    slows down when its operands toggle and again when the int8 conversion runs beside it."""
+    import ctypes
+    from ek_hip import _capi as C
+    pk = C.ek_peaks()
+    C.check(C.load().ek_measure_peaks(0, ctypes.byref(pk)))
+    assert 2000.0 < pk.copy_gbps < 8000.0
+    assert 4000.0 < pk.read_nt_gbps < 8000.0
+    assert 1000.0 < pk.mfma_bf16_dequant_tflops < pk.mfma_bf16_random_tflops <= pk.mfma_bf16_tflops * 1.02
+    assert pk.mfma_bf16_tflops < 2500.0 * 1.02
+    assert C.load().ek_measure_peaks(0, None) == C.EK_INVALID_INPUT
