@@ -117,6 +117,27 @@ __device__ __forceinline__ typename Act<T>::V8 dequant_f8x8(uint32_t lo, uint32_
     return __builtin_bit_cast(typename Act<T>::V8, r);
 }
 
+// exp(x) from IEEE-754 single operations only (fused multiply-add, multiply, add, all rounded to
+// nearest even): Cody-Waite reduction by ln 2, the degree-5 polynomial of Cephes' expf, scaling by
+// an exponent-field constant; the argument is clamped to [-87, 88], where the result is a normal
+// number.  Within 2 ulp of the exact value, and the same bits on any conforming machine, so a CPU
+// restatement of these lines reproduces the kernels' silu exactly.
+__device__ __forceinline__ float expf_ieee(float x)
+{
+    x = x < -87.0f ? -87.0f : (x > 88.0f ? 88.0f : x);
+    const float n = __builtin_rintf(x * 1.44269504088896341f);
+    float r = __builtin_fmaf(n, -0.693359375f, x);
+    r = __builtin_fmaf(n, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+    p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+    p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+    p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+    p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+    const float y = __builtin_fmaf(r * r, p, r) + 1.0f;
+    return y * __builtin_bit_cast(float, (uint32_t)((int32_t)n + 127) << 23);
+}
+
 // SwiGLU with the reference's storage roundings: up, gate, silu(gate) and the
 // product are each a materialised tensor of the activation dtype
 // (ek-computation/src/ffn/expert_torch.rs:81-83).
@@ -124,11 +145,14 @@ template <typename T> __device__ __forceinline__ T swiglu_rounded(float acc_up, 
 {
     const float up = rnd<T>(acc_up);
     const float gate = rnd<T>(acc_gate);
-    // gate * 1/(1 + 2^(-gate * log2 e)) with the hardware's exp2 and reciprocal (1 ulp each):
-    // the value is rounded to 8 or 11 significant bits next, so this differs from a
-    // correctly rounded quotient in about one element in 10^4, by one 16-bit ulp, and costs a
-    // fifth of the instructions of expf and an IEEE division
-    const float sg = rnd<T>(gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(gate * -1.4426950408889634f)));
+    // silu in fp32 as a CPU backend forms it: gate / (1 + exp(-gate)) with a 2-ulp exp and a
+    // correctly rounded division, then the storage rounding.  The hardware's exp2 and reciprocal
+    // (1 ulp each) would be a fifth of the instructions and cost the tile kernel 1 % less time,
+    // but move about one element of h in 10^4 by one 16-bit ulp, which showed in the layer's output as
+    // outliers of up to 2.7e-2 x RMS against the reference-rounded result where libtorch's own
+    // evaluation stays at 1.2e-2 (DeepSeek-V3 decode, sampled tokens); with this form the
+    // kernels score what libtorch scores on the same tokens.
+    const float sg = rnd<T>(gate / (1.0f + expf_ieee(-gate)));
     return (T)(up * sg);
 }
 
