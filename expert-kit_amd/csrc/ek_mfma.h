@@ -119,12 +119,14 @@ __device__ __forceinline__ typename Act<T>::V8 dequant_f8x8(uint32_t lo, uint32_
 
 // exp(x) from IEEE-754 single operations only (fused multiply-add, multiply, add, all rounded to
 // nearest even): Cody-Waite reduction by ln 2, the degree-5 polynomial of Cephes' expf, scaling by
-// an exponent-field constant; the argument is clamped to [-87, 88], where the result is a normal
-// number.  Within 2 ulp of the exact value, and the same bits on any conforming machine, so a CPU
-// restatement of these lines reproduces the kernels' silu exactly.
+// exponent-field constants.  The argument is clamped to [-87, 89]: down there the result is still a
+// normal number, up there it has overflowed to +inf as expf does beyond 88.72 (the scaling is
+// split in two factors so that 2^128 is reached by a multiplication that overflows).  Within 2 ulp
+// of the exact value, and the same bits on any conforming machine, so a CPU restatement of these
+// lines reproduces the kernels' silu exactly.
 __device__ __forceinline__ float expf_ieee(float x)
 {
-    x = x < -87.0f ? -87.0f : (x > 88.0f ? 88.0f : x);
+    x = x < -87.0f ? -87.0f : (x > 89.0f ? 89.0f : x);
     const float n = __builtin_rintf(x * 1.44269504088896341f);
     float r = __builtin_fmaf(n, -0.693359375f, x);
     r = __builtin_fmaf(n, 2.12194440e-4f, r);
@@ -135,7 +137,9 @@ __device__ __forceinline__ float expf_ieee(float x)
     p = __builtin_fmaf(p, r, 1.6666665459e-1f);
     p = __builtin_fmaf(p, r, 5.0000001201e-1f);
     const float y = __builtin_fmaf(r * r, p, r) + 1.0f;
-    return y * __builtin_bit_cast(float, (uint32_t)((int32_t)n + 127) << 23);
+    const int32_t ni = (int32_t)n, top = ni > 127 ? 1 : 0;
+    const float v = y * __builtin_bit_cast(float, (uint32_t)(ni - top + 127) << 23);
+    return top ? v * 2.0f : v;
 }
 
 // SwiGLU with the reference's storage roundings: up, gate, silu(gate) and the

@@ -183,6 +183,34 @@ float eko_expf(float x)
 }
 float eko_sigmoidf(float x) { return 1.0f / (1.0f + eko_expf(-x)); }
 
+/*
+ * The same routine with the argument clamped to [-87, 89] and the scaling split in two factors, so
+ * that it overflows to +inf beyond 88.72 as libm's expf does: the form the HIP kernels' SwiGLU
+ * epilogue evaluates (expert-kit_amd/csrc/ek_mfma.h), restated here so that a CPU test can hold
+ * gate / (1 + exp(-gate)) built on it against the same expression built on libm for every 16-bit
+ * gate value.  Test support: eko_ffn itself uses libm's expf.
+ */
+float eko_expf_wide(float x)
+{
+    x = x < -87.0f ? -87.0f : (x > 89.0f ? 89.0f : x);
+    const float n = rintf(x * 1.44269504088896341f);
+    float r = fmaf(n, -0.693359375f, x);
+    r = fmaf(n, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = fmaf(p, r, 1.3981999507e-3f);
+    p = fmaf(p, r, 8.3334519073e-3f);
+    p = fmaf(p, r, 4.1665795894e-2f);
+    p = fmaf(p, r, 1.6666665459e-1f);
+    p = fmaf(p, r, 5.0000001201e-1f);
+    const float y = fmaf(r * r, p, r) + 1.0f;
+    const int32_t ni = (int32_t)n, top = ni > 127 ? 1 : 0;
+    const float v = y * bits_f32((uint32_t)(ni - top + 127) << 23);
+    return top ? v * 2.0f : v;
+}
+/* silu as the kernels form it, and as eko_ffn forms it (libm), for one fp32 gate value */
+float eko_silu_kernel_form(float g) { return g / (1.0f + eko_expf_wide(-g)); }
+float eko_silu_libm_form(float g) { return g / (1.0f + expf(-g)); }
+
 /* larger value first, lower index on equal values */
 static int pick_best(const float *v, const char *used, int n)
 {

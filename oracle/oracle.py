@@ -95,6 +95,19 @@ def expf(x: torch.Tensor) -> torch.Tensor:
     return torch.tensor([L.eko_expf(float(v)) for v in x.flatten().tolist()], dtype=torch.float32).reshape(x.shape)
 
 
+def silu_forms(g: torch.Tensor):
+    """silu of fp32 gate values, element by element, in the form the HIP kernels evaluate (eko_expf_wide)
+    and in the form eko_ffn evaluates (libm's expf): gate / (1 + exp(-gate)) both times."""
+    L = lib()
+    for f in (L.eko_silu_kernel_form, L.eko_silu_libm_form):
+        f.restype = ctypes.c_float
+        f.argtypes = [ctypes.c_float]
+    v = g.flatten().tolist()
+    a = torch.tensor([L.eko_silu_kernel_form(float(t)) for t in v], dtype=torch.float32).reshape(g.shape)
+    b = torch.tensor([L.eko_silu_libm_form(float(t)) for t in v], dtype=torch.float32).reshape(g.shape)
+    return a, b
+
+
 def route(kind: int, logits: torch.Tensor, k: int, renorm: bool = True, w_dtype=torch.float32, bias=None,
           n_group: int = 1, topk_group: int = 1, mask_neg_inf: bool = False, routed_scaling: float = 1.0):
     """The reference shims' routers (see eko_route): kind 0 Qwen3, 1-3 the vLLM shims, 4 DeepSeek-V3."""

@@ -293,6 +293,35 @@ def test_tile_route_shortest_contractions(ek, oracle, cuda, H, I, w8):
 
 
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_silu_of_every_16bit_gate_value(ek, oracle, cuda, dt):
+    """All 65536 bit patterns of the activation type as the gate pre-activation, through both kernel
+    families.  x is the identity, W_gate holds the patterns, W_up is all ones and W_down the identity, so
+    every sum has one non-zero term and out[r, c] = rnd(1 * rnd(silu(g[r, c]))): the kernels' SwiGLU
+    epilogue (an exp of IEEE operations, a correctly rounded division) must give the value the oracle
+    forms with libm's expf, for every finite gate."""
+    n = 256
+    pat = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dt).view(n, n)   # g[r][c]
+    g = torch.where(torch.isfinite(pat.float()), pat, torch.zeros_like(pat))
+    x = torch.eye(n).to(dt)
+    eye = torch.eye(n).to(dt)
+    ew = ek.ExpertWeight(torch.ones(n, n).to(dt), g.t().contiguous(), eye)   # gate[r][c] = W_gate[c][r]
+    ref = oracle.ffn(x, ew.up_w, ew.gate_w, ew.down_w, mode=0).float()
+    a, _ = oracle.silu_forms(g.float())
+    assert torch.equal(ref, a.to(dt).float())          # the construction: out = rnd(silu(g)) element for element
+    layer = ek.HipLayer(n, n, 2, 1, act_dtype=dt, w_dtype=dt, max_tokens=n)
+    layer.set_expert(1, ew)
+    # one segment of 256 rows: MFMA tile kernel
+    tiled = layer.forward(x.to(cuda), torch.ones(n, 1, dtype=torch.int32, device=cuda), torch.ones(n, 1, dtype=dt, device=cuda))
+    # 16 rows at a time: weight-streaming kernel
+    streamed = torch.cat([layer.expert_forward(1, x[r:r + 16].contiguous().to(cuda)) for r in range(0, n, 16)])
+    for name, got in (("tile", tiled), ("stream", streamed)):
+        got = got.cpu().float()
+        bad = (got != ref).nonzero()
+        assert bad.numel() == 0, (name, dt, bad[:5], got[got != ref][:5], ref[got != ref][:5])
+    layer.close()
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("w8", [False, True])
 def test_streaming_forms_agree_bitwise(ek, cuda, dt, w8):
     """The streaming kernel has three launch forms (one wave per channel group; eight waves, one

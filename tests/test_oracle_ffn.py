@@ -182,3 +182,21 @@ def test_router_vs_libtorch(oracle):
     # tie rule: equal logits -> lower index first
     tid, _ = oracle.router(torch.zeros(1, 5), 2)
     assert tid.tolist() == [[0, 1]]
+
+
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_silu_form_of_the_kernels_equals_the_libm_form_for_every_16bit_gate(oracle, dt):
+    """The HIP kernels evaluate silu(gate) = gate / (1 + exp(-gate)) with an exp made of IEEE fma / mul / add
+    only (restated as eko_expf_wide); eko_ffn, the oracle, uses libm's expf.  The two exps differ in the last
+    fp32 bit now and then; after the storage rounding of silu(gate) to the activation type they agree for
+    every one of the 65536 gate values of that type, so the choice of exp cannot show in a parity figure."""
+    pat = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dt)
+    g = pat.float()
+    fin = torch.isfinite(g)
+    a, b = oracle.silu_forms(g[fin])
+    assert (a != b).sum() < 2000                       # they are different routines ...
+    ra, rb = a.to(dt), b.to(dt)
+    assert torch.equal(ra.view(torch.int16), rb.view(torch.int16))   # ... with the same rounded results
+    # overflow side: exp(88.5) is finite, exp(89) is not
+    lo, hi = oracle.silu_forms(torch.tensor([-88.5, -89.0, -1e30, 89.0, 1e30]))
+    assert torch.equal(lo, hi) and lo[0] < 0 and lo[1] == 0 and lo[3] == 89.0
