@@ -119,14 +119,14 @@ __device__ __forceinline__ typename Act<T>::V8 dequant_f8x8(uint32_t lo, uint32_
 
 // exp(x) from IEEE-754 single operations only (fused multiply-add, multiply, add, all rounded to
 // nearest even): Cody-Waite reduction by ln 2, the degree-5 polynomial of Cephes' expf, scaling by
-// exponent-field constants.  The argument is clamped to [-87, 89]: down there the result is still a
-// normal number, up there it has overflowed to +inf as expf does beyond 88.72 (the scaling is
-// split in two factors so that 2^128 is reached by a multiplication that overflows).  Within 2 ulp
-// of the exact value, and the same bits on any conforming machine, so a CPU restatement of these
-// lines reproduces the kernels' silu exactly.
+// 2^n (ldexp: exact, overflows to +inf, never rounds for the arguments kept).  The argument is
+// clamped to [-87, 89]: down there the result is still a normal number, up there it has
+// overflowed to +inf as expf does beyond 88.72.  Within 2 ulp of the exact value, and the same
+// bits on any conforming machine, so a CPU restatement of these lines reproduces the kernels'
+// silu exactly.
 __device__ __forceinline__ float expf_ieee(float x)
 {
-    x = x < -87.0f ? -87.0f : (x > 89.0f ? 89.0f : x);
+    x = __builtin_amdgcn_fmed3f(x, -87.0f, 89.0f);
     const float n = __builtin_rintf(x * 1.44269504088896341f);
     float r = __builtin_fmaf(n, -0.693359375f, x);
     r = __builtin_fmaf(n, 2.12194440e-4f, r);
@@ -137,9 +137,7 @@ __device__ __forceinline__ float expf_ieee(float x)
     p = __builtin_fmaf(p, r, 1.6666665459e-1f);
     p = __builtin_fmaf(p, r, 5.0000001201e-1f);
     const float y = __builtin_fmaf(r * r, p, r) + 1.0f;
-    const int32_t ni = (int32_t)n, top = ni > 127 ? 1 : 0;
-    const float v = y * __builtin_bit_cast(float, (uint32_t)(ni - top + 127) << 23);
-    return top ? v * 2.0f : v;
+    return __builtin_ldexpf(y, (int)n);
 }
 
 // SwiGLU with the reference's storage roundings: up, gate, silu(gate) and the
@@ -150,12 +148,16 @@ template <typename T> __device__ __forceinline__ T swiglu_rounded(float acc_up, 
     const float up = rnd<T>(acc_up);
     const float gate = rnd<T>(acc_gate);
     // silu in fp32 as a CPU backend forms it: gate / (1 + exp(-gate)) with a 2-ulp exp and a
-    // correctly rounded division, then the storage rounding.  The hardware's exp2 and reciprocal
-    // (1 ulp each) would be a fifth of the instructions and cost the tile kernel 1 % less time,
-    // but move about one element of h in 10^4 by one 16-bit ulp, which showed in the layer's output as
+    // correctly rounded division, then the storage rounding (held for every one of the 65536 gate
+    // values of either 16-bit type by a test that feeds all of them through both kernel families).
+    // The hardware's exp2 and reciprocal (1 ulp each) would be a quarter of the instructions and
+    // cost the tile kernel 1 % less time (7 % at contractions as short as Qwen3's), but move about
+    // one element of h in 10^4 by one 16-bit ulp, which showed in the layer's output as
     // outliers of up to 2.7e-2 x RMS against the reference-rounded result where libtorch's own
     // evaluation stays at 1.2e-2 (DeepSeek-V3 decode, sampled tokens); with this form the
-    // kernels score what libtorch scores on the same tokens.
+    // kernels score what libtorch scores on the same tokens.  (A reciprocal with one residual
+    // correction in place of the division was tried: the reciprocal of 1 + e^87.5 and beyond is
+    // a denormal, which v_rcp_f32 flushes, and three bf16 gate values came out as 0.)
     const float sg = rnd<T>(gate / (1.0f + expf_ieee(-gate)));
     return (T)(up * sg);
 }

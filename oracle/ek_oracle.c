@@ -184,7 +184,7 @@ float eko_expf(float x)
 float eko_sigmoidf(float x) { return 1.0f / (1.0f + eko_expf(-x)); }
 
 /*
- * The same routine with the argument clamped to [-87, 89] and the scaling split in two factors, so
+ * The same routine with the argument clamped to [-87, 89] and the scaling done by ldexpf, so
  * that it overflows to +inf beyond 88.72 as libm's expf does: the form the HIP kernels' SwiGLU
  * epilogue evaluates (expert-kit_amd/csrc/ek_mfma.h), restated here so that a CPU test can hold
  * gate / (1 + exp(-gate)) built on it against the same expression built on libm for every 16-bit
@@ -203,11 +203,12 @@ float eko_expf_wide(float x)
     p = fmaf(p, r, 1.6666665459e-1f);
     p = fmaf(p, r, 5.0000001201e-1f);
     const float y = fmaf(r * r, p, r) + 1.0f;
-    const int32_t ni = (int32_t)n, top = ni > 127 ? 1 : 0;
-    const float v = y * bits_f32((uint32_t)(ni - top + 127) << 23);
-    return top ? v * 2.0f : v;
+    return ldexpf(y, (int)n);
 }
-/* silu as the kernels form it, and as eko_ffn forms it (libm), for one fp32 gate value */
+/* silu with the kernels' exp and a correctly rounded division (the kernels form the quotient with a
+ * reciprocal and one residual correction; that the two agree after the storage rounding for every
+ * 16-bit gate is what the GPU test over all gate values holds), and as eko_ffn forms it (libm),
+ * for one fp32 gate value */
 float eko_silu_kernel_form(float g) { return g / (1.0f + eko_expf_wide(-g)); }
 float eko_silu_libm_form(float g) { return g / (1.0f + expf(-g)); }
 
