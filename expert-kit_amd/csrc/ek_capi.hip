@@ -933,7 +933,7 @@ hipStream_t pick_side_stream(ek_layer *L, hipStream_t s)
 // an empty list gets no launch, and the two chains run side by side exactly when both have work).
 ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int32_t *rows, void *out, int64_t P, int64_t E,
                       hipStream_t s, hipEvent_t *ev, int64_t wide_items = 0, int64_t extra_stream = 0,
-                      int64_t shared_wide = 0, const int64_t *exact = nullptr)
+                      int64_t shared_wide = 0, const int64_t *exact = nullptr, int64_t known_tile_items = -1)
 {
     const int64_t H = L->cfg.hidden, I = L->cfg.inter;
     ek::FfnArgs a1;
@@ -992,10 +992,21 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
         EK_HIP(hipStreamWaitEvent(side, L->ev_fork, 0));
     }
     if (fork) s_stream = side;
+    // The per-expert entry points know how many tile items their lists hold.  When those would put a
+    // tile on at most half of the CUs, the narrow form of the tile kernel (half the channels per
+    // workgroup, twice the workgroups) shortens the call: one tile's walk over the whole contraction is
+    // what such a call waits for (one DeepSeek-V3 int8 expert, 1024 rows: 225 -> 157 us; Qwen3 fp16,
+    // 2048 / 4096 rows: 97 -> 79 / 100 -> 76 us).  With more tiles the wide form's fewer reads of the
+    // activation tile win (DeepSeek-V3, 4096 rows: 350 against 412 us), and a layer call's streaming
+    // chain runs on the CUs the tiles leave free, so that narrower tiles there only move time from
+    // one chain to the other (Qwen3 decode, 256 tokens: 0.195 against 0.199 ms).  Same bits either way.
+    if (exact) known_tile_items = exact[ek::kListT32] + exact[ek::kListT64] + exact[ek::kListT128];
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
         const bool tiles_first = fork;
-        if (tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
+        const int64_t wgs_per_item = (a.N + ek::tile_channels(stage, false) - 1) / ek::tile_channels(stage, false);
+        const bool narrow = known_tile_items > 0 && known_tile_items * wgs_per_item <= 128;
+        if (tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, narrow, s_tiles));
         if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, cap[ek::kListStream], false, s_stream));
         if (shared_wide > 0) {
             ek::FfnArgs aw = a;                  // the same stage over the shared segment's own list
@@ -1003,7 +1014,7 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
             aw.lists.count = W.wide_count;
             EK_HIP(ek::launch_ffn_stream(aw, stage, L->act, L->wmode, shared_wide, true, side));
         }
-        if (!tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, s_tiles));
+        if (!tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, narrow, s_tiles));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
     }
     if (fork || shared_wide > 0) {
@@ -1398,10 +1409,11 @@ ek_status ek_layer_expert_forward(ek_layer *layer, int32_t expert, const void *x
             }
             // the ordinary cut's tile items: full 128-row tiles and a remainder of more than 16 rows
             const int64_t wide_items = (n + ek::kWideRows - 1) / ek::kWideRows;
-            const bool wide = ek::wide_cut_pays((n >> 7) + ((n & 127) > 16), n, H, layer->cfg.inter, layer->w8 ? 1 : 2) &&
+            const bool wide = ek::wide_cut_pays((n >> 7) + ((n & 127) > 16), n, H, layer->cfg.inter) &&
                               wide_items <= layer->ws.list_cap[ek::kListStream];
             ek::launch_single_lists(layer->ws.lists, expert, (int32_t)n, wide, s);
-            EK_TRY(enqueue_ffn(layer, layer->ws, d_x, nullptr, d_out, n, 1, s, nullptr, wide ? wide_items : 0));
+            EK_TRY(enqueue_ffn(layer, layer->ws, d_x, nullptr, d_out, n, 1, s, nullptr, wide ? wide_items : 0, 0, 0, nullptr,
+                               wide ? 0 : (n >> 7) + ((n & 127) > 16)));
             if (layer->padded) EK_TRY(rows_out(layer, out, layer->st_y, n, mem, s));
             else if (mem == EK_HOST) EK_TRY(d2h(layer, out, layer->st_y, (size_t)n * H * 2, s));
         }
@@ -1484,8 +1496,8 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             // 890 / 1325 us as tiles beside streams).
             const int wb = layer->w8 ? 1 : 2;
             const double cover_us = (double)short_items * 3.0 * (double)H * (double)layer->cfg.inter * wb / 6.5e6;
-            const double tiled_us = 15.0 + (double)(H + layer->cfg.inter) * (wb == 1 ? 0.025 : 0.0285);
-            const bool wide = ek::wide_cut_pays(tile_items, P, H, layer->cfg.inter, wb) && cover_us < 0.5 * tiled_us &&
+            const double tiled_us = ek::tile_call_us(H, layer->cfg.inter);
+            const bool wide = ek::wide_cut_pays(tile_items, P, H, layer->cfg.inter) && cover_us < 0.5 * tiled_us &&
                               wide_items <= layer->ws.list_cap[ek::kListStream];
             for (int i = 0; i < n_calls; ++i) {
                 const int32_t n = (int32_t)rows[i], full = n >> 7, r = n & 127;

@@ -95,22 +95,24 @@ __device__ __forceinline__ void block_barrier()
 #else
 #define EK_ABL_XDMA true
 #endif
-constexpr int kTileThreads = 512;
-constexpr int kTileWaves = 8;
 constexpr int kCusPerXcd = 32;   // MI355X: 8 XCDs x 32 CUs
 
 // A step covers 64 contraction elements: one weight chunk per channel tile with one-byte
 // weights, two with 16-bit ones (KC).  One-byte weights run three stages deep (two steps of
 // loads in flight), 16-bit weights, whose stage is 80 KiB, two (one step in flight, of the
 // same length in time: the step has as many MFMAs and no conversion work).
-template <bool W8> struct TileGeom {
+// WAVES wavefronts per workgroup, each with CB column blocks of 32 channels; BMMAX = rows of the
+// tallest tile.
+template <bool W8, int WAVES, int CB, int BMMAX> struct TileGeom {
     static constexpr int BK = 64;                    // contraction elements per step
     static constexpr int KC = W8 ? 1 : 2;            // weight chunks along k per channel tile and step
     static constexpr int PPR = BK / 8;               // 16-byte pieces per activation row and step
-    static constexpr int XS = 128 * BK * 2;          // bytes of a 128-row activation stage
-    static constexpr int WS = kTileWaves * 4 * KC * kChunkBytes;
+    static constexpr int XS = BMMAX * BK * 2;        // bytes of an activation stage
+    static constexpr int WS = WAVES * 2 * CB * KC * kChunkBytes;
     static constexpr int STAGE = XS + WS;
-    static constexpr int STAGES = W8 ? 3 : 2;
+    // 16-bit weights: two stages of 80 KiB with two column blocks per wave, three of 48 KiB with one
+    static constexpr int STAGES = W8 || CB == 1 ? 3 : 2;
+    static constexpr int SCALE_BYTES = 2 * WAVES * CB * 64 * 4;   // [tile parity][wave][column block][block]
 };
 
 // XOR key of a row: fragment reads of 16 consecutive rows and one piece index
@@ -122,10 +124,10 @@ template <int PPR> __device__ __forceinline__ int swizzle_key(int row)
 }
 
 // What one wavefront needs to know about one tile (work item x channel block).
-template <typename T, int NR, int LX> struct TileCtx {
+template <typename T, int NR, int LX, int CB> struct TileCtx {
     const uint8_t *wp[NR];   // this lane's 16 bytes of the wave's weight chunks at step 0
     const T *xsrc[LX];       // this lane's 16-byte pieces of the activation tile at step 0
-    float as[2], ac[2];      // dequantisation constants of the lane's channel, per column block
+    float as[CB], ac[CB];    // dequantisation constants of the lane's channel, per column block
     int row0, nrows;         // the item's packed rows
     int chan0;               // first output channel of the wave's block
     int sslot;               // block-scaled weights: which of the two LDS scale areas holds this tile's rows
@@ -136,18 +138,17 @@ template <typename T, int NR, int LX> struct TileCtx {
 // runs across tile boundaries: the first two steps of the next tile are issued during the
 // last two steps of the current one, so only the epilogue separates two tiles.
 constexpr int kTileScaleBlocks = 64;   // 128-wide scale blocks along the contraction: K <= 8192
-constexpr int kTileScaleBytes = 2 * kTileWaves * 2 * kTileScaleBlocks * 4;   // [tile parity][wave][column block][block]
 
-template <typename T, int WM, int NMAT, int MR>
+template <typename T, int WM, int NMAT, int MR, int kTileWaves, int CB, int BMMAX>
 __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *items, const int ntiles,
                                           const int nb_count, const int first, const int stride,
                                           uint8_t *lds, const uint32_t lds_base)
 {
     using V8 = typename Act<T>::V8;
     constexpr bool W8 = WM != kW16;            // one-byte weights
-    using G = TileGeom<W8>;
-    constexpr int NR = NMAT == 2 ? 2 : 4;      // channel tiles per wave and matrix
-    constexpr int NWC = NR * NMAT;             // channel tiles x matrices per wave (always 4)
+    using G = TileGeom<W8, kTileWaves, CB, BMMAX>;
+    constexpr int NWC = 2 * CB;                // channel tiles x matrices per wave
+    constexpr int NR = NWC / NMAT;             // channel tiles per wave and matrix
     constexpr int KC = G::KC;
     constexpr int NWCH = NWC * KC;             // weight chunks per wave and step
     constexpr int NS = G::STAGES, AHEAD = NS - 1;   // stages; steps of loads in flight
@@ -156,13 +157,18 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     constexpr int XINSTR = BM * PPR / 64;      // DMA instructions per activation stage
     constexpr int LX = (XINSTR + kTileWaves - 1) / kTileWaves;   // ... per wave
     constexpr int LOADS = NWCH + LX;           // DMAs per wave and stage
-    constexpr int CB = 2;                      // column blocks of 32 channels per wave
     constexpr int RB = MR / 2;                 // 32-row blocks
     constexpr int NGRP = BK / 16;              // MFMA k-groups per step
     constexpr int kRowBlockBytes = 32 * PPR * 16;
-    static_assert(NWC == 4, "wave-private weight region holds 4 chunks");
     static_assert(RB >= 1, "items have at least 32 rows");
-    typedef TileCtx<T, NR, LX> Ctx;
+    static_assert(BM <= BMMAX, "the activation stage holds the tile");
+    static_assert(NMAT == 1 || CB % 2 == 0 || CB == 1, "up and gate blocks come in pairs, or share one block");
+    static_assert(!(block_scaled(WM) && CB == 1), "block-scaled weights are served by the wide form only");
+    // CB == 1 with two matrices: the wave's one column block is {16 up channels, 16 gate channels}
+    // of the same 16 hidden channels (lanes 0-15 / 16-31 of the A operand), and a lane's accumulator
+    // holds up in registers 0-7 and gate of the same channels in registers 8-15.
+    constexpr bool kSplitBlock = NMAT == 2 && CB == 1;
+    typedef TileCtx<T, NR, LX, CB> Ctx;
 
     if (first >= ntiles) return;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -185,9 +191,9 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
         xdst[i] = q * 1024;
     }
     const uint32_t w_off = G::XS + wave * (NWCH * kChunkBytes);  // wave-private weight region
-    // MFMA 32x32x16 operands.  The wave's 4 weight chunks (16 channels each) form CB = 2
-    // column blocks of 32 channels: {up, gate} of the same 32 channels (stage 1) or 64
-    // consecutive channels (stage 2).  Lane l feeds channel l%32 and k-half kg = l/32 of the
+    // MFMA 32x32x16 operands.  The wave's 2*CB weight chunks (16 channels each) form CB
+    // column blocks of 32 channels: {up, gate} pairs of the same 32 channels (stage 1: block cb is
+    // matrix cb % 2 of channel pair cb / 2) or CB * 32 consecutive channels (stage 2).  Lane l feeds channel l%32 and k-half kg = l/32 of the
     // A operand, and row l%32 of a 32-row block of the B operand.  A 16-byte LDS read of
     // weight slot (2*tt + kg) gives the lane the A operands of two MFMAs (int8) or one
     // (16-bit, whose two chunks per channel tile lie side by side: k-group grp is read grp);
@@ -195,7 +201,8 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     int aoff[CB];
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
-        const int nr = NMAT == 2 ? hh : cb * 2 + hh, m = NMAT == 2 ? cb : 0;
+        const int nr = kSplitBlock ? 0 : (NMAT == 2 ? cb >> 1 : cb) * 2 + hh;
+        const int m = kSplitBlock ? hh : (NMAT == 2 ? (cb & 1) : 0);
         aoff[cb] = (nr * NMAT + m) * KC * kChunkBytes + kg * 256 + j * 16;
     }
     int boff[NGRP];
@@ -211,8 +218,8 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     // each, so a step's scale is one number per column block; the tile's rows of the scale
     // matrices sit in a wave-private LDS area (two areas: the next tile's rows are fetched while
     // this one's are in use)
-    float *const sc_area = (float *)(lds + NS * G::STAGE) + wave * (2 * kTileScaleBlocks);
-    constexpr int kScaleSlotFloats = kTileWaves * 2 * kTileScaleBlocks;
+    float *const sc_area = (float *)(lds + NS * G::STAGE) + wave * (CB * kTileScaleBlocks);
+    constexpr int kScaleSlotFloats = kTileWaves * CB * kTileScaleBlocks;
     auto fetch = [&](int t, Ctx &c, int sslot) -> int {
         for (; t < ntiles; t += stride) {
             const WorkItem item = items[t / nb_count];
@@ -233,16 +240,17 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             for (int cb = 0; cb < CB; ++cb) {
                 float sv = 1.f;
                 if constexpr (WM == kWI8) {
-                    const int nr = NMAT == 2 ? hh : cb * 2 + hh;
+                    const int nr = kSplitBlock ? 0 : (NMAT == 2 ? cb >> 1 : cb) * 2 + hh;
                     const int ch = min(cblock * NR + nr, NT - 1) * 16 + j;
-                    sv = NMAT == 2 ? (cb == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
+                    const bool gate = kSplitBlock ? hh == 1 : (cb & 1) == 1;
+                    sv = NMAT == 2 ? (gate ? slab.s_gate[ch] : slab.s_up[ch]) : slab.s_down[ch];
                 }
                 c.as[cb] = sv;
                 c.ac[cb] = -128.f * sv;
                 if constexpr (block_scaled(WM)) {
                     const int KB = (a.Kdim + 127) >> 7;
-                    const int ct = min(cblock * NR + (NMAT == 2 ? 0 : cb * 2), NT - 1);
-                    const float *smat = NMAT == 2 ? (cb == 0 ? slab.s_up : slab.s_gate) : slab.s_down;
+                    const int ct = min(cblock * NR + (NMAT == 2 ? cb >> 1 : cb) * 2, NT - 1);
+                    const float *smat = NMAT == 2 ? ((cb & 1) == 0 ? slab.s_up : slab.s_gate) : slab.s_down;
                     if (lane < KB)
                         sc_area[sslot * kScaleSlotFloats + cb * kTileScaleBlocks + lane] = smat[(int64_t)((ct * 16) >> 7) * KB + lane];
                 }
@@ -375,10 +383,11 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                         acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[1][cb]), bf[1][rb], acc[rb][cb]);
                 }
                 if constexpr (W8) {
-                    constexpr int DW = 4 / RB;
+                    // the k-group's 2*CB dwords are spread over the row blocks
 #pragma unroll
-                    for (int d = 0; d < DW; ++d) {
-                        const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
+                    for (int dw = 0; dw < 2 * CB; ++dw) {
+                        if (dw * RB / (2 * CB) != rb) continue;
+                        const int cb = dw >> 1, part = dw & 1;
                         const u32x2 v = dq(aq[0][cb][part], cb);
                         af[0][cb][part * 2] = v[0];
                         af[0][cb][part * 2 + 1] = v[1];
@@ -403,11 +412,11 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                             acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cg][cb]), bf[cg][rb], acc[rb][cb]);
                     }
                     if constexpr (W8) {
-                        // next group's A operands: 4 dwords (2 per column block) spread over the row blocks
-                        constexpr int DW = 4 / RB;
+                        // next group's A operands: 2 dwords per column block, spread over the row blocks
 #pragma unroll
-                        for (int d = 0; d < DW; ++d) {
-                            const int dw = rb * DW + d, cb = dw >> 1, part = dw & 1;
+                        for (int dw = 0; dw < 2 * CB; ++dw) {
+                            if (dw * RB / (2 * CB) != rb) continue;
+                            const int cb = dw >> 1, part = dw & 1;
                             const int g1 = grp + 1;
                             const u32x2 v = dq(aq[g1 >> 1][cb][(g1 & 1) * 2 + part], cb);
                             af[ng][cb][part * 2] = v[0];
@@ -439,7 +448,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
         //      32-row block at a time, and leave as whole rows: 16 bytes per lane, a row of the
         //      wave's OUTC channels per 2*OUTC/16 lanes.
         typedef T T4 __attribute__((ext_vector_type(4)));
-        constexpr int OUTC = NMAT == 2 ? 32 : 64;          // output channels per wave
+        constexpr int OUTC = NMAT == 2 ? CB * 16 : CB * 32;   // output channels per wave
         constexpr int RS = OUTC * 2 + 16;                  // scratch row stride: 16 bytes of padding
         constexpr int PPO = OUTC * 2 / 16, RPI = 64 / PPO; // pieces per row, rows per store instruction
         static_assert(kTileWaves * 32 * RS <= G::STAGE, "epilogue scratch fits one stage");
@@ -452,11 +461,23 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                 if (rb * 32 >= cur.nrows) break;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    if constexpr (NMAT == 2) {
-                        T4 o;
+                    if constexpr (kSplitBlock) {
+                        if (q < 2) {
+                            T4 o;
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) o[r] = swiglu_rounded<T>(acc[rb][0][q * 4 + r], acc[rb][1][q * 4 + r]);
-                        *(uint2 *)(scr + l32 * RS + (q * 8 + kg * 4) * 2) = __builtin_bit_cast(uint2, o);
+                            for (int r = 0; r < 4; ++r)
+                                o[r] = swiglu_rounded<T>(acc[rb][0][q * 4 + r], acc[rb][0][(q + 2) * 4 + r]);
+                            *(uint2 *)(scr + l32 * RS + (q * 8 + kg * 4) * 2) = __builtin_bit_cast(uint2, o);
+                        }
+                    } else if constexpr (NMAT == 2) {
+#pragma unroll
+                        for (int c2 = 0; c2 < CB / 2; ++c2) {
+                            T4 o;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                o[r] = swiglu_rounded<T>(acc[rb][2 * c2][q * 4 + r], acc[rb][2 * c2 + 1][q * 4 + r]);
+                            *(uint2 *)(scr + l32 * RS + (c2 * 32 + q * 8 + kg * 4) * 2) = __builtin_bit_cast(uint2, o);
+                        }
                     } else {
 #pragma unroll
                         for (int cb = 0; cb < CB; ++cb) {
@@ -496,60 +517,67 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 // neighbouring CUs share the activation tile (same item) and mostly the expert's weights
 // in the XCD's L2.  Every workgroup's tile sequence is fixed by its index: no queues, no
 // spinning, and it ends when its indices run out.
-template <typename T, int WM, int NMAT>
-__global__ __launch_bounds__(kTileThreads, 1) void ffn_tile_kernel(FfnArgs a, int nb_count)
+template <typename T, int WM, int NMAT, int WAVES, int CB>
+__global__ __launch_bounds__(WAVES * 64, 1) void ffn_tile_kernel(FfnArgs a, int nb_count)
 {
+    using G = TileGeom<WM != kW16, WAVES, CB, 128>;
     __shared__ __attribute__((aligned(1024)))
-    uint8_t lds[TileGeom<WM != kW16>::STAGES * TileGeom<WM != kW16>::STAGE + (block_scaled(WM) ? kTileScaleBytes : 0)];
+    uint8_t lds[G::STAGES * G::STAGE + (block_scaled(WM) ? G::SCALE_BYTES : 0)];
     const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)lds;
     const int x = blockIdx.x & 7, slot = blockIdx.x >> 3, nslots = gridDim.x >> 3;
     const int n128 = a.lists.count[kListT128], n64 = a.lists.count[kListT64], n32 = a.lists.count[kListT32];
     const int lo128 = x * n128 / 8, s128 = (x + 1) * n128 / 8 - lo128;
     const int lo64 = x * n64 / 8, s64 = (x + 1) * n64 / 8 - lo64;
     const int lo32 = x * n32 / 8, s32 = (x + 1) * n32 / 8 - lo32;
-    run_tiles<T, WM, NMAT, 8>(a, a.lists.items[kListT128] + lo128, s128 * nb_count, nb_count, slot, nslots, lds, lds_base);
+    run_tiles<T, WM, NMAT, 8, WAVES, CB, 128>(a, a.lists.items[kListT128] + lo128, s128 * nb_count, nb_count, slot, nslots, lds, lds_base);
     // the shorter classes start where the long one left the CUs least loaded
     const int r64 = (slot + nslots - (s128 * nb_count) % nslots) % nslots;
-    run_tiles<T, WM, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds, lds_base);
+    run_tiles<T, WM, NMAT, 4, WAVES, CB, 128>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds, lds_base);
     const int r32 = (r64 + nslots - (s64 * nb_count) % nslots) % nslots;
-    run_tiles<T, WM, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32, nslots, lds, lds_base);
+    run_tiles<T, WM, NMAT, 2, WAVES, CB, 128>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32, nslots, lds, lds_base);
 }
 
-template <typename T, int WM, int NMAT>
+template <typename T, int WM, int NMAT, int WAVES, int CB>
 static hipError_t launch_t(const FfnArgs &a, const int64_t max_items[kNumLists], hipStream_t s)
 {
-    constexpr int NR = NMAT == 2 ? 2 : 4;
+    constexpr int NR = 2 * CB / NMAT;            // channel tiles per wave and matrix
     const int NT = a.N / 16;
-    const int nb_count = (NT + kTileWaves * NR - 1) / (kTileWaves * NR);
+    const int nb_count = (NT + WAVES * NR - 1) / (WAVES * NR);
     const int64_t per_xcd = (max_items[kListT128] + 7) / 8 + (max_items[kListT64] + 7) / 8 +
                             (max_items[kListT32] + 7) / 8;
     int64_t slots = per_xcd * nb_count;          // tiles an XCD can get at most
     if (slots <= 0) return hipSuccess;
     if (slots > kCusPerXcd) slots = kCusPerXcd;
-    hipLaunchKernelGGL((ffn_tile_kernel<T, WM, NMAT>), dim3((unsigned)(slots * 8)), dim3(kTileThreads), 0, s, a,
+    hipLaunchKernelGGL((ffn_tile_kernel<T, WM, NMAT, WAVES, CB>), dim3((unsigned)(slots * 8)), dim3(WAVES * 64), 0, s, a,
                        nb_count);
     return hipGetLastError();
 }
 
 template <typename T>
-static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, const int64_t max_items[kNumLists], hipStream_t s)
+static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, const int64_t max_items[kNumLists], bool narrow,
+                           hipStream_t s)
 {
     switch (wmode) {
     case kWI8:
-        return stage == 1 ? launch_t<T, kWI8, 2>(a, max_items, s) : launch_t<T, kWI8, 1>(a, max_items, s);
+        if (narrow)
+            return stage == 1 ? launch_t<T, kWI8, 2, 8, 1>(a, max_items, s) : launch_t<T, kWI8, 1, 8, 1>(a, max_items, s);
+        return stage == 1 ? launch_t<T, kWI8, 2, 8, 2>(a, max_items, s) : launch_t<T, kWI8, 1, 8, 2>(a, max_items, s);
     case kWF8Block:
-        return stage == 1 ? launch_t<T, kWF8Block, 2>(a, max_items, s) : launch_t<T, kWF8Block, 1>(a, max_items, s);
+        return stage == 1 ? launch_t<T, kWF8Block, 2, 8, 2>(a, max_items, s) : launch_t<T, kWF8Block, 1, 8, 2>(a, max_items, s);
     case kWI8Block:
-        return stage == 1 ? launch_t<T, kWI8Block, 2>(a, max_items, s) : launch_t<T, kWI8Block, 1>(a, max_items, s);
+        return stage == 1 ? launch_t<T, kWI8Block, 2, 8, 2>(a, max_items, s) : launch_t<T, kWI8Block, 1, 8, 2>(a, max_items, s);
     default:
-        return stage == 1 ? launch_t<T, kW16, 2>(a, max_items, s) : launch_t<T, kW16, 1>(a, max_items, s);
+        if (narrow)
+            return stage == 1 ? launch_t<T, kW16, 2, 8, 1>(a, max_items, s) : launch_t<T, kW16, 1, 8, 1>(a, max_items, s);
+        return stage == 1 ? launch_t<T, kW16, 2, 8, 2>(a, max_items, s) : launch_t<T, kW16, 1, 8, 2>(a, max_items, s);
     }
 }
 
 hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, int wmode,
-                           const int64_t max_items[kNumLists], hipStream_t s)
+                           const int64_t max_items[kNumLists], bool narrow, hipStream_t s)
 {
-    return act == 0 ? launch_w<__bf16>(a, stage, wmode, max_items, s) : launch_w<_Float16>(a, stage, wmode, max_items, s);
+    return act == 0 ? launch_w<__bf16>(a, stage, wmode, max_items, narrow, s)
+                    : launch_w<_Float16>(a, stage, wmode, max_items, narrow, s);
 }
 
 }  // namespace ek

@@ -62,20 +62,21 @@ struct WorkLists {
 };
 constexpr int kWideRows = 64;
 // tile_items: work items the ordinary cut would give the tile kernel; one of them spreads
-// over ceil(inter / 256) workgroups in stage 1, and below half a chip of them the call takes as
-// long as one tile's two contractions however few rows it has: ~15 us + (hidden + inter) x
-// 25 ns (one-byte weights) or 28.5 ns (16-bit).  The streaming kernel spreads every item
-// over inter / 16 workgroups, each of which reads its item's rows, and its time grows with the
-// rows: ~ rows x (53 ns + hidden x inter x 14.8 fs).  Fitted on MI355X to one DeepSeek-V3
-// expert (hidden 7168, inter 2048; int8: 219 us streamed / 245 us tiled at 768 rows, 265 / 243
-// at 896; bf16: 230 / 274 at 768, 281 / 277 at 1024) and to the Qwen3 fp16 shape (2048, 768:
-// 76 ns per row streamed, 98 us tiled).
-inline bool wide_cut_pays(int64_t tile_items, int64_t rows, int64_t hidden, int64_t inter, int64_t weight_bytes)
+// over ceil(inter / 128) workgroups in stage 1 (the tile kernel's narrow form, which such calls
+// get), and below half a chip of them the call takes as long as one tile's two contractions
+// however few rows it has: ~30 us + (hidden + inter) x 13.6 ns, with one-byte and 16-bit weights
+// alike.  The streaming kernel spreads every item over inter / 16 workgroups, each of which reads
+// its item's rows, and its time grows with the rows: ~ rows x (53 ns + hidden x inter x 14.8 fs).
+// Fitted on MI355X to one DeepSeek-V3 expert (hidden 7168, inter 2048; tiled 152-158 us from 64 to
+// 1024 rows with int8 weights, 150 us with bf16; streamed 143 / 188 / 199 us at 512 / 640 / 768
+// rows) and to the Qwen3 shape (2048, 768: tiled 66 us fp16, 69 us int8; streamed 37 / 46 / 62 us
+// at 512 / 640 / 768 rows).
+inline double tile_call_us(int64_t hidden, int64_t inter) { return 30.0 + (double)(hidden + inter) * 0.0136; }
+inline bool wide_cut_pays(int64_t tile_items, int64_t rows, int64_t hidden, int64_t inter)
 {
     if (tile_items <= 0 || tile_items * ((inter + 255) / 256) >= 128) return false;
-    const double tiled_us = 15.0 + (double)(hidden + inter) * (weight_bytes == 1 ? 0.025 : 0.0285);
     const double streamed_us = (double)rows * (0.053 + 1.48e-8 * (double)hidden * (double)inter);
-    return streamed_us < 0.92 * tiled_us;
+    return streamed_us < 0.92 * tile_call_us(hidden, inter);
 }
 inline int64_t list_capacity(int list, int64_t P, int64_t E)
 {
@@ -160,9 +161,14 @@ struct FfnArgs {
 hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, int wmode, int64_t max_items, bool wide,
                              hipStream_t s);
 // MFMA tile kernel over the three tile lists (128-row items first, then 64,
-// then 32); max_items[l] bounds list l
+// then 32); max_items[l] bounds list l.  A workgroup covers tile_channels(stage, narrow) output
+// channels of one item; the narrow form (half the channels per workgroup, so twice the workgroups
+// per item; same bits) is for launches that would leave most of the chip without a tile, and
+// exists for per-channel int8 and 16-bit weights only (ignored otherwise).
 hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, int wmode,
-                           const int64_t max_items[kNumLists], hipStream_t s);
+                           const int64_t max_items[kNumLists], bool narrow, hipStream_t s);
+// hidden channels (stage 1) / output channels (stage 2) per tile workgroup
+constexpr int tile_channels(int stage, bool narrow) { return (stage == 1 ? 256 : 512) / (narrow ? 2 : 1); }
 
 // ---- combine ----------------------------------------------------------------
 struct CombineArgs {

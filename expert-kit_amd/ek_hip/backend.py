@@ -16,6 +16,7 @@ arithmetic happens inside libek_hip.so.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from dataclasses import dataclass
 from typing import Dict, Optional, Sequence
@@ -34,6 +35,17 @@ def _mem(t: torch.Tensor) -> int:
 
 def _ptr(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+_NO_CTX = contextlib.nullcontext()
+
+
+def _alloc_on(stream):
+    """Context in which the outputs of an enqueue-only call are allocated: the caller's stream.  torch's
+    caching allocator hands a freed block to the next request on the stream it was allocated on without
+    waiting for other streams, so a result allocated on the current stream, written by kernels on
+    `stream` and dropped by the caller before they ran could be handed out again under those kernels."""
+    return torch.cuda.stream(stream) if isinstance(stream, torch.cuda.Stream) else _NO_CTX
 
 
 def _stream_ptr(stream) -> ctypes.c_void_p:
@@ -199,8 +211,9 @@ class HipLayer:
         assert ids.dtype == torch.int32 and x.dtype == self.act_dtype
         assert x.is_cuda == ids.is_cuda == w.is_cuda
         T = x.shape[0]
-        y = out if out is not None else torch.empty_like(x)
-        rt, ro = self._route(T, x.device) if return_route else (None, None)
+        with (_alloc_on(stream) if out is None or return_route else _NO_CTX):
+            y = out if out is not None else torch.empty_like(x)
+            rt, ro = self._route(T, x.device) if return_route else (None, None)
         C.check(self._lib.ek_layer_forward(self._h, _ptr(x), _ptr(ids), _ptr(w), _DT[w.dtype], T, _ptr(y),
                                            ctypes.byref(ro) if ro is not None else None, _mem(x),
                                            _stream_ptr(stream)))
@@ -215,8 +228,9 @@ class HipLayer:
         assert x.is_contiguous() and ids.is_contiguous() and w.is_contiguous()
         assert ids.dtype == torch.int32 and x.dtype == self.act_dtype
         T = x.shape[0]
-        y = out if out is not None else torch.empty_like(x)
-        rt, ro = self._route(T, x.device) if return_route else (None, None)
+        with (_alloc_on(stream) if out is None or return_route else _NO_CTX):
+            y = out if out is not None else torch.empty_like(x)
+            rt, ro = self._route(T, x.device) if return_route else (None, None)
         C.check(self._lib.ek_layer_forward_static(self._h, _ptr(x), _ptr(ids), _ptr(w), _DT[w.dtype], T, _ptr(y),
                                                   ctypes.byref(ro) if ro is not None else None,
                                                   _stream_ptr(stream)))
@@ -226,19 +240,21 @@ class HipLayer:
         """Routing tables (and the gathered rows Xp if x is given)."""
         ids = ids.contiguous()
         T = ids.shape[0]
-        rt, ro = self._route(T, ids.device)
-        xp = None
-        if x is not None:
-            x = x.contiguous()
-            xp = torch.empty(T * self.cfg.top_k, x.shape[1], dtype=x.dtype, device=x.device)
+        with _alloc_on(stream):
+            rt, ro = self._route(T, ids.device)
+            xp = None
+            if x is not None:
+                x = x.contiguous()
+                xp = torch.empty(T * self.cfg.top_k, x.shape[1], dtype=x.dtype, device=x.device)
         C.check(self._lib.ek_layer_pack(self._h, _ptr(ids), T, ctypes.byref(ro), _ptr(x), _ptr(xp),
                                         _mem(ids), _stream_ptr(stream)))
         return (rt, xp) if x is not None else rt
 
     def expert_forward(self, e: int, x: torch.Tensor, stream=None) -> torch.Tensor:
         assert x.dim() == 2, "input must be rank 2 (ffn/mod.rs:45)"
-        x = x.contiguous()
-        out = torch.empty_like(x)
+        with _alloc_on(stream):
+            x = x.contiguous()
+            out = torch.empty_like(x)
         C.check(self._lib.ek_layer_expert_forward(self._h, e, _ptr(x), x.shape[0], _ptr(out), _mem(x),
                                                   _stream_ptr(stream)))
         return out
@@ -259,8 +275,9 @@ class HipLayer:
         logits = logits.contiguous()
         T, K = logits.shape[0], self.cfg.top_k
         cfg, keep = self._router_cfg(router, logits)
-        ids = torch.empty(T, K, dtype=torch.int32, device=logits.device)
-        w = torch.empty(T, K, dtype=router.w_dtype or self.act_dtype, device=logits.device)
+        with _alloc_on(stream):
+            ids = torch.empty(T, K, dtype=torch.int32, device=logits.device)
+            w = torch.empty(T, K, dtype=router.w_dtype or self.act_dtype, device=logits.device)
         C.check(self._lib.ek_layer_route(self._h, _ptr(logits), ctypes.byref(cfg), T, _ptr(ids), _ptr(w),
                                          _mem(logits), _stream_ptr(stream)))
         del keep
@@ -272,9 +289,10 @@ class HipLayer:
         T, K = x.shape[0], self.cfg.top_k
         assert logits.shape[0] == T and _mem(x) == _mem(logits)
         cfg, keep = self._router_cfg(router, logits)
-        y = torch.empty_like(x)
-        ids = torch.empty(T, K, dtype=torch.int32, device=x.device)
-        w = torch.empty(T, K, dtype=router.w_dtype or self.act_dtype, device=x.device)
+        with _alloc_on(stream):
+            y = torch.empty_like(x)
+            ids = torch.empty(T, K, dtype=torch.int32, device=x.device)
+            w = torch.empty(T, K, dtype=router.w_dtype or self.act_dtype, device=x.device)
         C.check(self._lib.ek_layer_forward_logits(self._h, _ptr(x), _ptr(logits), ctypes.byref(cfg), T, _ptr(y),
                                                   _ptr(ids), _ptr(w), None, _mem(x), _stream_ptr(stream)))
         del keep
@@ -284,8 +302,9 @@ class HipLayer:
         """Several per-expert calls as one grouped launch; xs[i] is [n_i, H]."""
         n = len(experts)
         assert n == len(xs)
-        xs = [x.contiguous() for x in xs]
-        outs = [torch.empty_like(x) for x in xs]
+        with _alloc_on(stream):
+            xs = [x.contiguous() for x in xs]
+            outs = [torch.empty_like(x) for x in xs]
         mem = _mem(xs[0]) if n else C.EK_HOST
         assert all(_mem(x) == mem for x in xs)
         ex = (ctypes.c_int32 * n)(*experts)
@@ -369,7 +388,8 @@ class HipChain:
         assert x.is_cuda and ids.is_cuda and w.is_cuda and ids.dtype == torch.int32
         assert x.is_contiguous() and ids.is_contiguous() and w.is_contiguous()
         assert ids.dim() == 3 and ids.shape[0] == len(self.layers) and w.shape == ids.shape
-        y = out if out is not None else torch.empty_like(x)
+        with (_alloc_on(stream) if out is None else _NO_CTX):
+            y = out if out is not None else torch.empty_like(x)
         C.check(self._lib.ek_chain_forward(self._h, _ptr(x), _ptr(ids), _ptr(w), _DT[w.dtype], x.shape[0], _ptr(y),
                                            int(use_graph), _stream_ptr(stream)))
         return y
@@ -457,8 +477,9 @@ class HipFFN:
         return torch.rand(batch, self._instance.hidden).to(self._act_dtype)
 
     def forward(self, x: torch.Tensor, stream=None) -> torch.Tensor:
-        x = x.contiguous()
-        out = torch.empty_like(x)
+        with _alloc_on(stream):
+            x = x.contiguous()
+            out = torch.empty_like(x)
         C.check(self._lib.ek_expert_forward(self._h, _ptr(x), x.shape[0], _ptr(out), _mem(x), _stream_ptr(stream)))
         return out
 

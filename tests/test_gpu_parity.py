@@ -271,6 +271,26 @@ def test_tile_route_one_expert(ek, oracle, cuda, dt, w8, n):
     layer.close()
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("w8", [False, True])
+def test_narrow_and_wide_tiles_give_the_same_bits(ek, oracle, cuda, dt, w8):
+    """A per-expert call whose tiles would cover at most half the chip runs the tile kernel's narrow
+    form (half the channels per workgroup); the same rows routed to that expert through the layer
+    call run the wide form.  Every output element is the same sum in the same order: same bits;
+    and both hold the gate against the oracle."""
+    w = wl.Workload("t", 256, 192, 2, 1, 2000, dt, w8=w8)
+    layer, ws = load_layer(ek, w, experts=[1])
+    wu, wg, wd = [t[1] for t in oracle_weights(oracle, ws, 2, dt)]
+    for n in (1000, 2000):     # 7 full tiles + 104 rows, 15 full tiles + 80 rows (well below 700 rows a per-expert
+                               # call of this shape is cut for the streaming kernel instead)
+        x = torch.randn(n, w.hidden, generator=torch.Generator().manual_seed(n)).to(dt)
+        narrow = layer.expert_forward(1, x.to(cuda))
+        wide = layer.forward(x.to(cuda), torch.ones(n, 1, dtype=torch.int32, device=cuda), torch.ones(n, 1, dtype=dt, device=cuda))
+        assert torch.equal(narrow.view(torch.int16), wide.view(torch.int16)), (dt, w8, n)
+        ffn_gate(narrow, oracle.ffn(x, wu, wg, wd, mode=2), f"narrow tiles dt={dt} w8={w8} n={n}", plain=False)
+    layer.close()
+
+
 @pytest.mark.parametrize("H,I,w8", [(128, 64, False), (64, 128, False), (64, 64, False), (128, 128, True), (256, 128, True)])
 def test_tile_route_shortest_contractions(ek, oracle, cuda, H, I, w8):
     """The tile kernel's pipeline at its shortest: contractions of one and two 64-element steps
