@@ -30,6 +30,11 @@
 // Each XCD walks a contiguous eighth of every work list, so neighbouring
 // workgroups share the activation tile and mostly the expert's weights in
 // that XCD's L2.
+// The kernel exists in two forms, chosen by the host per launch: wide (two column blocks of 32
+// channels per wave: the figures above) and narrow (one column block per wave, so half the
+// channels per workgroup and twice the workgroups per item, three stages with 16-bit weights
+// too) for launches whose tiles would leave most of the chip idle.  Every output element is the
+// same sum in the same order in both.
 #include "ek_internal.h"
 #include "ek_mfma.h"
 
