@@ -85,6 +85,25 @@ def test_one_expert_streamed(ek, oracle, cuda, dt, n, kind):
 
 
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
+def test_one_expert_tiled(ek, oracle, cuda, kind):
+    """A per-expert call long enough to be cut into tiles: with per-channel int8 or 16-bit weights it
+    would run the tile kernel's narrow form; block-scaled weights have the wide form only, and the
+    same rows through the layer call give the same bits."""
+    H, I, n, dt = 384, 256, 1500, torch.bfloat16
+    layer = ek.HipLayer(H, I, 2, 1, act_dtype=dt, max_tokens=n, **KINDS[kind])
+    ew = make_expert(ek, H, I, 12, kind)
+    layer.set_expert(1, ew)
+    x = torch.randn(n, H, generator=torch.Generator().manual_seed(n)).to(dt)
+    ref = oracle.ffn(x, *ref_weights(oracle, ew, dt), mode=2)
+    got = layer.expert_forward(1, x.to(cuda))
+    ffn_gate(got, ref, f"{kind} block expert tiled n={n}", plain=False)
+    assert check_vs_rounded(got, ref) > 0.9
+    routed = layer.forward(x.to(cuda), torch.ones(n, 1, dtype=torch.int32, device=cuda), torch.ones(n, 1, dtype=dt, device=cuda))
+    assert torch.equal(routed.view(torch.int16), got.view(torch.int16))
+    layer.close()
+
+
+@pytest.mark.parametrize("kind", ["fp8", "int8"])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("T,E,K,H,I", [(24, 8, 2, 384, 256), (300, 6, 2, 512, 384), (700, 4, 1, 256, 640)])
 def test_layer_both_kernel_families(ek, oracle, cuda, dt, T, E, K, H, I, kind):
