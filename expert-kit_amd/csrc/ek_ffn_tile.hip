@@ -117,7 +117,10 @@ template <bool W8, int WAVES, int CB, int BMMAX> struct TileGeom {
     static constexpr int STAGE = XS + WS;
     // 16-bit weights: two stages of 80 KiB with two column blocks per wave, three of 48 KiB with one
     static constexpr int STAGES = W8 || CB == 1 ? 3 : 2;
-    static constexpr int SCALE_BYTES = 2 * WAVES * CB * 64 * 4;   // [tile parity][wave][column block][block]
+    // block scales: [tile parity][wave][scale row][block]; a wave has one scale row per column block,
+    // two (up, gate) when its single column block holds both matrices
+    static constexpr int SCALE_ROWS = CB == 1 ? 2 : CB;
+    static constexpr int SCALE_BYTES = 2 * WAVES * SCALE_ROWS * 64 * 4;
 };
 
 // XOR key of a row: fragment reads of 16 consecutive rows and one piece index
@@ -168,7 +171,6 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     static_assert(RB >= 1, "items have at least 32 rows");
     static_assert(BM <= BMMAX, "the activation stage holds the tile");
     static_assert(NMAT == 1 || CB % 2 == 0 || CB == 1, "up and gate blocks come in pairs, or share one block");
-    static_assert(!(block_scaled(WM) && CB == 1), "block-scaled weights are served by the wide form only");
     // CB == 1 with two matrices: the wave's one column block is {16 up channels, 16 gate channels}
     // of the same 16 hidden channels (lanes 0-15 / 16-31 of the A operand), and a lane's accumulator
     // holds up in registers 0-7 and gate of the same channels in registers 8-15.
@@ -223,8 +225,9 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
     // each, so a step's scale is one number per column block; the tile's rows of the scale
     // matrices sit in a wave-private LDS area (two areas: the next tile's rows are fetched while
     // this one's are in use)
-    float *const sc_area = (float *)(lds + NS * G::STAGE) + wave * (CB * kTileScaleBlocks);
-    constexpr int kScaleSlotFloats = kTileWaves * CB * kTileScaleBlocks;
+    constexpr int SCB = G::SCALE_ROWS;
+    float *const sc_area = (float *)(lds + NS * G::STAGE) + wave * (SCB * kTileScaleBlocks);
+    constexpr int kScaleSlotFloats = kTileWaves * SCB * kTileScaleBlocks;
     auto fetch = [&](int t, Ctx &c, int sslot) -> int {
         for (; t < ntiles; t += stride) {
             const WorkItem item = items[t / nb_count];
@@ -252,12 +255,16 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                 }
                 c.as[cb] = sv;
                 c.ac[cb] = -128.f * sv;
-                if constexpr (block_scaled(WM)) {
-                    const int KB = (a.Kdim + 127) >> 7;
-                    const int ct = min(cblock * NR + (NMAT == 2 ? cb >> 1 : cb) * 2, NT - 1);
-                    const float *smat = NMAT == 2 ? ((cb & 1) == 0 ? slab.s_up : slab.s_gate) : slab.s_down;
+            }
+            if constexpr (block_scaled(WM)) {
+                const int KB = (a.Kdim + 127) >> 7;
+#pragma unroll
+                for (int sr = 0; sr < (kSplitBlock ? 2 : CB); ++sr) {
+                    // scale row sr belongs to column block sr, or to matrix sr of the one split block
+                    const int ct = min(cblock * NR + (kSplitBlock ? 0 : (NMAT == 2 ? sr >> 1 : sr) * 2), NT - 1);
+                    const float *smat = NMAT == 2 ? ((sr & 1) == 0 ? slab.s_up : slab.s_gate) : slab.s_down;
                     if (lane < KB)
-                        sc_area[sslot * kScaleSlotFloats + cb * kTileScaleBlocks + lane] = smat[(int64_t)((ct * 16) >> 7) * KB + lane];
+                        sc_area[sslot * kScaleSlotFloats + sr * kTileScaleBlocks + lane] = smat[(int64_t)((ct * 16) >> 7) * KB + lane];
                 }
             }
             c.sslot = sslot;
@@ -362,7 +369,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             if constexpr (block_scaled(WM)) {
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
-                    sblk[cb] = sc_area[cur.sslot * kScaleSlotFloats + cb * kTileScaleBlocks + (step >> 1)];
+                    sblk[cb] = sc_area[cur.sslot * kScaleSlotFloats + (kSplitBlock ? hh : cb) * kTileScaleBlocks + (step >> 1)];
             }
             auto dq = [&](uint32_t w, int cb) -> u32x2 {
 #ifdef EK_ABL_NO_DEQUANT
@@ -568,8 +575,12 @@ static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, const int64_t
             return stage == 1 ? launch_t<T, kWI8, 2, 8, 1>(a, max_items, s) : launch_t<T, kWI8, 1, 8, 1>(a, max_items, s);
         return stage == 1 ? launch_t<T, kWI8, 2, 8, 2>(a, max_items, s) : launch_t<T, kWI8, 1, 8, 2>(a, max_items, s);
     case kWF8Block:
+        if (narrow)
+            return stage == 1 ? launch_t<T, kWF8Block, 2, 8, 1>(a, max_items, s) : launch_t<T, kWF8Block, 1, 8, 1>(a, max_items, s);
         return stage == 1 ? launch_t<T, kWF8Block, 2, 8, 2>(a, max_items, s) : launch_t<T, kWF8Block, 1, 8, 2>(a, max_items, s);
     case kWI8Block:
+        if (narrow)
+            return stage == 1 ? launch_t<T, kWI8Block, 2, 8, 1>(a, max_items, s) : launch_t<T, kWI8Block, 1, 8, 1>(a, max_items, s);
         return stage == 1 ? launch_t<T, kWI8Block, 2, 8, 2>(a, max_items, s) : launch_t<T, kWI8Block, 1, 8, 2>(a, max_items, s);
     default:
         if (narrow)

@@ -163,8 +163,7 @@ hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, int wmode, in
 // MFMA tile kernel over the three tile lists (128-row items first, then 64,
 // then 32); max_items[l] bounds list l.  A workgroup covers tile_channels(stage, narrow) output
 // channels of one item; the narrow form (half the channels per workgroup, so twice the workgroups
-// per item; same bits) is for launches that would leave most of the chip without a tile, and
-// exists for per-channel int8 and 16-bit weights only (ignored otherwise).
+// per item; same bits) is for launches that would leave most of the chip without a tile.
 hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, int wmode,
                            const int64_t max_items[kNumLists], bool narrow, hipStream_t s);
 // hidden channels (stage 1) / output channels (stage 2) per tile workgroup

@@ -86,9 +86,9 @@ def test_one_expert_streamed(ek, oracle, cuda, dt, n, kind):
 
 @pytest.mark.parametrize("kind", ["fp8", "int8"])
 def test_one_expert_tiled(ek, oracle, cuda, kind):
-    """A per-expert call long enough to be cut into tiles: with per-channel int8 or 16-bit weights it
-    would run the tile kernel's narrow form; block-scaled weights have the wide form only, and the
-    same rows through the layer call give the same bits."""
+    """A per-expert call long enough to be cut into tiles runs the tile kernel's narrow form (a wave's
+    single column block then holds up and gate channels, each with the scale row of its own matrix);
+    the same rows through the layer call run the wide form and give the same bits."""
     H, I, n, dt = 384, 256, 1500, torch.bfloat16
     layer = ek.HipLayer(H, I, 2, 1, act_dtype=dt, max_tokens=n, **KINDS[kind])
     ew = make_expert(ek, H, I, 12, kind)
