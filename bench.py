@@ -284,6 +284,9 @@ def main():
                          "DeepSeek-V3 checkpoint stores them, instead of the configuration's int8 per channel; "
                          "bf16: the same layer with 16-bit weights")
     ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--tokens", type=int, default=0,
+                    help="run the workload's layer at another token count (a parity-test style variation, e.g. other "
+                         "decode batch sizes of c3; implies --no-prefill)")
     ap.add_argument("--no-prefill", dest="prefill", action="store_false",
                     help="with --workload c3: do not also measure the c4 prefill call on the same experts")
     ap.add_argument("--no-parity", dest="parity", action="store_false", help="skip the oracle's output gate before timing")
@@ -315,6 +318,11 @@ def main():
         assert w.w8, "--weights bf16 applies to the W8A16 configurations (c3, c4)"
         from dataclasses import replace
         w = replace(w, w8=False)
+    if args.tokens > 0:
+        assert w.n_layers == 1, "--tokens applies to the single-layer configurations"
+        from dataclasses import replace
+        w = replace(w, tokens=args.tokens, name=f"{w.name}_T{args.tokens}")
+        args.prefill = False
     if w.n_layers > 1:
         return bench_chain(args, w, dev)
     # the decode configuration the metric is quoted on and the prefill configuration hold the same
