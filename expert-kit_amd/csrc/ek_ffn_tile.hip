@@ -72,6 +72,12 @@ __device__ __forceinline__ void block_barrier()
 {
     asm volatile("s_barrier" : : : "memory");
 }
+// Workgroup barrier that publishes LDS only: this wave's LDS reads and writes have completed, its
+// global loads stay in flight (__syncthreads would wait for them as well).
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
+}
 
 // Timing-only builds (`make ablation ABL=...`, WRONG RESULTS, never the shipped library): the
 // tile kernel with one part of its step left out, to measure what that part costs in cycles
@@ -523,6 +529,243 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 #undef EK_ISSUE
 }
 
+// ---- short tiles with weights streamed into registers ------------------------------------------
+// 32- and 64-row items whose expert has one or two tiles (a few dozen rows per expert: layer
+// calls between the decode and the prefill regime, the mid-sized experts of a skewed prefill) read
+// weights that are cold in every cache, and with 32 or 64 rows the accumulators take 32 to 64
+// registers.  This form gives the rest to the loads: a lane's 16 bytes of a 1 KiB weight chunk are
+// exactly its A-operand bytes (two runs of 512 contiguous bytes per load instruction), so the
+// weights come straight from HBM into registers, kMidDepth steps ahead, as the weight-streaming
+// kernel fetches them, and never touch LDS.  Only the activation tile (4 or 8 KiB per step) goes
+// through LDS: one 16-byte piece per thread and step, fetched one to two windows of kMidDepth
+// steps ahead into a register and stored (XOR-swizzled as in run_tiles) into the other of two
+// window buffers during the window before its own; one workgroup barrier per window publishes it,
+// so the waves drift apart by up to a window instead of meeting at every step.  All loads are
+// ordinary loads: the compiler counts them.
+// Loads run across tile boundaries like run_tiles' DMAs.  Arithmetic, operand layouts, channel
+// split over the waves and the epilogue are run_tiles' (wide form): same bits.
+// Needs per-channel int8 weights and a contraction of a multiple of 64 * kMidDepth elements, at
+// least 2 * kMidDepth steps long; the caller falls back to run_tiles otherwise.
+constexpr int kMidDepth = 4;
+constexpr int kMidXStep = 8192;                 // bytes reserved per step of the activation tile (64 rows x 64 k x 2)
+constexpr int kMidXBuf = kMidDepth * kMidXStep; // one window
+constexpr int kMidScratch = 2 * kMidXBuf;       // epilogue scratch behind the two window buffers
+
+template <typename T> struct MidCtx {
+    const uint8_t *wl[2];    // this lane's bytes of the column block's weight chunks at step 0, slot tt = 0
+    const T *xsrc;           // this thread's 16-byte piece of the activation tile at step 0
+    float as[2], ac[2];
+    int row0, nrows, chan0;
+};
+
+template <typename T, int NMAT, int MR>
+__device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items, const int ntiles,
+                                        const int nb_count, const int first, const int stride, uint8_t *lds)
+{
+    using V8 = typename Act<T>::V8;
+    constexpr int WAVES = 8, CB = 2, NR = 4 / NMAT, D = kMidDepth;
+    constexpr int BM = MR * 16, RB = MR / 2, BK = 64, PPR = 8, NGRP = 4;
+    constexpr int kRowBlockBytes = 32 * PPR * 16;
+    static_assert(MR == 2 || MR == 4, "32- and 64-row items");
+    typedef MidCtx<T> Ctx;
+    if (first >= ntiles) return;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15, l32 = lane & 31, kg = lane >> 5, hh = l32 >> 4;
+    const int NT = a.N >> 4;
+    const int nsteps = a.Kdim / BK;
+    // this thread's piece of the activation tile
+    const int xrow = tid / PPR, xpiece = tid % PPR;
+    const bool xactive = xrow < BM;
+    const int xdst = (xrow * PPR + (xpiece ^ swizzle_key<PPR>(xrow))) * 16;
+    int boff[NGRP];
+#pragma unroll
+    for (int grp = 0; grp < NGRP; ++grp) {
+        const int c = ((grp >> 1) * 2 + kg) * 2 + (grp & 1);
+        boff[grp] = (l32 * PPR + (c ^ swizzle_key<PPR>(j))) * 16;
+    }
+    auto fetch = [&](int t, Ctx &c) -> int {
+        for (; t < ntiles; t += stride) {
+            const WorkItem item = items[t / nb_count];
+            const int nb = t % nb_count;
+            const ExpertSlab slab = a.slabs[item.expert];
+            const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
+            if (wmat == nullptr) continue;       // not loaded: pack has flagged the call
+            c.row0 = item.row0;
+            c.nrows = item.nrows;
+            const int cblock = nb * WAVES + wave;
+            c.chan0 = cblock * NR * 16;
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                const int nr = (NMAT == 2 ? 0 : cb) * 2 + hh, m = NMAT == 2 ? cb : 0;
+                const int ctc = min(cblock * NR + nr, NT - 1);   // tiles past N recompute the last one
+                c.wl[cb] = wmat + ((int64_t)ctc * nsteps * NMAT + m) * kChunkBytes + (kg * 16 + j) * 16;
+                const int ch = ctc * 16 + j;
+                const float sv = NMAT == 2 ? (cb == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
+                c.as[cb] = sv;
+                c.ac[cb] = -128.f * sv;
+            }
+            const int rr = min(min(xrow, BM - 1), item.nrows - 1);   // rows past the item (and threads past the tile) re-read its last row
+            const int64_t row = a.rows ? (int64_t)a.rows[item.row0 + rr] : (int64_t)(item.row0 + rr);
+            c.xsrc = (const T *)a.x + row * a.x_stride + xpiece * 8;
+            return t;
+        }
+        return -1;
+    };
+    u32x4 wq[D][2][CB];      // ring of weight bytes: slot s % D holds step s
+    u32x4 xq[D];             // activation pieces of the window after next: slot u holds its step u
+    auto load_w = [&](const Ctx &c, int step, int slot) {
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+                wq[slot][tt][cb] = __builtin_bit_cast(u32x4, ldg16_once(c.wl[cb] + (int64_t)step * (NMAT * kChunkBytes) + tt * 512));
+    };
+    auto load_x = [&](const Ctx &c, int step, int slot) {
+        xq[slot] = __builtin_bit_cast(u32x4, ldg16(c.xsrc + step * BK));
+    };
+    // The loads of a step are unconditional and land in the ring slot they refill (no copies, no
+    // merges of register values across branches: the compiler then keeps the ring in place and waits
+    // for exactly the loads a step needs).  Past the last tile's end they re-read its first steps.
+
+    Ctx cur, nxt;
+    int tc = fetch(first, cur);
+    if (tc < 0) return;
+    nxt = cur;
+#pragma unroll
+    for (int v = 0; v < D; ++v) { load_w(cur, v, v); load_x(cur, v, v); }
+    block_barrier();                             // every wave has left the previous class's LDS
+    int par = 0;                                 // buffer of the current window
+#pragma unroll
+    for (int v = 0; v < D; ++v) {
+        if (xactive) *(u32x4 *)(lds + v * kMidXStep + xdst) = xq[v];
+        load_x(cur, D + v, v);                   // (nsteps >= 2 D)
+    }
+    lds_barrier();
+    const int fstep = nsteps - 2 * D;            // the next tile's addresses are needed from here on
+    while (true) {
+        int tn = -1;
+        f32x16 acc[RB][CB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[rb][cb][r] = 0.f;
+        for (int step0 = 0; step0 < nsteps; step0 += D) {
+#pragma unroll
+            for (int u = 0; u < D; ++u) {
+                const int step = step0 + u;
+                if (step == fstep) {
+                    tn = fetch(tc + stride, nxt);
+                    if (tn < 0) nxt = cur;
+                }
+                // the piece of step + D goes to the other window buffer; its slot takes step + 2 D
+                if (xactive) *(u32x4 *)(lds + (par ^ 1) * kMidXBuf + u * kMidXStep + xdst) = xq[u];
+                {
+                    const bool in_cur = step + 2 * D < nsteps;
+                    const T *xp = in_cur ? cur.xsrc : nxt.xsrc;
+                    const int xs = in_cur ? step + 2 * D : step + 2 * D - nsteps;
+                    xq[u] = __builtin_bit_cast(u32x4, ldg16(xp + xs * BK));
+                }
+                u32x4 (&aq)[2][CB] = wq[u];
+                const uint8_t *stage = lds + par * kMidXBuf + u * kMidXStep;
+                u32x4 af[2][CB];
+                V8 bf[2][RB];
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const u32x2 lo = dequant_u8x4<T>(aq[0][cb][0], cur.as[cb], cur.ac[cb]);
+                    const u32x2 hi = dequant_u8x4<T>(aq[0][cb][1], cur.as[cb], cur.ac[cb]);
+                    af[0][cb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+                }
+#pragma unroll
+                for (int grp = 0; grp < NGRP; ++grp) {
+                    const int cg = grp & 1, ng = cg ^ 1;
+                    if (grp + 1 < NGRP) {
+#pragma unroll
+                        for (int rb = 0; rb < RB; ++rb) bf[ng][rb] = *(const V8 *)(stage + boff[grp + 1] + rb * kRowBlockBytes);
+                    }
+#pragma unroll
+                    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                        for (int cb = 0; cb < CB; ++cb)
+                            acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cg][cb]), bf[cg][rb], acc[rb][cb]);
+                    if (grp + 1 < NGRP) {
+                        const int g1 = grp + 1;
+#pragma unroll
+                        for (int cb = 0; cb < CB; ++cb) {
+                            const u32x2 lo = dequant_u8x4<T>(aq[g1 >> 1][cb][(g1 & 1) * 2], cur.as[cb], cur.ac[cb]);
+                            const u32x2 hi = dequant_u8x4<T>(aq[g1 >> 1][cb][(g1 & 1) * 2 + 1], cur.as[cb], cur.ac[cb]);
+                            af[ng][cb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+                        }
+                    }
+                }
+                // this step's weight bytes have been converted: their slot takes step + D
+                {
+                    const bool in_cur = step + D < nsteps;
+                    const int ws = in_cur ? step + D : step + D - nsteps;
+#pragma unroll
+                    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                        for (int cb = 0; cb < CB; ++cb) {
+                            const uint8_t *wp_ = in_cur ? cur.wl[cb] : nxt.wl[cb];
+                            wq[u][tt][cb] = __builtin_bit_cast(u32x4, ldg16_once(wp_ + (int64_t)ws * (NMAT * kChunkBytes) + tt * 512));
+                        }
+                }
+            }
+            par ^= 1;
+            lds_barrier();         // the next window's buffer is complete; this window's may be overwritten
+        }
+        // ---- epilogue: as run_tiles, through a wave-private scratch behind the two buffers
+        typedef T T4 __attribute__((ext_vector_type(4)));
+        constexpr int OUTC = NMAT == 2 ? 32 : 64;
+        constexpr int RS = OUTC * 2 + 16;
+        constexpr int PPO = OUTC * 2 / 16, RPI = 64 / PPO;
+        if (cur.chan0 < a.N) {
+            uint8_t *scr = lds + kMidScratch + wave * (32 * RS);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                if (rb * 32 >= cur.nrows) break;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if constexpr (NMAT == 2) {
+                        T4 o;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) o[r] = swiglu_rounded<T>(acc[rb][0][q * 4 + r], acc[rb][1][q * 4 + r]);
+                        *(uint2 *)(scr + l32 * RS + (q * 8 + kg * 4) * 2) = __builtin_bit_cast(uint2, o);
+                    } else {
+#pragma unroll
+                        for (int cb = 0; cb < CB; ++cb) {
+                            T4 o;
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) o[r] = (T)acc[rb][cb][q * 4 + r];
+                            *(uint2 *)(scr + l32 * RS + (cb * 32 + q * 8 + kg * 4) * 2) = __builtin_bit_cast(uint2, o);
+                        }
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int i = 0; i < 32 / RPI; ++i) {
+                    const int r_in = rb * 32 + i * RPI + lane / PPO;
+                    const u32x4 v = *(const u32x4 *)(scr + (i * RPI + lane / PPO) * RS + (lane % PPO) * 16);
+                    if (r_in < cur.nrows)
+                        *(u32x4 *)((T *)a.out + (int64_t)(cur.row0 + r_in) * a.out_stride + cur.chan0 + (lane % PPO) * 8) = v;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+        if (tn < 0) break;
+        cur = nxt;
+        tc = tn;
+    }
+    lds_barrier();
+}
+
 // Persistent launch: one workgroup per CU (the LDS stages fill it), numbered so that
 // workgroup b runs on XCD b % 8 (round-robin dispatch).  Each XCD is given a contiguous
 // eighth of every work list, and its workgroups walk that eighth's tiles side by side:
@@ -544,6 +787,15 @@ __global__ __launch_bounds__(WAVES * 64, 1) void ffn_tile_kernel(FfnArgs a, int 
     run_tiles<T, WM, NMAT, 8, WAVES, CB, 128>(a, a.lists.items[kListT128] + lo128, s128 * nb_count, nb_count, slot, nslots, lds, lds_base);
     // the shorter classes start where the long one left the CUs least loaded
     const int r64 = (slot + nslots - (s128 * nb_count) % nslots) % nslots;
+    if constexpr (WM == kWI8 && CB == 2 && WAVES == 8) {
+        const int nsteps = a.Kdim / 64;
+        if (nsteps % kMidDepth == 0 && nsteps >= 2 * kMidDepth) {
+            const int r32m = (r64 + nslots - (s64 * nb_count) % nslots) % nslots;
+            run_mid<T, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds);
+            run_mid<T, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32m, nslots, lds);
+            return;
+        }
+    }
     run_tiles<T, WM, NMAT, 4, WAVES, CB, 128>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds, lds_base);
     const int r32 = (r64 + nslots - (s64 * nb_count) % nslots) % nslots;
     run_tiles<T, WM, NMAT, 2, WAVES, CB, 128>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32, nslots, lds, lds_base);
