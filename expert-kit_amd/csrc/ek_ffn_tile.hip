@@ -34,7 +34,8 @@
 // channels per wave: the figures above) and narrow (one column block per wave, so half the
 // channels per workgroup and twice the workgroups per item, three stages with 16-bit weights
 // too) for launches whose tiles would leave most of the chip idle.  Every output element is the
-// same sum in the same order in both.
+// same sum in the same order in both.  In the wide form the 32- and 64-row items of layers with
+// one-byte weights take a third path, run_mid below: weights from HBM straight into registers.
 #include "ek_internal.h"
 #include "ek_mfma.h"
 
@@ -544,21 +545,23 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 // ordinary loads: the compiler counts them.
 // Loads run across tile boundaries like run_tiles' DMAs.  Arithmetic, operand layouts, channel
 // split over the waves and the epilogue are run_tiles' (wide form): same bits.
-// Needs per-channel int8 weights and a contraction of a multiple of 64 * kMidDepth elements, at
-// least 2 * kMidDepth steps long; the caller falls back to run_tiles otherwise.
+// Needs one-byte weights and a contraction of a multiple of 64 * kMidDepth elements, at least
+// 2 * kMidDepth steps long; the caller falls back to run_tiles otherwise.
 constexpr int kMidDepth = 4;
 constexpr int kMidXStep = 8192;                 // bytes reserved per step of the activation tile (64 rows x 64 k x 2)
 constexpr int kMidXBuf = kMidDepth * kMidXStep; // one window
 constexpr int kMidScratch = 2 * kMidXBuf;       // epilogue scratch behind the two window buffers
+constexpr int kMidScales = kMidScratch + 8 * 32 * 144;   // block scales behind the scratch: [tile parity][wave][column block][block]
 
 template <typename T> struct MidCtx {
     const uint8_t *wl[2];    // this lane's bytes of the column block's weight chunks at step 0, slot tt = 0
     const T *xsrc;           // this thread's 16-byte piece of the activation tile at step 0
     float as[2], ac[2];
     int row0, nrows, chan0;
+    int sslot;               // block-scaled weights: which of the two LDS scale areas holds this tile's rows
 };
 
-template <typename T, int NMAT, int MR>
+template <typename T, int WM, int NMAT, int MR>
 __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items, const int ntiles,
                                         const int nb_count, const int first, const int stride, uint8_t *lds)
 {
@@ -567,6 +570,7 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
     constexpr int BM = MR * 16, RB = MR / 2, BK = 64, PPR = 8, NGRP = 4;
     constexpr int kRowBlockBytes = 32 * PPR * 16;
     static_assert(MR == 2 || MR == 4, "32- and 64-row items");
+    static_assert(WM != kW16, "one-byte weights");
     typedef MidCtx<T> Ctx;
     if (first >= ntiles) return;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -584,7 +588,10 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
         const int c = ((grp >> 1) * 2 + kg) * 2 + (grp & 1);
         boff[grp] = (l32 * PPR + (c ^ swizzle_key<PPR>(j))) * 16;
     }
-    auto fetch = [&](int t, Ctx &c) -> int {
+    // block scales: as in run_tiles, the tile's rows of the scale matrices in a wave-private LDS area
+    float *const sc_area = (float *)(lds + kMidScales) + wave * (CB * kTileScaleBlocks);
+    constexpr int kScaleSlotFloats = WAVES * CB * kTileScaleBlocks;
+    auto fetch = [&](int t, Ctx &c, int sslot) -> int {
         for (; t < ntiles; t += stride) {
             const WorkItem item = items[t / nb_count];
             const int nb = t % nb_count;
@@ -593,6 +600,7 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
             if (wmat == nullptr) continue;       // not loaded: pack has flagged the call
             c.row0 = item.row0;
             c.nrows = item.nrows;
+            c.sslot = sslot;
             const int cblock = nb * WAVES + wave;
             c.chan0 = cblock * NR * 16;
 #pragma unroll
@@ -600,10 +608,24 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
                 const int nr = (NMAT == 2 ? 0 : cb) * 2 + hh, m = NMAT == 2 ? cb : 0;
                 const int ctc = min(cblock * NR + nr, NT - 1);   // tiles past N recompute the last one
                 c.wl[cb] = wmat + ((int64_t)ctc * nsteps * NMAT + m) * kChunkBytes + (kg * 16 + j) * 16;
-                const int ch = ctc * 16 + j;
-                const float sv = NMAT == 2 ? (cb == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
+                float sv = 1.f;
+                if constexpr (WM == kWI8) {
+                    const int ch = ctc * 16 + j;
+                    sv = NMAT == 2 ? (cb == 0 ? slab.s_up[ch] : slab.s_gate[ch]) : slab.s_down[ch];
+                }
                 c.as[cb] = sv;
                 c.ac[cb] = -128.f * sv;
+                if constexpr (block_scaled(WM)) {
+                    const int KB = (a.Kdim + 127) >> 7;
+                    const int ct = min(cblock * NR + (NMAT == 2 ? 0 : cb * 2), NT - 1);
+                    const float *smat = NMAT == 2 ? (cb == 0 ? slab.s_up : slab.s_gate) : slab.s_down;
+                    if (lane < KB)
+                        sc_area[sslot * kScaleSlotFloats + cb * kTileScaleBlocks + lane] = smat[(int64_t)((ct * 16) >> 7) * KB + lane];
+                }
+            }
+            if constexpr (block_scaled(WM)) {
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
             }
             const int rr = min(min(xrow, BM - 1), item.nrows - 1);   // rows past the item (and threads past the tile) re-read its last row
             const int64_t row = a.rows ? (int64_t)a.rows[item.row0 + rr] : (int64_t)(item.row0 + rr);
@@ -629,7 +651,7 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
     // for exactly the loads a step needs).  Past the last tile's end they re-read its first steps.
 
     Ctx cur, nxt;
-    int tc = fetch(first, cur);
+    int tc = fetch(first, cur, 0);
     if (tc < 0) return;
     nxt = cur;
 #pragma unroll
@@ -657,7 +679,7 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
             for (int u = 0; u < D; ++u) {
                 const int step = step0 + u;
                 if (step == fstep) {
-                    tn = fetch(tc + stride, nxt);
+                    tn = fetch(tc + stride, nxt, cur.sslot ^ 1);
                     if (tn < 0) nxt = cur;
                 }
                 // the piece of step + D goes to the other window buffer; its slot takes step + 2 D
@@ -674,10 +696,21 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
                 V8 bf[2][RB];
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) bf[0][rb] = *(const V8 *)(stage + boff[0] + rb * kRowBlockBytes);
+                float sblk[CB] = {};        // block-scaled weights: this step's scale per column block
+                if constexpr (block_scaled(WM)) {
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb)
+                        sblk[cb] = sc_area[cur.sslot * kScaleSlotFloats + cb * kTileScaleBlocks + (step >> 1)];
+                }
+                auto dq = [&](uint32_t w, int cb) -> u32x2 {
+                    if constexpr (WM == kWF8Block) return dequant_f8x4<T>(w, sblk[cb]);
+                    else if constexpr (WM == kWI8Block) return dequant_u8x4<T>(w, sblk[cb], -128.f * sblk[cb]);
+                    else return dequant_u8x4<T>(w, cur.as[cb], cur.ac[cb]);
+                };
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
-                    const u32x2 lo = dequant_u8x4<T>(aq[0][cb][0], cur.as[cb], cur.ac[cb]);
-                    const u32x2 hi = dequant_u8x4<T>(aq[0][cb][1], cur.as[cb], cur.ac[cb]);
+                    const u32x2 lo = dq(aq[0][cb][0], cb);
+                    const u32x2 hi = dq(aq[0][cb][1], cb);
                     af[0][cb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
                 }
 #pragma unroll
@@ -696,8 +729,8 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
                         const int g1 = grp + 1;
 #pragma unroll
                         for (int cb = 0; cb < CB; ++cb) {
-                            const u32x2 lo = dequant_u8x4<T>(aq[g1 >> 1][cb][(g1 & 1) * 2], cur.as[cb], cur.ac[cb]);
-                            const u32x2 hi = dequant_u8x4<T>(aq[g1 >> 1][cb][(g1 & 1) * 2 + 1], cur.as[cb], cur.ac[cb]);
+                            const u32x2 lo = dq(aq[g1 >> 1][cb][(g1 & 1) * 2], cb);
+                            const u32x2 hi = dq(aq[g1 >> 1][cb][(g1 & 1) * 2 + 1], cb);
                             af[ng][cb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
                         }
                     }
@@ -787,12 +820,12 @@ __global__ __launch_bounds__(WAVES * 64, 1) void ffn_tile_kernel(FfnArgs a, int 
     run_tiles<T, WM, NMAT, 8, WAVES, CB, 128>(a, a.lists.items[kListT128] + lo128, s128 * nb_count, nb_count, slot, nslots, lds, lds_base);
     // the shorter classes start where the long one left the CUs least loaded
     const int r64 = (slot + nslots - (s128 * nb_count) % nslots) % nslots;
-    if constexpr (WM == kWI8 && CB == 2 && WAVES == 8) {
+    if constexpr (WM != kW16 && CB == 2 && WAVES == 8) {
         const int nsteps = a.Kdim / 64;
         if (nsteps % kMidDepth == 0 && nsteps >= 2 * kMidDepth) {
             const int r32m = (r64 + nslots - (s64 * nb_count) % nslots) % nslots;
-            run_mid<T, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds);
-            run_mid<T, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32m, nslots, lds);
+            run_mid<T, WM, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds);
+            run_mid<T, WM, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32m, nslots, lds);
             return;
         }
     }
