@@ -545,11 +545,14 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 // ordinary loads: the compiler counts them.
 // Loads run across tile boundaries like run_tiles' DMAs.  Arithmetic, operand layouts, channel
 // split over the waves and the epilogue are run_tiles' (wide form): same bits.
-// Needs one-byte weights and a contraction of a multiple of 64 * kMidDepth elements, at least
-// 2 * kMidDepth steps long; the caller falls back to run_tiles otherwise.
-constexpr int kMidDepth = 4;
+// 16-bit weights bring twice the bytes per step: two steps ahead then hold what four steps of
+// one-byte weights hold (64 registers per lane, 128 KiB per CU in flight).
+// Needs a contraction of a multiple of 64 * mid_depth elements, at least 2 * mid_depth steps long;
+// the caller falls back to run_tiles otherwise.
+constexpr int kMidDepth = 4;                    // one-byte weights
+constexpr int mid_depth(int wm) { return wm == kW16 ? 2 : kMidDepth; }
 constexpr int kMidXStep = 8192;                 // bytes reserved per step of the activation tile (64 rows x 64 k x 2)
-constexpr int kMidXBuf = kMidDepth * kMidXStep; // one window
+constexpr int kMidXBuf = kMidDepth * kMidXStep; // one window (of kMidDepth steps at most)
 constexpr int kMidScratch = 2 * kMidXBuf;       // epilogue scratch behind the two window buffers
 constexpr int kMidScales = kMidScratch + 8 * 32 * 144;   // block scales behind the scratch: [tile parity][wave][column block][block]
 
@@ -566,11 +569,12 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
                                         const int nb_count, const int first, const int stride, uint8_t *lds)
 {
     using V8 = typename Act<T>::V8;
-    constexpr int WAVES = 8, CB = 2, NR = 4 / NMAT, D = kMidDepth;
+    constexpr bool W8 = WM != kW16;
+    constexpr int WAVES = 8, CB = 2, NR = 4 / NMAT, D = mid_depth(WM), KC = W8 ? 1 : 2;
+    constexpr int NQ = W8 ? 2 : 4;             // 16-byte loads per lane, column block and step
     constexpr int BM = MR * 16, RB = MR / 2, BK = 64, PPR = 8, NGRP = 4;
     constexpr int kRowBlockBytes = 32 * PPR * 16;
     static_assert(MR == 2 || MR == 4, "32- and 64-row items");
-    static_assert(WM != kW16, "one-byte weights");
     typedef MidCtx<T> Ctx;
     if (first >= ntiles) return;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -585,7 +589,7 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
     int boff[NGRP];
 #pragma unroll
     for (int grp = 0; grp < NGRP; ++grp) {
-        const int c = ((grp >> 1) * 2 + kg) * 2 + (grp & 1);
+        const int c = W8 ? ((grp >> 1) * 2 + kg) * 2 + (grp & 1) : grp * 2 + kg;
         boff[grp] = (l32 * PPR + (c ^ swizzle_key<PPR>(j))) * 16;
     }
     // block scales: as in run_tiles, the tile's rows of the scale matrices in a wave-private LDS area
@@ -607,7 +611,7 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
             for (int cb = 0; cb < CB; ++cb) {
                 const int nr = (NMAT == 2 ? 0 : cb) * 2 + hh, m = NMAT == 2 ? cb : 0;
                 const int ctc = min(cblock * NR + nr, NT - 1);   // tiles past N recompute the last one
-                c.wl[cb] = wmat + ((int64_t)ctc * nsteps * NMAT + m) * kChunkBytes + (kg * 16 + j) * 16;
+                c.wl[cb] = wmat + ((int64_t)ctc * nsteps * KC * NMAT + m) * kChunkBytes + (kg * 16 + j) * 16;
                 float sv = 1.f;
                 if constexpr (WM == kWI8) {
                     const int ch = ctc * 16 + j;
@@ -634,14 +638,20 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
         }
         return -1;
     };
-    u32x4 wq[D][2][CB];      // ring of weight bytes: slot s % D holds step s
+    u32x4 wq[D][NQ][CB];     // ring of weight bytes: slot s % D holds step s
+    // load q of a step: one-byte weights, the two halves of the step's chunk; 16-bit weights, the
+    // two halves of its two chunks (k-group q)
+    auto w_off = [&](int step, int q) -> int64_t {
+        return W8 ? (int64_t)step * (NMAT * kChunkBytes) + q * 512
+                  : (int64_t)(step * 2 + (q >> 1)) * (NMAT * kChunkBytes) + (q & 1) * 512;
+    };
     u32x4 xq[D];             // activation pieces of the window after next: slot u holds its step u
     auto load_w = [&](const Ctx &c, int step, int slot) {
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
+        for (int q = 0; q < NQ; ++q)
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb)
-                wq[slot][tt][cb] = __builtin_bit_cast(u32x4, ldg16_once(c.wl[cb] + (int64_t)step * (NMAT * kChunkBytes) + tt * 512));
+                wq[slot][q][cb] = __builtin_bit_cast(u32x4, ldg16_once(c.wl[cb] + w_off(step, q)));
     };
     auto load_x = [&](const Ctx &c, int step, int slot) {
         xq[slot] = __builtin_bit_cast(u32x4, ldg16(c.xsrc + step * BK));
@@ -690,7 +700,7 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
                     const int xs = in_cur ? step + 2 * D : step + 2 * D - nsteps;
                     xq[u] = __builtin_bit_cast(u32x4, ldg16(xp + xs * BK));
                 }
-                u32x4 (&aq)[2][CB] = wq[u];
+                u32x4 (&aq)[NQ][CB] = wq[u];
                 const uint8_t *stage = lds + par * kMidXBuf + u * kMidXStep;
                 u32x4 af[2][CB];
                 V8 bf[2][RB];
@@ -709,9 +719,13 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
                 };
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
-                    const u32x2 lo = dq(aq[0][cb][0], cb);
-                    const u32x2 hi = dq(aq[0][cb][1], cb);
-                    af[0][cb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+                    if constexpr (W8) {
+                        const u32x2 lo = dq(aq[0][cb][0], cb);
+                        const u32x2 hi = dq(aq[0][cb][1], cb);
+                        af[0][cb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+                    } else {
+                        af[0][cb] = aq[0][cb];
+                    }
                 }
 #pragma unroll
                 for (int grp = 0; grp < NGRP; ++grp) {
@@ -729,9 +743,13 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
                         const int g1 = grp + 1;
 #pragma unroll
                         for (int cb = 0; cb < CB; ++cb) {
-                            const u32x2 lo = dq(aq[g1 >> 1][cb][(g1 & 1) * 2], cb);
-                            const u32x2 hi = dq(aq[g1 >> 1][cb][(g1 & 1) * 2 + 1], cb);
-                            af[ng][cb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+                            if constexpr (W8) {
+                                const u32x2 lo = dq(aq[g1 >> 1][cb][(g1 & 1) * 2], cb);
+                                const u32x2 hi = dq(aq[g1 >> 1][cb][(g1 & 1) * 2 + 1], cb);
+                                af[ng][cb] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+                            } else {
+                                af[ng][cb] = aq[g1][cb];
+                            }
                         }
                     }
                 }
@@ -740,11 +758,11 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
                     const bool in_cur = step + D < nsteps;
                     const int ws = in_cur ? step + D : step + D - nsteps;
 #pragma unroll
-                    for (int tt = 0; tt < 2; ++tt)
+                    for (int q = 0; q < NQ; ++q)
 #pragma unroll
                         for (int cb = 0; cb < CB; ++cb) {
                             const uint8_t *wp_ = in_cur ? cur.wl[cb] : nxt.wl[cb];
-                            wq[u][tt][cb] = __builtin_bit_cast(u32x4, ldg16_once(wp_ + (int64_t)ws * (NMAT * kChunkBytes) + tt * 512));
+                            wq[u][q][cb] = __builtin_bit_cast(u32x4, ldg16_once(wp_ + w_off(ws, q)));
                         }
                 }
             }
@@ -820,9 +838,14 @@ __global__ __launch_bounds__(WAVES * 64, 1) void ffn_tile_kernel(FfnArgs a, int 
     run_tiles<T, WM, NMAT, 8, WAVES, CB, 128>(a, a.lists.items[kListT128] + lo128, s128 * nb_count, nb_count, slot, nslots, lds, lds_base);
     // the shorter classes start where the long one left the CUs least loaded
     const int r64 = (slot + nslots - (s128 * nb_count) % nslots) % nslots;
-    if constexpr (WM != kW16 && CB == 2 && WAVES == 8) {
+    if constexpr (CB == 2 && WAVES == 8) {
+        // the register-streamed form for the short items of a launch whose tiles fill the chip
+        // (measured: DeepSeek-V3 int8 layer at 512 / 1024 tokens -5 / -8 %, the ragged Qwen3 fp16
+        // chain -2.5 %); with a few tiles beside a long streaming chain (Qwen3 fp16 decode with
+        // skewed routing: +5 %) run_tiles' form is the faster one
         const int nsteps = a.Kdim / 64;
-        if (nsteps % kMidDepth == 0 && nsteps >= 2 * kMidDepth) {
+        if (nsteps % mid_depth(WM) == 0 && nsteps >= 2 * mid_depth(WM) &&
+            (int64_t)(n128 + n64 + n32) * nb_count >= (int64_t)gridDim.x) {
             const int r32m = (r64 + nslots - (s64 * nb_count) % nslots) % nslots;
             run_mid<T, WM, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds);
             run_mid<T, WM, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32m, nslots, lds);
