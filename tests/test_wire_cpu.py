@@ -217,3 +217,37 @@ def test_deeply_nested_header_is_refused_not_recursed_into():
         # unbalanced: only openers
         blob = _blob_with_header(b'{"x":' + b"[" * depth, data)
         assert lib.ek_safetensors_find(blob, len(blob), b"data", ctypes.byref(view)) == C.EK_INVALID_INPUT
+
+
+def test_parser_under_the_host_sanitizers(tmp_path):
+    """The same kind of mutations, 300 000 of them, through a build of the wire parser's host code
+    with AddressSanitizer and UndefinedBehaviorSanitizer (tests/wire_fuzz.cpp; blobs are exact-size
+    heap copies): an out-of-bounds read, a signed overflow or a bad shift inside the parser ends the
+    run with a report instead of going unnoticed."""
+    import os
+    import shutil
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    hipcc, clang = "/opt/rocm/bin/hipcc", "/opt/rocm/llvm/bin/clang++"
+    lib_dir = os.path.join(root, "expert-kit_amd", "lib")
+    if not (os.path.exists(hipcc) and os.path.exists(clang)):
+        pytest.skip("no ROCm compiler here")
+    assert os.path.exists(os.path.join(lib_dir, "libek_hip.so")), "build the library first"
+    san = ["-fsanitize=address", "-fsanitize=undefined", "-fno-sanitize-recover=undefined"]
+    host_san = [a for s in san for a in ("-Xarch_host", s)]
+    obj, drv, exe = (str(tmp_path / n) for n in ("ek_wire.o", "wire_fuzz.o", "wire_fuzz"))
+    src = os.path.join(root, "expert-kit_amd", "csrc")
+    run = lambda cmd: subprocess.run(cmd, check=True, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    run([hipcc, "--offload-arch=gfx950", "-O1", "-g", "-std=c++17", "-fPIC", *host_san, "-Xclang", "-target-feature",
+         "-Xclang", "-packed-fp32-ops", "-I" + src, "-c", os.path.join(src, "ek_wire.hip"), "-o", obj])
+    run([clang, "-O1", "-g", "-std=c++17", *san, "-I" + os.path.join(root, "include"), "-c",
+         os.path.join(root, "tests", "wire_fuzz.cpp"), "-o", drv])
+    # the executable's own (instrumented) parser takes precedence over the library's copy, which
+    # only supplies the layer entry points ek_wire.hip refers to
+    run([clang, *san[:2], drv, obj, "-L" + lib_dir, "-lek_hip", "-L/opt/rocm/lib", "-lamdhip64",
+         "-Wl,-rpath," + lib_dir, "-Wl,-rpath,/opt/rocm/lib", "-o", exe])
+    got = subprocess.run([exe, "300000"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert got.returncode == 0, got.stdout[-3000:]
+    ok, bad = (int(f.split("=")[1]) for f in got.stdout.split()[-2:])
+    assert ok > 1000 and bad > 100000
+    shutil.rmtree(tmp_path, ignore_errors=True)
