@@ -93,11 +93,18 @@ __global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
     const int e = threadIdx.x;
     int32_t total = 0;
     if (e < a.E) {
-        for (int b = 0; b < a.nblocks; ++b) {
-            const int64_t idx = (int64_t)b * a.E + e;
-            const int32_t t = a.block_hist[idx];
-            a.block_hist[idx] = total;   // exclusive prefix over chunks
-            total += t;
+        // exclusive prefix over chunks, 16 chunks' counts in flight at a time (one dependent load
+        // per chunk made this kernel's time: 10 us at 9 chunks)
+        for (int b0 = 0; b0 < a.nblocks; b0 += 16) {
+            int32_t v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                v[u] = b0 + u < a.nblocks ? a.block_hist[(int64_t)(b0 + u) * a.E + e] : 0;
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                if (b0 + u < a.nblocks) a.block_hist[(int64_t)(b0 + u) * a.E + e] = total;
+                total += v[u];
+            }
         }
         a.counts[e] = total;
         if (a.activation) a.activation[e] += (uint64_t)total;
@@ -353,8 +360,11 @@ void launch_pack(const PackArgs &a, hipStream_t s)
     }
     int nbits = 0;
     while ((1 << nbits) < a.E) ++nbits;
-    if (a.P <= kPackFusedMax) {
-        const size_t lds_bytes = sizeof(int32_t) * (16 * (size_t)a.E + 32);
+    // the one-workgroup form keeps 16 histograms in dynamic LDS: up to 64 KiB of it (E <= 1022).
+    // (One workgroup for longer calls was measured and is slower, 85 against 43 us at 65536 pairs:
+    // a single CU's memory pipeline then takes every scattered store of perm and row_token.)
+    const size_t lds_bytes = sizeof(int32_t) * (16 * (size_t)a.E + 32);
+    if (a.P <= kPackFusedMax && lds_bytes <= 65536) {
         hipLaunchKernelGGL(pack_fused_kernel, dim3(1), dim3(1024), lds_bytes, s, a, nbits);
         return;
     }

@@ -138,7 +138,8 @@ def oracle_weights(oracle, ws, E, dt=torch.bfloat16):
 # ----------------------------------------------------------------- routing
 
 PACK_CASES = [(0, 2, 16), (1, 1, 1), (1, 8, 256), (63, 1, 3), (64, 2, 16), (65, 3, 5), (128, 8, 256), (256, 8, 128),
-              (511, 8, 128), (513, 8, 1000), (4099, 2, 33), (8192, 8, 256)]
+              (511, 8, 128), (513, 8, 1000), (4099, 2, 33), (8192, 8, 256),
+              (8, 8, 1024), (500, 8, 1024), (4000, 8, 1022), (1100, 8, 1000), (8192, 7, 300), (8193, 8, 64), (20000, 4, 128)]
 
 
 @pytest.mark.parametrize("T,K,E", PACK_CASES)
@@ -546,20 +547,23 @@ def test_error_paths(ek, cuda):
     layer.close()                                               # idempotent
 
 
-def test_error_word_large_calls(ek, cuda):
-    """Calls too long for the single-workgroup pack (more than 4096 pairs): one bad pair among
-    thousands is reported, and the next good call is clean (the word is written per call)."""
+@pytest.mark.parametrize("tokens", [3000, 40000])
+def test_error_word_large_calls(ek, cuda, tokens):
+    """Calls too long for the single-workgroup pack (more than 4096 pairs; the second size has several
+    chunks per kernel): one bad pair among thousands is reported, and the next good call is clean
+    (the word is written per call)."""
     from ek_hip import _capi as C
-    w = wl.Workload("t", 128, 64, 8, 2, 3000, torch.bfloat16)
+    w = wl.Workload("t", 128, 64, 8, 2, tokens, torch.bfloat16)
     layer, ws = load_layer(ek, w, experts=[0, 1, 2, 3])
     g = torch.Generator().manual_seed(4)
     x = torch.randn(w.tokens, 128, generator=g).to(torch.bfloat16).to(cuda)
     gw = torch.full((w.tokens, 2), 0.5).to(torch.bfloat16).to(cuda)
     ok_ids = torch.stack([torch.randperm(4, generator=g)[:2] for _ in range(w.tokens)]).to(torch.int32).to(cuda)
     y0 = layer.forward(x, ok_ids, gw)
-    for bad, status in ((8, C.EK_INVALID_INPUT), (-1, C.EK_INVALID_INPUT), (7, C.EK_EXPERT_NOT_FOUND)):
+    for bad, status in ((8, C.EK_INVALID_INPUT), (-1, C.EK_INVALID_INPUT), (-2, C.EK_INVALID_INPUT),
+                        (-(1 << 31), C.EK_INVALID_INPUT), (7, C.EK_EXPERT_NOT_FOUND)):
         ids = ok_ids.clone()
-        ids[2999, 1] = bad
+        ids[tokens - 1, 1] = bad
         with pytest.raises(ek.EKError) as ei:
             layer.forward(x, ids, gw)
         assert ei.value.status == status, bad
