@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <mutex>
 #include <memory>
 #include <new>
@@ -188,6 +189,14 @@ struct ek_chain {
     int32_t *d_err = nullptr;                // [L] per-layer routing error words, gathered
     int32_t *h_err = nullptr;                // pinned
     hipStream_t stream = nullptr;
+    // Every layer's ids are the caller's, known when the call starts: the routing halves of layers
+    // 1 .. L-1 (pack and work lists, ~50 us each on a stream where they wait their turn) run on
+    // route_stream from the start of the call, beside layer 0's kernels; layer l waits for
+    // ev_routed[l].  Only when the layers are L different objects (each has its own workspace).
+    hipStream_t route_stream = nullptr;
+    hipEvent_t ev_begin = nullptr;
+    std::vector<hipEvent_t> ev_routed;
+    bool distinct = false;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     // key of the captured graph
@@ -1024,9 +1033,48 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
     return EK_OK;
 }
 
+// How a call's shared-expert segment (if the layer has one) is cut.
+struct SharedCut {
+    bool shared, streamed, wide;
+};
+SharedCut shared_cut(const ek_layer *L, int64_t T)
+{
+    SharedCut c;
+    c.shared = L->expert_mem[L->cfg.n_experts] != nullptr && T > 0;
+    c.streamed = c.shared && T <= kSharedStreamRows;
+    c.wide = c.shared && !c.streamed && T <= kSharedWideRows;
+    return c;
+}
+
+// The routing half of a layer call on stream s: pack, and the shared expert's segment appended to
+// its work lists.  It reads nothing but the ids, so a chain may run it ahead of the layer's turn.
+ek_status enqueue_route(ek_layer *L, const Workspace &W, const int32_t *ids, int64_t T, hipStream_t s)
+{
+    const int E = L->cfg.n_experts;
+    const int64_t P = T * L->cfg.top_k;
+    ek::launch_pack(pack_args(L, W, ids, P, true), s);
+    const SharedCut sc = shared_cut(L, T);
+    if (sc.wide) {
+        ek::WorkLists own = W.lists;
+        own.items[ek::kListStream] = W.wide_items;
+        own.count = W.wide_count;
+        ek::launch_append_segment(own, E, (int32_t)P, (int32_t)T, W.row_token, 2, s);
+    } else if (sc.shared) {
+        ek::launch_append_segment(W.lists, E, (int32_t)P, (int32_t)T, W.row_token, sc.streamed ? 1 : 0, s);
+    }
+    EK_HIP(hipGetLastError());
+    return EK_OK;
+}
+
 // pack -> stage 1 -> stage 2 -> combine on stream s; all pointers are device.
+// routed: enqueue_route for these ids has been enqueued already (s waits for it).
+// before_combine: called between the FFN launches and the combine (a chain enqueues the later
+// layers' routing halves and waits for the next layer's there: the wait costs nothing at that
+// point, and the next layer's first kernel then depends on nothing but this layer's combine in
+// its own queue).
 ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const int32_t *ids, const void *w, int w_f32,
-                          int64_t T, void *y, hipStream_t s)
+                          int64_t T, void *y, hipStream_t s, bool routed = false,
+                          const std::function<ek_status()> *before_combine = nullptr)
 {
     const int64_t H = L->cfg.hidden;
     const int E = L->cfg.n_experts, K = L->cfg.top_k;
@@ -1037,24 +1085,15 @@ ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const 
         L->events_used += 5;
     }
     if (ev) EK_HIP(hipEventRecord(ev[0], s));
-    ek::launch_pack(pack_args(L, W, ids, P, true), s);
-    // the shared expert is one more segment: every token once, rows P .. P+T-1 of the packed buffers
-    const bool shared = L->expert_mem[E] != nullptr && T > 0;
+    if (!routed) EK_TRY(enqueue_route(L, W, ids, T, s));
+    // the shared expert is one more segment: every token once, rows P .. P+T-1 of the packed buffers.
     // As tiles a decode-sized shared segment would occupy 8 to 14 CUs for the length of the whole
     // contraction.  Up to kSharedStreamRows tokens it is cut into 16-row streaming items
     // (measured on the DeepSeek-V3 shape at 64 tokens: 1.62 ms against 1.76 ms as a tile); each
     // item re-reads the expert's weights, so beyond that it is cut into items of up to 64 rows,
     // which the streaming kernel's wide form takes in a launch of its own.
-    const bool shared_streamed = shared && T <= kSharedStreamRows;
-    const bool shared_wide = shared && !shared_streamed && T <= kSharedWideRows;
-    if (shared_wide) {
-        ek::WorkLists own = W.lists;
-        own.items[ek::kListStream] = W.wide_items;
-        own.count = W.wide_count;
-        ek::launch_append_segment(own, E, (int32_t)P, (int32_t)T, W.row_token, 2, s);
-    } else if (shared) {
-        ek::launch_append_segment(W.lists, E, (int32_t)P, (int32_t)T, W.row_token, shared_streamed ? 1 : 0, s);
-    }
+    const SharedCut sc = shared_cut(L, T);
+    const bool shared = sc.shared, shared_streamed = sc.streamed, shared_wide = sc.wide;
     if (ev) EK_HIP(hipEventRecord(ev[1], s));
     if (P > 0) {
         const bool in_lists = shared && !shared_wide;   // the shared segment's items sit in the routed pairs' lists
@@ -1062,14 +1101,18 @@ ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const 
                            shared_streamed ? (T + 15) / 16 : 0,
                            shared_wide ? (T + ek::kWideRows - 1) / ek::kWideRows : 0));
         if (ev) EK_HIP(hipEventRecord(ev[3], s));
+        if (before_combine) EK_TRY((*before_combine)());
         ek::CombineArgs c;
         c.yp = W.yp; c.inv_perm = W.inv_perm; c.w = w; c.y = y; c.T = T; c.K = K; c.H = H;
         c.act = L->act; c.w_f32 = w_f32;
         c.shared = shared ? (const char *)W.yp + (size_t)P * H * 2 : nullptr;
         ek::launch_combine(c, s);
-    } else if (ev) {
-        EK_HIP(hipEventRecord(ev[2], s));
-        EK_HIP(hipEventRecord(ev[3], s));
+    } else {
+        if (ev) {
+            EK_HIP(hipEventRecord(ev[2], s));
+            EK_HIP(hipEventRecord(ev[3], s));
+        }
+        if (before_combine) EK_TRY((*before_combine)());
     }
     if (ev) EK_HIP(hipEventRecord(ev[4], s));
     EK_HIP(hipGetLastError());
@@ -1733,6 +1776,9 @@ static void free_chain(ek_chain *c)
     if (c->d_err) (void)hipFree(c->d_err);
     if (c->h_err) (void)hipHostFree(c->h_err);
     if (c->stream) (void)hipStreamDestroy(c->stream);
+    if (c->route_stream) (void)hipStreamDestroy(c->route_stream);
+    if (c->ev_begin) (void)hipEventDestroy(c->ev_begin);
+    for (hipEvent_t e : c->ev_routed) if (e) (void)hipEventDestroy(e);
     delete c;
 }
 
@@ -1771,6 +1817,16 @@ ek_status ek_chain_create(ek_layer *const *layers, int32_t n_layers, ek_chain **
         if (st == EK_OK) {
             hipError_t e = hipHostMalloc((void **)&c->h_err, sizeof(int32_t) * n_layers, hipHostMallocDefault);
             if (e == hipSuccess) e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+            std::vector<ek_layer *> uniq(c->layers);
+            std::sort(uniq.begin(), uniq.end());
+            c->distinct = std::adjacent_find(uniq.begin(), uniq.end()) == uniq.end();
+            if (c->distinct && n_layers > 1) {
+                if (e == hipSuccess) e = hipStreamCreateWithFlags(&c->route_stream, hipStreamNonBlocking);
+                if (e == hipSuccess) e = hipEventCreateWithFlags(&c->ev_begin, hipEventDisableTiming);
+                c->ev_routed.assign(n_layers, nullptr);
+                for (int i = 1; i < n_layers && e == hipSuccess; ++i)
+                    e = hipEventCreateWithFlags(&c->ev_routed[i], hipEventDisableTiming);
+            }
             if (e != hipSuccess) st = hip_fail(e, "chain setup");
         }
         if (st != EK_OK) {
@@ -1796,13 +1852,36 @@ static ek_status enqueue_chain(ek_chain *c, const void *x, const int32_t *ids, c
         EK_TRY(rows_in(c->layers[0], c->act_in, x, T, EK_DEVICE, s));
         in = c->act_in;
     }
+    const bool ahead = c->route_stream != nullptr && T > 0;
+    if (ahead) {
+        // layer 0's routing half first, alone
+        EK_TRY(enqueue_route(c->layers[0], c->layers[0]->ws, ids, T, s));
+        EK_HIP(hipEventRecord(c->ev_begin, s));
+    }
     for (int l = 0; l < L; ++l) {
         void *outp = l == L - 1 && !c->act_in ? y : c->act[l & 1];
         ek_layer *ly = c->layers[l];
+        // Between layer l's FFN launches and its combine: (l = 0) the other layers' routing halves go
+        // to their own stream behind layer 0's, where they run in what layer 0's kernels leave free
+        // of the chip (enqueued after layer 0's FFN kernels, so that under capture the tile kernel
+        // stays the first successor of layer 0's pack and follows it in its queue); then s
+        // waits for layer l + 1's.
+        const std::function<ek_status()> mid = [&]() -> ek_status {
+            if (l == 0) {
+                EK_HIP(hipStreamWaitEvent(c->route_stream, c->ev_begin, 0));
+                for (int m = 1; m < L; ++m) {
+                    EK_TRY(enqueue_route(c->layers[m], c->layers[m]->ws, ids + (size_t)m * T * K, T, c->route_stream));
+                    EK_HIP(hipEventRecord(c->ev_routed[m], c->route_stream));
+                }
+            }
+            if (l + 1 < L) EK_HIP(hipStreamWaitEvent(s, c->ev_routed[l + 1], 0));
+            return EK_OK;
+        };
         const bool prof = ly->profiling;
         ly->profiling = false;               // no event records inside a chain (capture-safe)
         ek_status st = enqueue_forward(ly, ly->ws, in, ids + (size_t)l * T * K,
-                                       (const char *)w + (size_t)l * T * K * w_es, w_f32, T, outp, s);
+                                       (const char *)w + (size_t)l * T * K * w_es, w_f32, T, outp, s, ahead,
+                                       ahead ? &mid : nullptr);
         ly->profiling = prof;
         EK_TRY(st);
         // collect the layer's error word with a copy kernel-free D2D memcpy node

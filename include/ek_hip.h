@@ -439,6 +439,10 @@ ek_status ek_layer_forward_logits(ek_layer *layer, const void *x, const void *lo
  *   layers [L]: same hidden / top_k / act_dtype / device; each keeps its own
  *               experts and workspace and must outlive the chain
  *   ids [L,T,K] int32, w [L,T,K] w_dtype, x [T,H] -> y [T,H]; device pointers.
+ * All L layers' ids are the caller's and known when the call starts, so when the
+ * layers are L different objects the pack steps of layers 1 .. L-1 run on a
+ * stream of their own beside layer 0's kernels instead of between two layers
+ * (a layer named twice shares one workspace between its steps: no running ahead).
  * use_graph = 0 runs the same launches eagerly (the reference for graph tests).
  * A graph is re-captured when T, a pointer or w_dtype changes.  stream as in
  * ek_layer_forward (NULL = blocking on the library's stream); routing errors

@@ -77,6 +77,28 @@ def test_chain_small_vs_layers_and_oracle(ek, oracle, cuda):
         layer.close()
 
 
+def test_chain_with_a_layer_used_twice(ek, cuda):
+    """A chain may name one layer object more than once (tied weights).  Its workspace is then used
+    by two steps of the chain, so the chain must not run those steps' routing ahead of their turn
+    (it does for chains of distinct layers); eager and graph results equal the layer-by-layer calls."""
+    w0 = wl.Workload("ragged_x3", 256, 128, 16, 4, 0, torch.float16, zipf_s=1.2, n_layers=3, ragged=True)
+    w0 = wl.Workload(**{**w0.__dict__, "tokens": 90})
+    w, layers, weights, ids, gw = build_chain(ek, w0, cuda, std=0.08)
+    order = [layers[0], layers[1], layers[0]]
+    xd = wl.make_x(w).to(cuda)
+    cur = xd
+    for l, layer in enumerate(order):
+        cur = layer.forward(cur, ids[l].contiguous(), gw[l].contiguous())
+    chain = ek.HipChain(order)
+    assert torch.equal(bits(chain.forward(xd, ids, gw, use_graph=False)), bits(cur))
+    for rep in range(3):
+        assert torch.equal(bits(chain.forward(xd, ids, gw, use_graph=True)), bits(cur)), f"replay {rep}"
+        torch.cuda.synchronize()
+    chain.close()
+    for layer in layers:
+        layer.close()
+
+
 def test_chain_c5_full_shape_properties(ek, cuda):
     """Qwen3 shape, 128 experts, top-8, 4 layers, 48 requests (40 decode + 8 prefill chunks):
     too large for the oracle, so the chain is checked through properties that do not
