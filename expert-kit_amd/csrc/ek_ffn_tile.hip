@@ -34,8 +34,8 @@
 // channels per wave: the figures above) and narrow (one column block per wave, so half the
 // channels per workgroup and twice the workgroups per item, three stages with 16-bit weights
 // too) for launches whose tiles would leave most of the chip idle.  Every output element is the
-// same sum in the same order in both.  In the wide form the 32- and 64-row items of layers with
-// one-byte weights take a third path, run_mid below: weights from HBM straight into registers.
+// same sum in the same order in both.  In the wide form the 32- and 64-row items of a launch whose
+// tiles fill the chip take a third path, run_mid below: weights from HBM straight into registers.
 #include "ek_internal.h"
 #include "ek_mfma.h"
 
