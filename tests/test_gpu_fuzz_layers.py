@@ -1,0 +1,63 @@
+"""Forty seeded draws of a whole layer call: weight kind (16-bit, int8 per channel, fp8 / int8 with
+128 x 128 block scales), activation type, hidden and intermediate size, expert count, top-k, token
+count from a handful to a few thousand, and the routing's shape (uniform, a few hot experts, a
+power law), so that segments of every class and both kernel families meet in combinations the
+hand-picked cases do not list.  Each call is held to the oracle's layer (pack tables bit for bit,
+outputs by the layer gate; arithmetic of ek-computation/src/ffn/expert_torch.rs:81-84 and
+expertkit_torch/models/qwen3_moe.py:102-104) and to the same call on host tensors.
+EKSEED=n draws another forty."""
+import os
+import pytest
+import torch
+from ek_hip import workloads as wl
+from test_gpu_block_scaled import KINDS, make_expert as make_block_expert, ref_weights
+from test_gpu_parity import layer_gate, oracle_weights
+
+pytestmark = pytest.mark.gpu
+SEED = int(os.environ.get("EKSEED", "0"))
+
+
+@pytest.mark.parametrize("case", range(40))
+def test_fuzz(ek, oracle, cuda, case):
+    g = torch.Generator().manual_seed(SEED * 1000 + case)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    kind = ["w16", "i8", "fp8", "int8"][r(0, 3)]
+    dt = [torch.bfloat16, torch.float16][r(0, 1)]
+    step = 64 if kind == "w16" else 128
+    H, I = step * r(1, 8), step * r(1, 6)
+    E, K = r(1, 40), r(1, 4)
+    K = min(K, E)
+    T = [r(1, 8), r(9, 80), r(81, 700), r(701, 2500)][r(0, 3)]
+    skew = r(0, 2)
+    print(f"fuzz seed={SEED} case={case} kind={kind} dt={dt} H={H} I={I} E={E} K={K} T={T} skew={skew}", flush=True)
+    if kind in KINDS:
+        layer = ek.HipLayer(H, I, E, K, act_dtype=dt, max_tokens=T, **KINDS[kind])
+        ws = [make_block_expert(ek, H, I, 100 * case + e, kind) for e in range(min(E, 6))]
+        ref_w = [ref_weights(oracle, ew, dt) for ew in ws]
+    else:
+        w = wl.Workload("t", H, I, E, K, T, dt, w8=kind == "i8")
+        layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=torch.int8 if w.w8 else dt, max_tokens=T)
+        ws = [wl.make_expert(w, 100 * case + e) for e in range(min(E, 6))]
+        if kind == "w16":
+            ws = [ek.ExpertWeight(ew.up_w * 3, ew.gate_w * 3, ew.down_w * 3) for ew in ws]
+        cols = oracle_weights(oracle, dict(enumerate(ws)), len(ws), dt)
+        ref_w = [tuple(c[i] for c in cols) for i in range(len(ws))]
+    for e in range(E):
+        layer.set_expert(e, ws[e % len(ws)])
+    p = torch.ones(E)
+    if skew == 1:
+        p[: max(1, E // 8)] = 20.0
+    elif skew == 2:
+        p = 1.0 / torch.arange(1, E + 1).float() ** 1.3
+    ids = torch.stack([torch.multinomial(p, K, generator=g) for _ in range(T)]).to(torch.int32)
+    gw = torch.rand(T, K, generator=g) + 0.1
+    gw = (gw / gw.sum(-1, keepdim=True)).to(dt)
+    x = torch.randn(T, H, generator=g).to(dt)
+    wu, wg, wd = zip(*[ref_w[e % len(ws)] for e in range(E)])
+    ref, counts, offsets, perm, inv, y3 = oracle.layer_forward(x, ids, gw, list(wu), list(wg), list(wd), mode=2, return_y3=True)
+    y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
+    assert torch.equal(rt.perm.cpu(), perm) and torch.equal(rt.counts.cpu(), counts)
+    layer_gate(y, ref, y3, gw, f"fuzz {case}", plain=False)
+    y2 = layer.forward(x, ids, gw)
+    assert torch.equal(y2.view(torch.int16), y.cpu().view(torch.int16))
+    layer.close()
