@@ -1,0 +1,56 @@
+"""Thirty seeded draws of the per-expert contract (one expert per call, [n, H] -> [n, H]:
+ek-computation/src/worker/core.rs:47-74): weight kind, activation type, sizes, and a handful of calls
+of 1 to 2600 rows, so that the streaming kernel's three forms, the wide cut, the narrow and the wide
+tile form are met at sizes around their thresholds.  Every call alone, and all of them in one grouped
+launch, against the oracle's FFN (ek-computation/src/ffn/expert_torch.rs:81-84).
+EKSEED=n draws another thirty."""
+import os
+import pytest
+import torch
+from ek_hip import workloads as wl
+from test_gpu_block_scaled import KINDS, make_expert as make_block_expert, ref_weights
+from test_gpu_parity import ffn_gate, oracle_weights
+
+pytestmark = pytest.mark.gpu
+SEED = int(os.environ.get("EKSEED", "0"))
+
+
+@pytest.mark.parametrize("case", range(30))
+def test_fuzz(ek, oracle, cuda, case):
+    g = torch.Generator().manual_seed(SEED * 1000 + case + 77)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    kind = ["w16", "i8", "fp8", "int8"][r(0, 3)]
+    dt = [torch.bfloat16, torch.float16][r(0, 1)]
+    step = 64 if kind == "w16" else 128
+    H, I = step * r(1, 10), step * r(1, 6)
+    E = 4
+    sizes = [[r(1, 16), r(17, 64), r(65, 200)][r(0, 2)] for _ in range(r(1, 6))] + [[r(200, 900), r(900, 2600)][r(0, 1)]]
+    print(f"fuzz-expert seed={SEED} case={case} kind={kind} dt={dt} H={H} I={I} sizes={sizes}", flush=True)
+    mt = max(sum(sizes), 1)
+    if kind in KINDS:
+        layer = ek.HipLayer(H, I, E, 1, act_dtype=dt, max_tokens=mt, **KINDS[kind])
+        ws = [make_block_expert(ek, H, I, 100 * case + e, kind) for e in range(E)]
+        ref_w = [ref_weights(oracle, ew, dt) for ew in ws]
+    else:
+        w = wl.Workload("t", H, I, E, 1, mt, dt, w8=kind == "i8")
+        layer = ek.HipLayer(H, I, E, 1, act_dtype=dt, w_dtype=torch.int8 if w.w8 else dt, max_tokens=mt)
+        ws = [wl.make_expert(w, 100 * case + e) for e in range(E)]
+        if kind == "w16":
+            ws = [ek.ExpertWeight(ew.up_w * 3, ew.gate_w * 3, ew.down_w * 3) for ew in ws]
+        cols = oracle_weights(oracle, dict(enumerate(ws)), E, dt)
+        ref_w = [tuple(c[i] for c in cols) for i in range(E)]
+    for e in range(E):
+        layer.set_expert(e, ws[e])
+    xs = [torch.randn(n, H, generator=g).to(dt) for n in sizes]
+    es = [r(0, E - 1) for _ in sizes]
+    # alone
+    alone = []
+    for e, x in zip(es, xs):
+        got = layer.expert_forward(e, x.to(cuda))
+        ffn_gate(got, oracle.ffn(x, *ref_w[e], mode=2), f"fuzz-expert {case} n={x.shape[0]}", plain=False, small=2)
+        alone.append(got)
+    # grouped: one launch for all of them; rows alone and grouped differ at most by accumulation order
+    outs = layer.experts_forward(es, [x.to(cuda) for x in xs])
+    for e, x, o in zip(es, xs, outs):
+        ffn_gate(o, oracle.ffn(x, *ref_w[e], mode=2), f"fuzz-expert grouped {case} n={x.shape[0]}", plain=False, small=2)
+    layer.close()
