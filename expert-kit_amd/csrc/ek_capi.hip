@@ -991,8 +991,18 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
     const bool have_tiles = cap[ek::kListT32] + cap[ek::kListT64] + cap[ek::kListT128] > 0;
     const bool small_expert = 3 * H * I * (L->w8 ? 1 : 2) <= (16ll << 20);
     const bool tiles_lately = exact ? true : ((volatile int32_t *)L->h_err)[1] > 0;   // (exact: have_tiles says it)
+    // Above 4 pairs per expert tiles are the rule; but when the last call cut none at all, this one's
+    // tile launches will most likely find empty lists too, and the fork's event records and waits are
+    // host time (~30 us of a 57 us call of 64 tokens on 16 small experts).  Not under capture: what is
+    // recorded there is replayed for other routings, and the sizes decide alone.
+    bool capturing = false;
+    if (P > 4 * E && !tiles_lately) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cs) != hipSuccess) (void)hipGetLastError();
+        capturing = cs != hipStreamCaptureStatusNone;
+    }
     const bool fork = have_stream && have_tiles &&
-                      (P > 4 * E ? P <= 128 * E || small_expert : tiles_lately);
+                      (P > 4 * E ? (P <= 128 * E || small_expert) && (tiles_lately || capturing) : tiles_lately);
     hipStream_t s_stream = s, s_tiles = s;
     hipStream_t side = nullptr;
     if (fork || shared_wide > 0) {
