@@ -71,7 +71,7 @@ def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
     sample = set(ws_sample)
     times, pairs = [], 0
     t_all = time.time()
-    while len(times) < 5 and (time.time() - t_all < target_s or not times):
+    while len(times) < 15 and (time.time() - t_all < target_s or not times):
         t0 = time.time()
         _, pairs = oracle.torch_layer_forward(x, ids, gw, wu, wg, wd, experts=sample)
         times.append(time.time() - t0)
@@ -283,7 +283,7 @@ def main():
                     help="fp8: the c3 / c4 layer with fp8 e4m3fn weights and 128x128 block scales kept as a "
                          "DeepSeek-V3 checkpoint stores them, instead of the configuration's int8 per channel; "
                          "bf16: the same layer with 16-bit weights")
-    ap.add_argument("--cpu-experts", type=int, default=24, help="experts in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--cpu-experts", type=int, default=96, help="experts in the CPU-baseline sample (0 = skip)")
     ap.add_argument("--tokens", type=int, default=0,
                     help="run the workload's layer at another token count (a parity-test style variation, e.g. other "
                          "decode batch sizes of c3; implies --no-prefill)")
