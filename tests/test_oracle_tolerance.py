@@ -144,3 +144,68 @@ def test_accumulation_order_moves_outputs_by_more_than_half_an_ulp(oracle):
         print(f"seed {seed}: libtorch vs y_ref max|err|/rms = {float(err.max()) / rms:.3e}")
     assert over_plain >= 6, over_plain
     assert over_half >= 1, "no seed showed a flipped intermediate at a large term"
+
+
+def test_a_tie_in_a_hidden_activation_moves_one_ffn_output_by_two_ulps(oracle):
+    """One expert's FFN alone (fp8 weights with block scales, 896 -> 512 -> 896, a case the seeded
+    fuzz of per-expert calls drew: EKSEED=8, case 23, row 1106, output channel 175).  The gate
+    pre-activation of hidden channel 350 is 1.37890641: 1.6e-7 above the midpoint of the bf16
+    neighbours 1.375 and 1.3828125.  The oracle's double sum and a sequential fp32 sum store
+    1.3828125; an fp32 sum kept as eight interleaved partial sums, as legitimate an evaluation of
+    x.matmul(w3.T) (ffn/expert_torch.rs:82), lands on the midpoint and stores 1.375.  silu and the
+    product with `up` turn that one ulp into two ulps of h, that hidden channel carries 92 % of
+    the output, and the output moves by 2.9e-2 * rms: past 2e-2 * rms plus half an output ulp,
+    the one-expert gate of the GPU tests.  Nothing in it is an error; the GPU kernels' MFMA
+    order lands on the 1.375 side."""
+    import ek_hip
+    from test_gpu_block_scaled import make_expert as make_block_expert, ref_weights
+    dt, H, I, case, row, col, j = torch.bfloat16, 896, 512, 23, 1106, 175, 350
+    g = torch.Generator().manual_seed(8 * 1000 + case + 77)
+    draws = [int(torch.randint(lo, hi + 1, (1,), generator=g)) for lo, hi in ((0, 3), (0, 1), (1, 10), (1, 6))]
+    assert draws == [2, 0, 7, 4]                      # fp8, bf16, 7 x 128, 4 x 128: the generator stream of the fuzz
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    sizes = [[r(1, 16), r(17, 64), r(65, 200)][r(0, 2)] for _ in range(r(1, 6))] + [[r(200, 900), r(900, 2600)][r(0, 1)]]
+    assert sizes == [171, 3, 1898]
+    ws = [make_block_expert(ek_hip, H, I, 100 * case + e, "fp8") for e in range(4)]
+    xs = [torch.randn(n, H, generator=g).to(dt) for n in sizes]
+    es = [r(0, 3) for _ in sizes]
+    wu, wg, wd = ref_weights(oracle, ws[es[-1]], dt)
+    x = xs[-1][1024:1152]                              # the 128-row work item that holds the row
+    ref = oracle.ffn(x, wu, wg, wd, mode=2)
+    rms = float(ref.pow(2).mean().sqrt())
+    xr = x[row - 1024].float()
+
+    def interleaved8(w_row):                           # eight running fp32 sums over k mod 8, then added in order
+        parts = torch.zeros(8, dtype=torch.float32)
+        for k in range(0, H, 8):
+            parts = parts + w_row[k:k + 8] * xr[k:k + 8]
+        tot = torch.zeros((), dtype=torch.float32)
+        for p in parts:
+            tot = tot + p
+        return tot
+
+    seq = torch.zeros((), dtype=torch.float32)
+    for k in range(H):
+        seq = seq + wg[j].float()[k] * xr[k]
+    alt = interleaved8(wg[j].float())
+    assert abs(float(seq) - float(alt)) < 1e-6 and float(alt) == 1.37890625
+    assert float(seq.to(dt)) == 1.3828125 and float(alt.to(dt)) == 1.375
+
+    def out_with(gate_b):                              # the reference's rounding points from the stored gate value on
+        up_b = (wu.double() @ xr.double()).float().to(dt)
+        gates = (wg.double() @ xr.double()).float().to(dt)
+        gates[j] = gate_b
+        silu_b = torch.nn.functional.silu(gates.float()).to(dt)
+        h = (up_b.float() * silu_b.float()).to(dt)
+        return float(h.double() @ wd[col].double())
+
+    a, b = out_with(1.3828125), out_with(1.375)
+    assert abs(a - float(ref[row - 1024, col])) < 1e-6             # the oracle's side of the tie
+    stored = float(torch.tensor(b).to(dt))                          # what an implementation on that side writes
+    moved = abs(stored - float(ref[row - 1024, col]))
+    half_ulp = 0.5 * float(ulp_of(ref[row - 1024, col], dt))
+    print(f"tie in gate[{j}]: output {a:.6f} -> {b:.6f}, stored {stored:.6f}: {moved / rms:.3e} x rms, "
+          f"{moved / (2 * half_ulp):.2f} output ulps from y_ref")
+    assert stored == -0.359375                                      # the value the GPU kernels write
+    assert moved > TOL * rms + half_ulp
+    assert moved < 1.6 * TOL * rms
