@@ -1024,7 +1024,10 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
         const bool tiles_first = fork;
         const int64_t wgs_per_item = (a.N + ek::tile_channels(stage, false) - 1) / ek::tile_channels(stage, false);
-        const bool narrow = known_tile_items > 0 && known_tile_items * wgs_per_item <= 128;
+        // (the narrow form runs three stages deep also with 16-bit weights, i.e. starts a tile with the
+        // loads of its first two steps: a contraction of one 64-element step has no second one, and
+        // the load would read past the last row of x and past the expert's last weight chunk)
+        const bool narrow = known_tile_items > 0 && known_tile_items * wgs_per_item <= 128 && a.Kdim >= 128;
         if (tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, narrow, s_tiles));
         if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, cap[ek::kListStream], false, s_stream));
         if (shared_wide > 0) {

@@ -900,6 +900,9 @@ static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, const int64_t
 hipError_t launch_ffn_tile(const FfnArgs &a, int stage, int act, int wmode,
                            const int64_t max_items[kNumLists], bool narrow, hipStream_t s)
 {
+    // forms that run three stages deep issue a tile's first two steps up front: the contraction
+    // must have two (one-byte weights: hidden, inter >= 128 always; 16-bit: the narrow form)
+    if ((narrow || wmode != kW16) && a.Kdim < 128) return hipErrorInvalidValue;
     return act == 0 ? launch_w<__bf16>(a, stage, wmode, max_items, narrow, s)
                     : launch_w<_Float16>(a, stage, wmode, max_items, narrow, s);
 }

@@ -313,6 +313,23 @@ def test_tile_route_shortest_contractions(ek, oracle, cuda, H, I, w8):
     layer.close()
 
 
+@pytest.mark.parametrize("H,I", [(64, 128), (128, 64), (64, 64), (64, 320)])
+@pytest.mark.parametrize("n", [600, 1500])
+def test_one_step_contractions_in_a_per_expert_call(ek, oracle, cuda, H, I, n):
+    """16-bit weights and a contraction of a single 64-element step, in a per-expert call long enough
+    to be cut into tiles but too short to fill the chip: such a call must not take the tile kernel's
+    narrow form, which starts every tile with the loads of its first two steps (a second step's load
+    would read past the last row of x and past the expert's weights).  Held to the oracle."""
+    dt = torch.float16
+    w = wl.Workload("t", H, I, 2, 1, n, dt)
+    layer, ws = load_layer(ek, w, experts=[1])
+    wu, wg, wd = [t[1] for t in oracle_weights(oracle, ws, 2, dt)]
+    x = torch.randn(n, H, generator=torch.Generator().manual_seed(n + H)).to(dt)
+    got = layer.expert_forward(1, x.to(cuda))
+    ffn_gate(got, oracle.ffn(x, wu, wg, wd, mode=2), f"one-step contraction H={H} I={I} n={n}", plain=False)
+    layer.close()
+
+
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 def test_silu_of_every_16bit_gate_value(ek, oracle, cuda, dt):
     """All 65536 bit patterns of the activation type as the gate pre-activation, through both kernel
