@@ -1,0 +1,52 @@
+"""Fifteen seeded draws at the expert sizes of published models (DeepSeek-V3 7168 / 2048, Qwen3
+2048 / 768, DeepSeek-V2-Lite 2048 / 1408, and two more): weight kind, activation type and four
+calls of 1 to 520 rows, each alone, all grouped, and the same rows through the layer call, against the
+oracle's FFN (ek-computation/src/ffn/expert_torch.rs:81-84).  EKSEED=n draws another fifteen."""
+import os
+import pytest
+import torch
+from ek_hip import workloads as wl
+from test_gpu_block_scaled import KINDS, make_expert as make_block_expert, ref_weights
+from test_gpu_parity import ffn_gate, oracle_weights
+pytestmark = pytest.mark.gpu
+SEED = int(os.environ.get("EKSEED", "0"))
+SHAPES = [(7168, 2048), (2048, 768), (2048, 1408), (5120, 1536), (4096, 1024)]
+
+@pytest.mark.parametrize("case", range(15))
+def test_fuzz(ek, oracle, cuda, case):
+    g = torch.Generator().manual_seed(SEED * 1000 + case + 999)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    H, I = SHAPES[case % len(SHAPES)]
+    kind = ["w16", "i8", "fp8"][(case // len(SHAPES)) % 3]
+    if kind != "w16" and I % 128: kind = "w16"
+    dt = [torch.bfloat16, torch.float16][r(0, 1)]
+    sizes = [r(1, 16), r(17, 64), r(65, 200), r(201, 520)]
+    print(f"fuzz-model seed={SEED} case={case} kind={kind} dt={dt} H={H} I={I} sizes={sizes}", flush=True)
+    E = 2
+    if kind in KINDS:
+        layer = ek.HipLayer(H, I, E, 1, act_dtype=dt, max_tokens=sum(sizes), **KINDS[kind])
+        ws = [make_block_expert(ek, H, I, 100 * case + e, kind) for e in range(E)]
+        ref_w = [ref_weights(oracle, ew, dt) for ew in ws]
+    else:
+        w = wl.Workload("t", H, I, E, 1, sum(sizes), dt, w8=kind == "i8")
+        layer = ek.HipLayer(H, I, E, 1, act_dtype=dt, w_dtype=torch.int8 if w.w8 else dt, max_tokens=sum(sizes))
+        ws = [wl.make_expert(w, 100 * case + e) for e in range(E)]
+        cols = oracle_weights(oracle, dict(enumerate(ws)), E, dt)
+        ref_w = [tuple(c[i] for c in cols) for i in range(E)]
+    for e in range(E):
+        layer.set_expert(e, ws[e])
+    xs = [torch.randn(n, H, generator=g).to(dt) for n in sizes]
+    es = [r(0, E - 1) for _ in sizes]
+    refs = [oracle.ffn(x, *ref_w[e], mode=2) for e, x in zip(es, xs)]
+    for e, x, ref in zip(es, xs, refs):
+        ffn_gate(layer.expert_forward(e, x.to(cuda)), ref, f"fuzz-model {case} n={x.shape[0]}", plain=False, small=2)
+    for o, ref in zip(layer.experts_forward(es, [x.to(cuda) for x in xs]), refs):
+        ffn_gate(o, ref, f"fuzz-model grouped {case} n={ref.shape[0]}", plain=False, small=2)
+    xa = torch.cat(xs)
+    ids = torch.cat([torch.full((x.shape[0], 1), e, dtype=torch.int32) for e, x in zip(es, xs)])
+    y = layer.forward(xa.to(cuda), ids.to(cuda), torch.ones(xa.shape[0], 1, dtype=dt, device=cuda))
+    o0 = 0
+    for x, ref in zip(xs, refs):
+        ffn_gate(y[o0:o0 + x.shape[0]], ref, f"fuzz-model layer {case} n={x.shape[0]}", plain=False, small=2)
+        o0 += x.shape[0]
+    layer.close()
