@@ -60,6 +60,42 @@ __device__ __forceinline__ int32_t block_exclusive_scan(int32_t v, int32_t *wave
     return base + incl - v;
 }
 
+// The same for five ints per thread at once (one pair of barriers instead of five): the offsets
+// and the four work lists' positions of the one-workgroup pack.  wave_tot: [16][5].
+__device__ __forceinline__ void block_exclusive_scan5(const int32_t (&v)[5], int32_t (*wave_tot)[5],
+                                                      int32_t (&excl)[5], int32_t (&total)[5])
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int32_t incl[5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i) incl[i] = v[i];
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            const int32_t up = __shfl_up(incl[i], d, 64);
+            if (lane >= d) incl[i] += up;
+        }
+    }
+    __syncthreads();   // wave_tot may still be read from a previous scan
+    if (lane == 63) {
+#pragma unroll
+        for (int i = 0; i < 5; ++i) wave_tot[wave][i] = incl[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+        int32_t base = 0, sum = 0;
+        for (int w = 0; w < 16; ++w) {
+            const int32_t t = wave_tot[w][i];
+            if (w < wave) base += t;
+            sum += t;
+        }
+        total[i] = sum;
+        excl[i] = base + incl[i] - v[i];
+    }
+}
+
 // How one segment of n rows is cut into work items (see WorkLists).
 struct SegmentCut {
     int32_t n128, n64, n32, ns;
@@ -265,9 +301,9 @@ __global__ __launch_bounds__(kPackThreads) void pack_rank_kernel(PackArgs a, int
 constexpr int kPackFusedMax = 4096;
 __global__ __launch_bounds__(1024) void pack_fused_kernel(PackArgs a, int nbits)
 {
-    extern __shared__ int32_t lds[];          // wbase[16][E], then wave_tot[16], err
-    int32_t *wave_tot = lds + 16 * a.E;
-    int32_t *lerr = wave_tot + 16;
+    extern __shared__ int32_t lds[];          // wbase[16][E], then wave_tot5[16][5], err
+    int32_t (*wave_tot5)[5] = (int32_t (*)[5])(lds + 16 * a.E);
+    int32_t *lerr = lds + 16 * a.E + 80;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     constexpr int kIter = kPackFusedMax / 1024;   // 64-pair groups per wave
     for (int i = threadIdx.x; i < 16 * a.E; i += 1024) lds[i] = 0;
@@ -295,8 +331,12 @@ __global__ __launch_bounds__(1024) void pack_fused_kernel(PackArgs a, int nbits)
         if (a.activation) a.activation[e] += (uint64_t)total;
         if (total > 0 && a.slabs != nullptr && a.slabs[e].upgate == nullptr) atomicOr(lerr, 2);
     }
-    int32_t sum;
-    const int32_t off = block_exclusive_scan(total, wave_tot, &sum);
+    // offsets and the four lists' positions in one scan
+    const SegmentCut c = cut_segment(total);
+    const int32_t v5[5] = {total, c.n128, c.n64, c.n32, c.ns};
+    int32_t ex[5], tot5[5];
+    block_exclusive_scan5(v5, wave_tot5, ex, tot5);
+    const int32_t off = ex[0];
     if (e < a.E) {
         a.offsets[e] = off;
         int32_t run = off;
@@ -306,21 +346,15 @@ __global__ __launch_bounds__(1024) void pack_fused_kernel(PackArgs a, int nbits)
             run += t;
         }
     }
-    if (e == 0) a.offsets[a.E] = sum;
+    if (e == 0) a.offsets[a.E] = tot5[0];
     if (a.lists.count != nullptr) {
-        const SegmentCut c = cut_segment(total);
-        int32_t s128, s64, s32, ss;
-        const int32_t p128 = block_exclusive_scan(c.n128, wave_tot, &s128);
-        const int32_t p64 = block_exclusive_scan(c.n64, wave_tot, &s64);
-        const int32_t p32 = block_exclusive_scan(c.n32, wave_tot, &s32);
-        const int32_t ps = block_exclusive_scan(c.ns, wave_tot, &ss);
-        if (e < a.E && total > 0) emit_items(a.lists, e, off, total, p128, p64, p32, ps);
+        if (e < a.E && total > 0) emit_items(a.lists, e, off, total, ex[1], ex[2], ex[3], ex[4]);
         if (e == 0) {
-            a.lists.count[kListT128] = s128;
-            a.lists.count[kListT64] = s64;
-            a.lists.count[kListT32] = s32;
-            a.lists.count[kListStream] = ss;
-        if (a.tile_items_host) *a.tile_items_host = s128 + s64 + s32;
+            a.lists.count[kListT128] = tot5[1];
+            a.lists.count[kListT64] = tot5[2];
+            a.lists.count[kListT32] = tot5[3];
+            a.lists.count[kListStream] = tot5[4];
+            if (a.tile_items_host) *a.tile_items_host = tot5[1] + tot5[2] + tot5[3];
         }
     }
     __syncthreads();
@@ -360,10 +394,10 @@ void launch_pack(const PackArgs &a, hipStream_t s)
     }
     int nbits = 0;
     while ((1 << nbits) < a.E) ++nbits;
-    // the one-workgroup form keeps 16 histograms in dynamic LDS: up to 64 KiB of it (E <= 1022).
+    // the one-workgroup form keeps 16 histograms in dynamic LDS: up to 64 KiB of it (E <= 1018).
     // (One workgroup for longer calls was measured and is slower, 85 against 43 us at 65536 pairs:
     // a single CU's memory pipeline then takes every scattered store of perm and row_token.)
-    const size_t lds_bytes = sizeof(int32_t) * (16 * (size_t)a.E + 32);
+    const size_t lds_bytes = sizeof(int32_t) * (16 * (size_t)a.E + 96);
     if (a.P <= kPackFusedMax && lds_bytes <= 65536) {
         hipLaunchKernelGGL(pack_fused_kernel, dim3(1), dim3(1024), lds_bytes, s, a, nbits);
         return;
