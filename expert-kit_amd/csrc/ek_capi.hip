@@ -341,10 +341,16 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     A((void **)&L->ws.wide_items, sizeof(ek::WorkItem) * kSharedWideItems, "shared expert's work list");
     A((void **)&L->ws.wide_count, sizeof(int32_t) * ek::kNumLists, "shared expert's work list count");
     for (int l = 0; l < ek::kNumLists; ++l) {
-        // the per-expert entry point cuts one segment of up to pmax rows: capacity for E = 1 too
-        // (and the wide cut, see wide_cut_pays: fewer than 128 tile items of at most 128 rows
-        // become at most two streaming items each)
-        const int64_t cap = ek::list_capacity(l, rows_max, E + 1) + (l == ek::kListStream ? 264 : 1);
+        // A layer call's lists hold at most one remainder item per expert (list_capacity); a grouped
+        // launch of per-expert calls may name an expert many times, each call a segment of its own,
+        // so this workspace's lists are sized by rows alone: rows_max / 17 items of 17..32 rows, and
+        // so on (16 bytes an item).  The streaming list also takes the wide cut's items (see
+        // wide_cut_pays: fewer than 128 tile items of at most 128 rows become at most two streaming
+        // items each) and is bounded by what one launch's grid can number.
+        const int64_t min_rows[ek::kNumLists] = {1, 17, 33, 65};
+        int64_t cap = rows_max / min_rows[l] + (l == ek::kListStream ? 264 : 1);
+        if (l == ek::kListStream && cap > 65535) cap = 65535;
+        if (cap < ek::list_capacity(l, rows_max, E + 1) + 1) cap = ek::list_capacity(l, rows_max, E + 1) + 1;
         L->ws.list_cap[l] = cap;
         A((void **)&L->ws.lists.items[l], sizeof(ek::WorkItem) * cap, "work list");
     }

@@ -254,8 +254,9 @@ ek_status ek_layer_describe(ek_layer *layer, int64_t *hidden, int64_t *inter, in
  * the whole launch is small (a lone expert with up to a few hundred rows), the
  * MFMA tile kernel otherwise, and the two differ in accumulation order (both
  * within the parity tolerance).
- * The same expert may appear more than once; sum(rows) is bounded like n of
- * ek_layer_expert_forward.  All pointers of one call share `mem`. */
+ * The same expert may appear more than once, any number of times; sum(rows) is
+ * bounded like n of ek_layer_expert_forward (and one launch takes at most 65535
+ * calls of up to 16 rows).  All pointers of one call share `mem`. */
 ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32_t *experts,
                                    const void *const *xs, const int64_t *rows, void *const *outs,
                                    int32_t mem, void *stream);

@@ -313,6 +313,34 @@ def test_tile_route_shortest_contractions(ek, oracle, cuda, H, I, w8):
     layer.close()
 
 
+def test_grouped_launch_with_many_calls_per_expert(ek, oracle, cuda):
+    """A worker that collects concurrent requests may hand over many calls for one expert
+    (controller/executor.rs:141-195 fires one per expert and forward; forwards of several sequences
+    meet in the collector).  Every call is a segment of its own, so one grouped launch can hold far
+    more 17..64-row items than a layer call's one-per-expert: 130 calls on 4 experts here.  Each
+    result is held to the oracle; calls of at most 16 rows also to the same call alone, bit for bit."""
+    dt, H, I, E = torch.bfloat16, 256, 128, 4
+    w = wl.Workload("t", H, I, E, 1, 4096, dt, w8=True)
+    layer, ws = load_layer(ek, w)
+    wu, wg, wd = oracle_weights(oracle, ws, E, dt)
+    g = torch.Generator().manual_seed(11)
+    sizes = [20] * 40 + [40] * 30 + [5] * 50 + [200] * 3 + [64, 17, 33, 65, 128, 129, 16]
+    order = torch.randperm(len(sizes), generator=g).tolist()
+    sizes = [sizes[i] for i in order]
+    es = [int(torch.randint(0, E, (1,), generator=g)) for _ in sizes]
+    xs = [torch.randn(n, H, generator=g).to(dt) for n in sizes]
+    outs = layer.experts_forward(es, [x.to(cuda) for x in xs])
+    assert len(outs) == len(sizes)
+    for i, (e, x, o) in enumerate(zip(es, xs, outs)):
+        ffn_gate(o, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"grouped call {i} n={x.shape[0]}", plain=False, small=2)
+        if x.shape[0] <= 16:
+            assert torch.equal(layer.expert_forward(e, x.to(cuda)).view(torch.int16), o.view(torch.int16)), i
+    host = layer.experts_forward(es, xs)
+    for o, h in zip(outs, host):
+        assert torch.equal(o.cpu().view(torch.int16), h.view(torch.int16))
+    layer.close()
+
+
 @pytest.mark.parametrize("H,I", [(64, 128), (128, 64), (64, 64), (64, 320)])
 @pytest.mark.parametrize("n", [600, 1500])
 def test_one_step_contractions_in_a_per_expert_call(ek, oracle, cuda, H, I, n):
