@@ -221,8 +221,7 @@ def time_layer(layer, w, args, dev, stream):
     dev_s = ev0.elapsed_time(ev1) * 1e-3
     st = layer.stats()
     layer.profile(False)
-    if args.repeat_check:
-        assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), "timed calls changed the output"
+    assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), "timed calls changed the output"
     step_s = max(wall, dev_s) / args.steps
     n_prof = max(st["profiled_calls"], 1)
     return {"w": w, "x": x, "ids": ids, "gw": gw, "counts": counts, "step_s": step_s, "dev_s": dev_s / args.steps,
@@ -291,9 +290,6 @@ def main():
                     help="with --workload c3: do not also measure the c4 prefill call on the same experts")
     ap.add_argument("--no-parity", dest="parity", action="store_false", help="skip the oracle's output gate before timing")
     ap.add_argument("--no-peaks", dest="peaks", action="store_false", help="skip the copy / read / MFMA microbenchmarks")
-    ap.add_argument("--no-repeat-check", dest="repeat_check", action="store_false",
-                    help="do not require the timed calls to reproduce the first call's output bit for bit (only for "
-                         "the timing-only ablation builds of the library, whose results are wrong by construction)")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
                          "used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")

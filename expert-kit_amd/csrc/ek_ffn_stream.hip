@@ -264,20 +264,10 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
     }
 }
 
-// Tuned on MI355X at the DeepSeek-V3 shape (see the profiles): channel tiles per wave (NG)
-// and prefetch depth in k steps (D) per stage.
-#ifndef EK_TUNE_S1_NG
-#define EK_TUNE_S1_NG 1
-#endif
-#ifndef EK_TUNE_S1_D
-#define EK_TUNE_S1_D 8
-#endif
-#ifndef EK_TUNE_S2_NG
-#define EK_TUNE_S2_NG 2
-#endif
-#ifndef EK_TUNE_S2_D
-#define EK_TUNE_S2_D 4
-#endif
+// Channel tiles per wave and prefetch depth in k steps, per stage: stage 1 one tile eight steps
+// deep, stage 2 two tiles four deep (the fastest of the shapes measured on MI355X at the
+// DeepSeek-V3 shape).
+constexpr int kStage1Tiles = 1, kStage1Depth = 8, kStage2Tiles = 2, kStage2Depth = 4;
 
 template <typename T, int WM, int NMAT, int NG, int D>
 static hipError_t launch_d(const FfnArgs &a, int32_t nseg, hipStream_t s)
@@ -304,8 +294,8 @@ constexpr int64_t kSplitBelow = 1536;
 template <typename T, int WM, int NMAT>
 static hipError_t launch_g(const FfnArgs &a, int32_t nseg, bool wide, hipStream_t s)
 {
-    constexpr int NG = NMAT == 2 ? EK_TUNE_S1_NG : EK_TUNE_S2_NG;
-    constexpr int D = NMAT == 2 ? EK_TUNE_S1_D : EK_TUNE_S2_D;
+    constexpr int NG = NMAT == 2 ? kStage1Tiles : kStage2Tiles;
+    constexpr int D = NMAT == 2 ? kStage1Depth : kStage2Depth;
     const int NT = a.N / 16;
     if (wide) {
         // four activation fragments per prefetch slot: shallower, the eight slices make up for it

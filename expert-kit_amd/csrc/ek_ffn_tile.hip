@@ -80,33 +80,6 @@ __device__ __forceinline__ void lds_barrier()
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" : : : "memory");
 }
 
-// Timing-only builds (`make ablation ABL=...`, WRONG RESULTS, never the shipped library): the
-// tile kernel with one part of its step left out, to measure what that part costs in cycles
-// and in clock under the chip's power limit.
-//   EK_ABL_NO_DMA      no LDS-DMA after a workgroup's first loads (tiles compute on stale data)
-//   EK_ABL_NO_MFMA     no MFMA in the step loop;  EK_ABL_HALF_MFMA  every second row block's only
-//   EK_ABL_NO_DEQUANT  one-byte weights are fed to the MFMAs as they are stored
-//   EK_ABL_NO_BARRIER  no workgroup barrier per step
-//   EK_ABL_NO_VMWAIT   a step does not wait for its own LDS-DMA (one-byte weights)
-//   EK_ABL_NO_WDMA / EK_ABL_NO_XDMA  no LDS-DMA of the weights / of the activation tile at all
-// Several can be combined by giving the compiler more than one -DEK_ABL_... flag.
-#if defined(EK_ABL_HALF_MFMA)
-#define EK_ABL_MFMA(rb) ((rb) < (RB + 1) / 2)
-#elif defined(EK_ABL_NO_MFMA)
-#define EK_ABL_MFMA(rb) ((rb) < 0)
-#else
-#define EK_ABL_MFMA(rb) true
-#endif
-#if defined(EK_ABL_NO_WDMA)
-#define EK_ABL_WDMA false
-#else
-#define EK_ABL_WDMA true
-#endif
-#if defined(EK_ABL_NO_XDMA)
-#define EK_ABL_XDMA false
-#else
-#define EK_ABL_XDMA true
-#endif
 constexpr int kCusPerXcd = 32;   // MI355X: 8 XCDs x 32 CUs
 
 // A step covers 64 contraction elements: one weight chunk per channel tile with one-byte
@@ -296,11 +269,10 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
         _Pragma("unroll") for (int nr = 0; nr < NR; ++nr)                                       \
         _Pragma("unroll") for (int m = 0; m < NMAT; ++m)                                        \
         _Pragma("unroll") for (int kc = 0; kc < KC; ++kc)                                       \
-            if (EK_ABL_WDMA)                                                                    \
             dma16((ctx).wp[nr] + (int64_t)(((step) * KC + kc) * NMAT + m) * kChunkBytes,        \
                   st_ + w_off + ((nr * NMAT + m) * KC + kc) * kChunkBytes);                     \
         _Pragma("unroll") for (int i = 0; i < LX; ++i)                                          \
-            if (EK_ABL_XDMA) dma16((ctx).xsrc[i] + (step) * BK, st_ + xdst[i]);                 \
+            dma16((ctx).xsrc[i] + (step) * BK, st_ + xdst[i]);                                  \
     }
 
     Ctx cur, nxt;
@@ -336,10 +308,8 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             // the next tile) and than the previous epilogue's stores: wait until only those remain
             if constexpr (AHEAD == 2) {
                 if (step + 1 < nsteps || tn >= 0) {
-#ifndef EK_ABL_NO_VMWAIT
                     if (step < 2 && pend_st) wait_vmcnt_dyn(LOADS + pend_st);
                     else wait_vmcnt<LOADS>();
-#endif
                 } else {
                     wait_vmcnt<0>();
                 }
@@ -349,19 +319,15 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                 if (step == 0 && pend_st) wait_vmcnt_dyn(pend_st);
                 else wait_vmcnt<0>();
             }
-#ifndef EK_ABL_NO_BARRIER
             block_barrier();   // this step's tile is visible to all waves; the stage of the
                                // previous step is free again
-#endif
             if (step == fstep) tn = fetch(tc + stride, nxt, cur.sslot ^ 1);
             const int ring2 = ring + AHEAD >= NS ? ring + AHEAD - NS : ring + AHEAD;   // (ring + AHEAD) % NS
-#ifndef EK_ABL_NO_DMA
             if (step + AHEAD < nsteps) {
                 EK_ISSUE(cur, step + AHEAD, ring2);
             } else if (tn >= 0) {
                 EK_ISSUE(nxt, step + AHEAD - nsteps, ring2);
             }
-#endif
 
             const uint8_t *stage = lds + ring * G::STAGE;
             const uint8_t *wreg = stage + w_off;
@@ -379,9 +345,6 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
                     sblk[cb] = sc_area[cur.sslot * kScaleSlotFloats + (kSplitBlock ? hh : cb) * kTileScaleBlocks + (step >> 1)];
             }
             auto dq = [&](uint32_t w, int cb) -> u32x2 {
-#ifdef EK_ABL_NO_DEQUANT
-                return u32x2{w, w ^ (uint32_t)cb};
-#endif
                 if constexpr (WM == kWF8Block) return dequant_f8x4<T>(w, sblk[cb]);
                 else if constexpr (WM == kWI8Block) return dequant_u8x4<T>(w, sblk[cb], -128.f * sblk[cb]);
                 else return dequant_u8x4<T>(w, cur.as[cb], cur.ac[cb]);
@@ -396,7 +359,7 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
             // the conversion of that step's first k-group, which nothing else could overlap.
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
-                if (step > 0 && EK_ABL_MFMA(rb)) {
+                if (step > 0) {
 #pragma unroll
                     for (int cb = 0; cb < CB; ++cb)
                         acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[1][cb]), bf[1][rb], acc[rb][cb]);
@@ -425,11 +388,9 @@ __device__ __forceinline__ void run_tiles(const FfnArgs &a, const WorkItem *item
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) {
                     bf[ng][rb] = *(const V8 *)(stage + boff[grp + 1] + rb * kRowBlockBytes);
-                    if (EK_ABL_MFMA(rb)) {
 #pragma unroll
-                        for (int cb = 0; cb < CB; ++cb)
-                            acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cg][cb]), bf[cg][rb], acc[rb][cb]);
-                    }
+                    for (int cb = 0; cb < CB; ++cb)
+                        acc[rb][cb] = Act<T>::mfma32(__builtin_bit_cast(V8, af[cg][cb]), bf[cg][rb], acc[rb][cb]);
                     if constexpr (W8) {
                         // next group's A operands: 2 dwords per column block, spread over the row blocks
 #pragma unroll
@@ -554,7 +515,12 @@ constexpr int mid_depth(int wm) { return wm == kW16 ? 2 : kMidDepth; }
 constexpr int kMidXStep = 8192;                 // bytes reserved per step of the activation tile (64 rows x 64 k x 2)
 constexpr int kMidXBuf = kMidDepth * kMidXStep; // one window (of kMidDepth steps at most)
 constexpr int kMidScratch = 2 * kMidXBuf;       // epilogue scratch behind the two window buffers
-constexpr int kMidScales = kMidScratch + 8 * 32 * 144;   // block scales behind the scratch: [tile parity][wave][column block][block]
+constexpr int kMidEnd = kMidScratch + 8 * 32 * 144;      // end of what this form stores into with waves of other tiles in flight
+// The block scales ([tile parity][wave][column block][block], wave-private) do not live in that
+// range: a wave fetches its first tile's scale rows before the barrier that separates this form from
+// the class that ran before it, while slower waves may still be reading that class's stages and
+// epilogue scratch.  They share run_tiles' own scale area behind its stages (same layout, and a wave
+// touches only its own part of it in either form).
 
 template <typename T> struct MidCtx {
     const uint8_t *wl[2];    // this lane's bytes of the column block's weight chunks at step 0, slot tt = 0
@@ -566,7 +532,8 @@ template <typename T> struct MidCtx {
 
 template <typename T, int WM, int NMAT, int MR>
 __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items, const int ntiles,
-                                        const int nb_count, const int first, const int stride, uint8_t *lds)
+                                        const int nb_count, const int first, const int stride, uint8_t *lds,
+                                        float *scales)
 {
     using V8 = typename Act<T>::V8;
     constexpr bool W8 = WM != kW16;
@@ -593,7 +560,7 @@ __device__ __forceinline__ void run_mid(const FfnArgs &a, const WorkItem *items,
         boff[grp] = (l32 * PPR + (c ^ swizzle_key<PPR>(j))) * 16;
     }
     // block scales: as in run_tiles, the tile's rows of the scale matrices in a wave-private LDS area
-    float *const sc_area = (float *)(lds + kMidScales) + wave * (CB * kTileScaleBlocks);
+    float *const sc_area = scales + wave * (CB * kTileScaleBlocks);
     constexpr int kScaleSlotFloats = WAVES * CB * kTileScaleBlocks;
     auto fetch = [&](int t, Ctx &c, int sslot) -> int {
         for (; t < ntiles; t += stride) {
@@ -847,8 +814,11 @@ __global__ __launch_bounds__(WAVES * 64, 1) void ffn_tile_kernel(FfnArgs a, int 
         if (nsteps % mid_depth(WM) == 0 && nsteps >= 2 * mid_depth(WM) &&
             (int64_t)(n128 + n64 + n32) * nb_count >= (int64_t)gridDim.x) {
             const int r32m = (r64 + nslots - (s64 * nb_count) % nslots) % nslots;
-            run_mid<T, WM, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds);
-            run_mid<T, WM, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32m, nslots, lds);
+            static_assert(kMidEnd <= G::STAGES * G::STAGE, "the register-streamed form's buffers end before the scale area");
+            static_assert(TileGeom<true, 8, 2, 128>::SCALE_ROWS == 2, "both forms lay the scale area out alike");
+            float *const scales = (float *)(lds + G::STAGES * G::STAGE);
+            run_mid<T, WM, NMAT, 4>(a, a.lists.items[kListT64] + lo64, s64 * nb_count, nb_count, r64, nslots, lds, scales);
+            run_mid<T, WM, NMAT, 2>(a, a.lists.items[kListT32] + lo32, s32 * nb_count, nb_count, r32m, nslots, lds, scales);
             return;
         }
     }

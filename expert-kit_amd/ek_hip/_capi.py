@@ -10,8 +10,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# EK_HIP_LIB overrides the in-tree library (e.g. an experimental build)
-LIB_PATH = os.environ.get("EK_HIP_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libek_hip.so")
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libek_hip.so")
 
 EK_OK, EK_INVALID_INPUT, EK_EXPERT_NOT_FOUND, EK_WEIGHT_NOT_FOUND, EK_OOM, EK_HIP_ERROR, EK_INTERNAL = range(7)
 EK_BF16, EK_F16, EK_F32, EK_I8, EK_F8E4M3 = range(5)
