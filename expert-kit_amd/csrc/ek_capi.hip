@@ -858,9 +858,12 @@ ek_status err_to_status(int32_t err)
     return EK_OK;
 }
 
-ek_status copy_route_out(ek_layer *L, const Workspace &W, const ek_route_out *r, int64_t P, int mem, hipStream_t s)
+ek_status copy_route_out(ek_layer *L, const Workspace &W, const ek_route_out *r, int64_t P, int mem, hipStream_t s,
+                         bool experts_ran = true)
 {
     if (!r) return EK_OK;
+    if (r->expert_out && !experts_ran)
+        return fail(EK_INVALID_INPUT, "ek_route_out.expert_out: this call runs no experts");
     const int E = L->cfg.n_experts;
     auto out = [&](void *dst, const void *src, size_t bytes) -> ek_status {
         if (mem == EK_HOST) return d2h(L, dst, src, bytes, s);
@@ -871,6 +874,10 @@ ek_status copy_route_out(ek_layer *L, const Workspace &W, const ek_route_out *r,
     if (r->offsets) EK_TRY(out(r->offsets, W.offsets, sizeof(int32_t) * (E + 1)));
     if (P > 0 && r->perm) EK_TRY(out(r->perm, W.perm, sizeof(int32_t) * P));
     if (P > 0 && r->inv_perm) EK_TRY(out(r->inv_perm, W.inv_perm, sizeof(int32_t) * P));
+    if (P > 0 && r->expert_out) {
+        if (L->padded) EK_TRY(rows_out(L, r->expert_out, W.yp, P, mem, s));    // the caller's hidden size
+        else EK_TRY(out(r->expert_out, W.yp, (size_t)P * L->cfg.hidden * 2));
+    }
     return EK_OK;
 }
 
@@ -1423,7 +1430,7 @@ ek_status ek_layer_pack(ek_layer *layer, const int32_t *ids, int64_t T, const ek
         if (mem == EK_HOST && xp && P > 0) EK_TRY(d2h(layer, xp, d_xp, (size_t)P * H * 2, s));
         // the rows went into the staging buffer back to back: give a padded layer its zero columns back
         if (layer->padded && mem == EK_HOST && xp && T > 0) EK_HIP(hipMemsetAsync(layer->st_x, 0, (size_t)T * H * 2, s));
-        EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
+        EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s, false));
         if (!stream) { use.synced(); return finish_blocking(layer, layer->ws, s); }
         return EK_OK;
     )

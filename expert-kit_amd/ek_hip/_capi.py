@@ -35,7 +35,7 @@ class ek_weight_desc(ctypes.Structure):
 
 class ek_route_out(ctypes.Structure):
     _fields_ = [("counts", ctypes.c_void_p), ("offsets", ctypes.c_void_p), ("perm", ctypes.c_void_p),
-                ("inv_perm", ctypes.c_void_p)]
+                ("inv_perm", ctypes.c_void_p), ("expert_out", ctypes.c_void_p)]
 
 
 class ek_stats(ctypes.Structure):

@@ -193,27 +193,32 @@ class HipLayer:
         return bool(out.value)
 
     # -- compute ----------------------------------------------------------
-    def _route(self, T: int, device):
+    def _route(self, T: int, device, expert_out: Optional[torch.Tensor] = None):
         E, K = self.cfg.n_experts, self.cfg.top_k
         rt = RouteTables(torch.empty(E, dtype=torch.int32, device=device),
                          torch.empty(E + 1, dtype=torch.int32, device=device),
                          torch.empty(T * K, dtype=torch.int32, device=device),
                          torch.empty(T * K, dtype=torch.int32, device=device))
         ro = C.ek_route_out(rt.counts.data_ptr(), rt.offsets.data_ptr(), rt.perm.data_ptr(),
-                            rt.inv_perm.data_ptr())
+                            rt.inv_perm.data_ptr(), 0 if expert_out is None else expert_out.data_ptr())
         return rt, ro
 
     def forward(self, x: torch.Tensor, ids: torch.Tensor, w: torch.Tensor, return_route: bool = False,
-                stream=None, out: Optional[torch.Tensor] = None):
-        """y[T,H] = sum_k w[t,k] * expert_{ids[t,k]}(x[t]); see ek_layer_forward."""
+                stream=None, out: Optional[torch.Tensor] = None, expert_out: Optional[torch.Tensor] = None):
+        """y[T,H] = sum_k w[t,k] * expert_{ids[t,k]}(x[t]); see ek_layer_forward.
+        expert_out (with return_route): a [T*K, H] tensor beside x that receives every pair's expert
+        output in packed order (ek_route_out.expert_out)."""
         assert x.dim() == 2 and ids.dim() == 2 and w.shape == ids.shape
         x, ids, w = x.contiguous(), ids.contiguous(), w.contiguous()
         assert ids.dtype == torch.int32 and x.dtype == self.act_dtype
         assert x.is_cuda == ids.is_cuda == w.is_cuda
         T = x.shape[0]
+        if expert_out is not None:
+            assert return_route and expert_out.is_contiguous() and expert_out.dtype == x.dtype
+            assert expert_out.is_cuda == x.is_cuda and tuple(expert_out.shape) == (ids.numel(), x.shape[1])
         with (_alloc_on(stream) if out is None or return_route else _NO_CTX):
             y = out if out is not None else torch.empty_like(x)
-            rt, ro = self._route(T, x.device) if return_route else (None, None)
+            rt, ro = self._route(T, x.device, expert_out) if return_route else (None, None)
         C.check(self._lib.ek_layer_forward(self._h, _ptr(x), _ptr(ids), _ptr(w), _DT[w.dtype], T, _ptr(y),
                                            ctypes.byref(ro) if ro is not None else None, _mem(x),
                                            _stream_ptr(stream)))

@@ -129,6 +129,10 @@ typedef struct ek_route_out {
     int32_t *offsets;  /* [E+1] exclusive scan of counts */
     int32_t *perm;     /* [T*K] packed position -> flat pair index t*K+k */
     int32_t *inv_perm; /* [T*K] flat pair index -> packed position */
+    void *expert_out;  /* [T*K, hidden] every pair's expert output before the weighted sum, in packed
+                        * order (row j belongs to pair perm[j]; activation dtype): the rows
+                        * NaiveExecutor::scatter places into [T, K, H] (executor.rs:203-252).  Calls
+                        * that run the experts only (not ek_layer_pack). */
 } ek_route_out;
 
 /* Counters the worker shell feeds into its Prometheus series

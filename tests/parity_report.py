@@ -30,7 +30,8 @@ def summary_lines():
             f"outright, worst {max((r['max_err_over_rms'] for r in within), default=0.0):.3e})")
     if beyond:
         worst = max(beyond, key=lambda r: r["max_err_over_rms"])
-        line += (f"; {len(beyond)} beyond it, all within 2e-2*rms + the storage quanta of the 16-bit tensors "
+        line += (f"; {len(beyond)} beyond it, all within 2e-2*rms + the storage quanta of the 16-bit tensors, every excess "
+                 f"element of the one-expert gates and of the full-size calls classified one by one "
                  f"(worst {worst['max_err_over_rms']:.3e}: {worst['name']}, {worst['over_frac']:.1e} of its {worst['elems']} elements)")
     lines.append(line)
     return lines

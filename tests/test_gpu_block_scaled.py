@@ -96,7 +96,8 @@ def test_one_expert_tiled(ek, oracle, cuda, kind):
     x = torch.randn(n, H, generator=torch.Generator().manual_seed(n)).to(dt)
     ref = oracle.ffn(x, *ref_weights(oracle, ew, dt), mode=2)
     got = layer.expert_forward(1, x.to(cuda))
-    ffn_gate(got, ref, f"{kind} block expert tiled n={n}", plain=False)
+    # (fp8: 2.19e-2 on 2 of the 576000 outputs, both y_ref rounded to bf16; int8: 1.27e-2)
+    ffn_gate(got, ref, f"{kind} block expert tiled n={n}", plain=kind != "fp8")
     assert check_vs_rounded(got, ref) > 0.9
     routed = layer.forward(x.to(cuda), torch.ones(n, 1, dtype=torch.int32, device=cuda), torch.ones(n, 1, dtype=dt, device=cuda))
     assert torch.equal(routed.view(torch.int16), got.view(torch.int16))
@@ -148,7 +149,8 @@ def test_batch_of_small_calls_and_blob_ingestion(ek, oracle, cuda, kind):
     x = torch.randn(16 * 200, H, generator=torch.Generator().manual_seed(9)).to(dt)
     outs = torch.cat(layer.experts_forward([0] * 200, list(x.to(cuda).split(16))))
     ref = oracle.ffn(x, *ref_weights(oracle, ew, dt), mode=2)
-    ffn_gate(outs, ref, "fp8 batch of 200 calls", plain=False)      # 2.45e-2: one of 1.2 million outputs, at 7 sigma
+    # (int8: 2.45e-2 on one of 1.2 million outputs, at 7 sigma, y_ref rounded to bf16; fp8: 1.8e-2)
+    ffn_gate(outs, ref, f"{kind} batch of 200 calls", plain=kind != "int8")
     one = layer.expert_forward(0, x[32:48].to(cuda))                    # the same rows alone: same bits
     assert torch.equal(one.view(torch.int16), outs[32:48].view(torch.int16))
     layer.close()

@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 SHAPES = [(16, 8), (72, 100), (200, 24), (64, 1), (8, 300)]
 
 
-def gate(oracle, got, x, wu, wg, wd, name):
+def gate(oracle, got, x, wu, wg, wd, name, plain=True):
     """test_gpu_parity's one-expert gate.  Below 64 intermediate channels an output is the sum of so
     few terms that one of them can be most of it, and the reference's own storage roundings of that
     term (up, gate, silu, their product: four, and a result that takes another summation order may
@@ -27,8 +27,7 @@ def gate(oracle, got, x, wu, wg, wd, name):
     output RMS: there the bound adds that budget, 4 steps * sum_j |h_j| |W_down[i, j]|."""
     ref, h = oracle.ffn(x, wu, wg, wd, mode=2, return_h=True)
     if wu.shape[0] >= 64:
-        # (weights 16 times the benchmark's on 72..300-term contractions: heavy tails, up to 2.4e-2)
-        ffn_gate(got, ref, name, small=2, plain=False)
+        ffn_gate(got, ref, name, small=2, plain=plain)
         return ref
     step = 2.0 ** (-8 if x.dtype == torch.bfloat16 else -11)
     budget = 4 * step * (h.float().abs() @ wd.float().abs().T)
@@ -145,7 +144,9 @@ def test_block_scaled(ek, oracle, cuda, H, I, kind):
         print(f"odd shape block-scaled {kind} H={H} I={I} n={n}", flush=True)
         x = torch.randn(n, H, generator=torch.Generator().manual_seed(n)).to(dt)
         got = layer.expert_forward(1, x.to(cuda))
-        gate(oracle, got, x, *ref_weights(oracle, ew, dt), f"odd block {kind} H={H} I={I} n={n}")
+        # (weights 16 times the benchmark's on 72..136-term contractions: heavy tails.  fp8 at 200 rows: 2.41e-2 /
+        # 2.45e-2 on 2 / 3 of the 40000 / 52800 outputs, each y_ref rounded to bf16; every other case <= 1.85e-2)
+        gate(oracle, got, x, *ref_weights(oracle, ew, dt), f"odd block {kind} H={H} I={I} n={n}", plain=not (kind == "fp8" and n == 200))
     layer.close()
 
 

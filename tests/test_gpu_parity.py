@@ -62,6 +62,17 @@ def ffn_gate(got: torch.Tensor, ref32: torch.Tensor, name: str, small: int = 0, 
         assert worst <= TOL, f"{name}: max|err|/rms = {worst:.3e} exceeds the plain bound"
     else:
         assert strict_viol <= 1e-4 or int((err > TOL * rms).sum()) <= small
+        # the sharp statement for whatever exceeds the plain bound: the stored output is y_ref rounded to
+        # the output type, or the 16-bit value next to it
+        over = err > TOL * rms
+        if bool(over.any()):
+            rounded = ref32.to(got.dtype)
+            step = (got.float().cpu() - rounded.float()).abs()[over]
+            exact = int((step == 0).sum())
+            near = int(((step > 0) & (step <= ulp_of(ref32, got.dtype)[over] * 1.0001)).sum())
+            print(f"{name}: {int(over.sum())} outputs over 2e-2*rms: {exact} are y_ref rounded to the output type, "
+                  f"{near} its 16-bit neighbour", flush=True)
+            assert exact + near == int(over.sum()), f"{name}: an output over the plain bound is two or more ulps from rne(y_ref)"
     return worst
 
 
@@ -288,7 +299,10 @@ def test_narrow_and_wide_tiles_give_the_same_bits(ek, oracle, cuda, dt, w8):
         narrow = layer.expert_forward(1, x.to(cuda))
         wide = layer.forward(x.to(cuda), torch.ones(n, 1, dtype=torch.int32, device=cuda), torch.ones(n, 1, dtype=dt, device=cuda))
         assert torch.equal(narrow.view(torch.int16), wide.view(torch.int16)), (dt, w8, n)
-        ffn_gate(narrow, oracle.ffn(x, wu, wg, wd, mode=2), f"narrow tiles dt={dt} w8={w8} n={n}", plain=False)
+        # (bf16, int8 weights, 1000 rows: 2.94e-2 on one of the 256000 outputs, which is y_ref rounded to bf16;
+        # the other seven cases 1.9e-3 .. 1.64e-2)
+        ffn_gate(narrow, oracle.ffn(x, wu, wg, wd, mode=2), f"narrow tiles dt={dt} w8={w8} n={n}",
+                 plain=not (dt == torch.bfloat16 and w8 and n == 1000))
     layer.close()
 
 
@@ -307,8 +321,9 @@ def test_tile_route_shortest_contractions(ek, oracle, cuda, H, I, w8):
     ref = oracle.ffn(x, wu, wg, wd, mode=2)
     got = layer.forward(x.to(cuda), torch.zeros(n, 1, dtype=torch.int32, device=cuda), torch.ones(n, 1, dtype=dt, device=cuda))
     # 0.3 to 1.3 million outputs of 64- to 256-term contractions reach 7 sigma, where half a bf16 ulp is
-    # 2.7e-2 * rms: measured 1.6e-2 .. 2.9e-2, 3e-6 of the elements beyond the plain bound
-    ffn_gate(got, ref, f"shortest contractions H={H} I={I} w8={w8}", plain=False)
+    # 2.7e-2 * rms.  Measured: (64, 128, bf16 weights) 2.015e-2 on one output and (256, 128, int8) 2.339e-2 on
+    # one, both y_ref rounded to bf16; the other three 1.43e-2 .. 1.93e-2
+    ffn_gate(got, ref, f"shortest contractions H={H} I={I} w8={w8}", plain=(H, I, w8) not in ((64, 128, False), (256, 128, True)))
     assert check_vs_rounded(got, ref) > 0.9
     layer.close()
 
@@ -332,7 +347,9 @@ def test_grouped_launch_with_many_calls_per_expert(ek, oracle, cuda):
     outs = layer.experts_forward(es, [x.to(cuda) for x in xs])
     assert len(outs) == len(sizes)
     for i, (e, x, o) in enumerate(zip(es, xs, outs)):
-        ffn_gate(o, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"grouped call {i} n={x.shape[0]}", plain=False, small=2)
+        # (call 50, 20 rows: 2.19e-2 on one of its 5120 outputs, which is y_ref rounded to bf16; the other 129 calls
+        # hold the plain bound, worst 1.9e-2)
+        ffn_gate(o, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"grouped call {i} n={x.shape[0]}", plain=i != 50, small=2)
         if x.shape[0] <= 16:
             assert torch.equal(layer.expert_forward(e, x.to(cuda)).view(torch.int16), o.view(torch.int16)), i
     host = layer.experts_forward(es, xs)
@@ -354,7 +371,7 @@ def test_one_step_contractions_in_a_per_expert_call(ek, oracle, cuda, H, I, n):
     wu, wg, wd = [t[1] for t in oracle_weights(oracle, ws, 2, dt)]
     x = torch.randn(n, H, generator=torch.Generator().manual_seed(n + H)).to(dt)
     got = layer.expert_forward(1, x.to(cuda))
-    ffn_gate(got, oracle.ffn(x, wu, wg, wd, mode=2), f"one-step contraction H={H} I={I} n={n}", plain=False)
+    ffn_gate(got, oracle.ffn(x, wu, wg, wd, mode=2), f"one-step contraction H={H} I={I} n={n}")      # (fp16: 1.6e-3 .. 1.9e-3)
     layer.close()
 
 
@@ -469,7 +486,7 @@ def test_layer_small_w8(ek, oracle, cuda):
 def test_layer_ragged_lengths(ek, oracle, cuda):
     """Segment lengths from 0 to a few hundred in one call (hot expert + empty experts)."""
     w = wl.Workload("ragged", 256, 128, 24, 2, 400, torch.bfloat16, zipf_s=2.0)
-    # 2.33e-2: the distance of the correctly rounded reference output itself from y_ref on this input
+    # 2.33e-2 on one of the 102400 outputs: the distance of the correctly rounded reference output itself from y_ref on this input
     # (tests/test_oracle_tolerance.py::test_last_storage_rounding_alone_exceeds_the_plain_bound)
     run_layer_parity(ek, oracle, cuda, w, plain=False)
 
@@ -520,8 +537,8 @@ def test_layer_full_size_sampled_tokens(ek, oracle, cuda, name):
     tokens = sampled.choose_tokens(ids, w.n_experts)
     print(f"{name} full size: tokens {tokens}", flush=True)
     r = sampled.check(y[tokens], x[tokens], ids[tokens], gw[tokens], w.n_experts, lambda e: ws[e])
-    # c3: 2.72e-2 on 3 of the 43008 sampled outputs (rounding floor of the reference's own output: see the summary)
-    layer_gate(y[tokens], r["ref"], r["y3"], gw[tokens], f"{name} full size, sampled tokens", plain=name != "c3")
+    # measured: c2 2.1e-3, c3 1.18e-2, c4 1.34e-2, c5 2.6e-3: the plain bound for all four
+    layer_gate(y[tokens], r["ref"], r["y3"], gw[tokens], f"{name} full size, sampled tokens")
     assert layer.stats()["pairs"] == w.pairs
     layer.close()
 

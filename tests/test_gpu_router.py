@@ -149,8 +149,8 @@ def test_forward_logits_is_route_then_forward(ek, oracle, cuda, dt, w8):
     else:
         wu, wg, wd = [e.up_w for e in experts], [e.gate_w for e in experts], [e.down_w for e in experts]
     out = oracle.layer_forward(x, ids.cpu(), w.cpu(), wu, wg, wd, mode=2, return_y3=True)
-    # (bf16 with int8 weights whose scales make |W| reach 0.5: 2.75e-2, 4e-5 of the outputs beyond the plain bound)
-    layer_gate(y, out[0], out[5], w.cpu(), f"forward_logits {dt} w8={w8}", plain=not (dt == torch.bfloat16 and w8))
+    # (measured: bf16 1.34e-2, fp16 1.7e-3, bf16 with int8 weights whose scales make |W| reach 0.5 1.25e-2)
+    layer_gate(y, out[0], out[5], w.cpu(), f"forward_logits {dt} w8={w8}")
     layer.close()
 
 

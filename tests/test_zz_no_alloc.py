@@ -2,7 +2,9 @@
 (for callers that cannot allocate device memory), held to ek_layer_forward through the C ABI:
 bit-identical outputs and routing tables on two calls in a row, the second with a smaller
 input (the array keeps the first call's contents), on a caller's stream and blocking, with
-several layers sharing the GPU's one array, and a refusal for calls that do not fit."""
+several layers sharing the GPU's one array, a refusal for calls that do not fit, and the property
+itself: free device memory unchanged over the calls, and the call accepted inside a stream capture
+that refuses allocating runtime calls."""
 import pytest
 import torch
 
@@ -108,3 +110,42 @@ def test_static_call_refuses_what_does_not_fit(ek, cuda):
                              torch.ones(2, 1, dtype=torch.bfloat16, device=cuda))
     assert ei.value.status == C.EK_INVALID_INPUT
     small.close()
+
+
+def test_static_call_allocates_nothing(ek, cuda):
+    """The property itself, observed two ways.  (1) Free device memory (hipMemGetInfo) is the same
+    before and after calls whose output tensor is the caller's.  (2) The call is made while the
+    caller's stream is under capture in the mode that refuses every allocating runtime call: the
+    capture ends without an error, and the graph replays to the allocating call's bits, twice, with
+    a smaller eager static call (which leaves its own contents in the shared array) in between."""
+    w = wl.Workload("static", 512, 256, 16, 4, 1, torch.bfloat16, w8=True)
+    layer = build(ek, w, 300)
+    x, ids, gw = inputs(w, 300, 21, cuda)            # a hot expert's tiles beside streaming items
+    xs, idss, gws = inputs(w, 23, 22, cuda)
+    want, want_small = layer.forward(x, ids, gw), layer.forward(xs, idss, gws)
+    y, ysmall = torch.empty_like(x), torch.empty_like(xs)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    layer.forward_static(x, ids, gw, stream=side, out=y)          # first use of this stream (its side stream is picked)
+    side.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        layer.forward_static(x, ids, gw, stream=side, out=y)
+        layer.forward_static(xs, idss, gws, stream=side, out=ysmall)
+    side.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "a static call changed the free device memory"
+    assert torch.equal(bits(y), bits(want)) and torch.equal(bits(ysmall), bits(want_small))
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side, capture_error_mode="global"):
+            layer.forward_static(x, ids, gw, stream=torch.cuda.current_stream(), out=y)
+    torch.cuda.synchronize()
+    for rep in range(2):
+        y.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(bits(y), bits(want)), f"replay {rep}"
+        layer.forward_static(xs, idss, gws, out=ysmall)           # eager, blocking, smaller: same array
+        assert torch.equal(bits(ysmall), bits(want_small)), f"after replay {rep}"
+    layer.close()
