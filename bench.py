@@ -10,9 +10,12 @@ metric is quoted on (c3), the roofline of its dominant kernel (per-phase HIP
 events recorded on the launch stream inside the timed region), `parity` (the
 CPU oracle's output gate on the timed input, sampled tokens), `prefill` (the
 8192-token configuration c4 measured on the same experts in the same run, with
-its MFMA roofline), `peaks` (copy / non-temporal read / MFMA ceilings measured by
-the library's microkernels) and `cpu_baseline` (the reference-equivalent CPU
-backend timed on this box's host cores on a bounded sample of the workload).
+its MFMA roofline and a CPU baseline of its own), `c1` / `c2` / `c5` (the other
+three benchmark configurations, each built, gated, timed and freed in turn: time
+per call, pairs/s, the roof that binds and the fraction reached), `peaks` (copy /
+non-temporal read / MFMA ceilings measured by the library's microkernels) and
+`cpu_baseline` (the reference-equivalent CPU backend timed on this box's host
+cores on a bounded sample of the workload).
 """
 import argparse
 import json
@@ -48,7 +51,7 @@ def measured_traffic(workload: str, stage: int, decode: bool):
     return total if seen else None
 
 
-def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
+def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0, max_runs=15):
     """Reference-equivalent CPU backend (libtorch ops of ffn/expert_torch.rs:81-84,
     grouped per expert, weighted sum of qwen3_moe.py:102-104) on the pairs routed to
     a sample of experts; weights pre-cast to the compute dtype as load_module does."""
@@ -71,7 +74,7 @@ def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0):
     sample = set(ws_sample)
     times, pairs = [], 0
     t_all = time.time()
-    while len(times) < 15 and (time.time() - t_all < target_s or not times):
+    while len(times) < max_runs and (time.time() - t_all < target_s or not times):
         t0 = time.time()
         _, pairs = oracle.torch_layer_forward(x, ids, gw, wu, wg, wd, experts=sample)
         times.append(time.time() - t0)
@@ -93,7 +96,8 @@ def calibration_copy(args, dev):
 
 
 def bench_chain(args, w, dev):
-    """The ragged continuous-batching mix over n_layers consecutive layers, one hipGraph."""
+    """The ragged continuous-batching mix over n_layers consecutive layers, one hipGraph.
+    Returns the JSON object of the run."""
     import torch
     import ek_hip
     from ek_hip import workloads as wl
@@ -111,6 +115,17 @@ def bench_chain(args, w, dev):
     y = torch.empty_like(xd)
     chain = ek_hip.HipChain(layers)
     stream = torch.cuda.Stream()          # enqueue-only calls on a stream of the caller's
+    # gates on the timed input: the first layer's routing tables against a CPU stable sort, its output
+    # on sampled tokens against the oracle (the later layers' inputs are the library's own outputs)
+    x0 = wl.make_x(w)
+    w0 = w
+    y0, rt0 = layers[0].forward(xd, ids[0].contiguous(), gw[0].contiguous(), return_route=True)
+    assert torch.equal(rt0.perm.cpu(), torch.argsort(routing[0][0].reshape(-1).long(), stable=True).to(torch.int32)), \
+        "routing permutation mismatch"
+    parity = None
+    if args.parity:
+        from dataclasses import replace
+        parity = parity_on_timed_input(replace(w0, n_layers=1), xd, routing[0][0], routing[0][1], y0, x0)
     y_eager = chain.forward(xd, ids, gw, use_graph=False).clone()
     calibration_copy(args, dev)
     res = {}
@@ -148,8 +163,13 @@ def bench_chain(args, w, dev):
                   "mfma_frac": f / step_s / MFMA_PEAK_16, "eager_ms_per_step": res["eager"] * 1e3,
                   "graph_ms_per_step": res["graph"] * 1e3},
     }
+    if parity is not None:
+        out["parity"] = parity
+        out["parity"]["of"] = "the first layer's output on the chain's input (later layers consume the library's own outputs)"
     chain.close()
-    print(json.dumps(out))
+    for layer in layers:
+        layer.close()
+    return out
 
 
 def cpu_model() -> str:
@@ -183,7 +203,7 @@ def parity_on_timed_input(w, xd, ids, gw, y, x):
     return r
 
 
-def time_layer(layer, w, args, dev, stream):
+def time_layer(layer, w, args, dev, stream, graph=False):
     """Parity gates on the workload's input, then warm-up and K timed enqueue-only layer calls on
     `stream` (a stream of the caller's, not the default one).  Returns the measurements."""
     import torch
@@ -224,8 +244,31 @@ def time_layer(layer, w, args, dev, stream):
     assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), "timed calls changed the output"
     step_s = max(wall, dev_s) / args.steps
     n_prof = max(st["profiled_calls"], 1)
+    graph_s = None
+    if graph:
+        # the same call captured once into a graph of the caller's and replayed: what a serving loop that
+        # replays its decode step pays (no launch gaps, no fork / join on the host)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(g, stream=stream):
+                layer.forward(xd, idd, gwd, stream=torch.cuda.current_stream(), out=y)
+        torch.cuda.synchronize()
+        for _ in range(args.warmup):
+            g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(args.steps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        graph_s = max(time.perf_counter() - t0, e0.elapsed_time(e1) * 1e-3) / args.steps
+        assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), "graph replays changed the output"
+        del g
     return {"w": w, "x": x, "ids": ids, "gw": gw, "counts": counts, "step_s": step_s, "dev_s": dev_s / args.steps,
-            "k_us": [v / n_prof for v in st["kernel_us"]], "parity": parity, "phase_calls": st["profiled_calls"]}
+            "k_us": [v / n_prof for v in st["kernel_us"]], "parity": parity, "phase_calls": st["profiled_calls"],
+            "graph_s": graph_s}
 
 
 def roofline_of(m):
@@ -272,17 +315,72 @@ def roofline_of(m):
     return roof, layer, config
 
 
+def build_layer(w, max_tokens, keep=()):
+    """The workload's layer with every expert resident; CPU copies of the experts named in `keep`."""
+    import torch
+    import ek_hip
+    from ek_hip import workloads as wl
+    w_dtype = torch.float8_e4m3fn if w.fp8_block else torch.int8 if w.w8 else w.act_dtype
+    layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype, w_dtype=w_dtype,
+                            max_tokens=max_tokens)
+    kept = {}
+    for e in range(w.n_experts):
+        ew = wl.make_expert(w, e, device="cuda")
+        layer.set_expert(e, ew)
+        if e in keep:
+            kept[e] = ek_hip.ExpertWeight(*[None if t is None else t.cpu() for t in
+                                            (ew.up_w, ew.gate_w, ew.down_w, ew.up_scale, ew.gate_scale, ew.down_scale)])
+        del ew
+    return layer, kept
+
+
+def sample_experts(w, n):
+    """n experts spread evenly over the workload's experts ordered by load."""
+    import torch
+    from ek_hip import workloads as wl
+    if n <= 0:
+        return []
+    ids, _ = wl.make_routing(w)
+    counts = torch.bincount(ids.reshape(-1).long(), minlength=w.n_experts)
+    order = torch.argsort(counts, descending=True, stable=True).tolist()
+    return sorted(order[:: max(1, w.n_experts // n)][:n])
+
+
+def compact(m, roof, layer_fig, config):
+    """One of the other configurations as a short object: time, throughput, the roof that binds the whole
+    call and the fraction of it reached, the dominant kernel's own fraction, the gates that were held."""
+    bound = "hbm" if layer_fig["hbm_frac"] >= layer_fig["mfma_frac"] else "mfma"
+    out = {"config": config, "ms_per_step": m["step_s"] * 1e3, "value": m["w"].pairs / m["step_s"], "unit": "pairs/s",
+           "bound": bound, "frac": layer_fig[bound + "_frac"], "hbm_frac": layer_fig["hbm_frac"], "mfma_frac": layer_fig["mfma_frac"],
+           "dominant_kernel": {"kernel": roof["kernel"], "us": roof["kernel_us"], "frac": roof["frac"], "bound": roof["bound"]},
+           "phase_us": layer_fig["phase_us"], "routing_bit_exact": True}
+    if m["graph_s"] is not None:
+        out["graph_replay_ms_per_step"] = m["graph_s"] * 1e3
+        out["graph_replay_frac"] = out["frac"] * m["step_s"] / m["graph_s"]
+    if m["parity"] is not None:
+        out["parity"] = {k: m["parity"][k] for k in ("max_err_over_rms", "over_frac", "elements", "tokens")}
+    return out
+
+
+def cpu_cores():
+    return os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"])
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2", "c3", "c4", "c5"],
+                    help="all (default): c3 as the headline, c4 on the same experts as `prefill`, then c1, c2 and c5 "
+                         "as short objects; one name: that configuration alone")
     ap.add_argument("--weights", choices=["config", "fp8", "bf16"], default="config",
                     help="fp8: the c3 / c4 layer with fp8 e4m3fn weights and 128x128 block scales kept as a "
                          "DeepSeek-V3 checkpoint stores them, instead of the configuration's int8 per channel; "
                          "bf16: the same layer with 16-bit weights")
     ap.add_argument("--cpu-experts", type=int, default=96, help="experts in the CPU-baseline sample (0 = skip)")
+    ap.add_argument("--cpu-experts-prefill", type=int, default=16,
+                    help="experts in the prefill configuration's CPU-baseline sample (0 = skip)")
     ap.add_argument("--tokens", type=int, default=0,
                     help="run the workload's layer at another token count (a parity-test style variation, e.g. other "
                          "decode batch sizes of c3; implies --no-prefill)")
@@ -290,6 +388,7 @@ def main():
                     help="with --workload c3: do not also measure the c4 prefill call on the same experts")
     ap.add_argument("--no-parity", dest="parity", action="store_false", help="skip the oracle's output gate before timing")
     ap.add_argument("--no-peaks", dest="peaks", action="store_false", help="skip the copy / read / MFMA microbenchmarks")
+    ap.add_argument("--graph", action="store_true", help="also time the call replayed from a graph of the caller's")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
                          "used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -301,50 +400,37 @@ def main():
     import torch
     import ek_hip
     from ek_hip import workloads as wl
+    from dataclasses import replace
 
     ek_hip.load()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
-    w = wl.resolve(wl.CONFIGS[args.workload])
+    everything = args.workload == "all"
+    w = wl.resolve(wl.CONFIGS["c3" if everything else args.workload])
     if args.weights == "fp8":
         assert w.w8, "--weights fp8 applies to the W8A16 configurations (c3, c4)"
-        from dataclasses import replace
         w = replace(w, fp8_block=True)
     if args.weights == "bf16":
         assert w.w8, "--weights bf16 applies to the W8A16 configurations (c3, c4)"
-        from dataclasses import replace
         w = replace(w, w8=False)
     if args.tokens > 0:
         assert w.n_layers == 1, "--tokens applies to the single-layer configurations"
-        from dataclasses import replace
         w = replace(w, tokens=args.tokens, name=f"{w.name}_T{args.tokens}")
         args.prefill = False
     if w.n_layers > 1:
-        return bench_chain(args, w, dev)
+        print(json.dumps(bench_chain(args, w, dev)))
+        return
     # the decode configuration the metric is quoted on and the prefill configuration hold the same
-    # 256 experts: the default run measures both on one layer object, decode first
+    # 256 experts: both are measured on one layer object, decode first
     also = None
-    if args.workload == "c3" and args.prefill:
-        from dataclasses import replace
+    if w.name.startswith("c3") and args.prefill:
         also = replace(wl.C4, fp8_block=w.fp8_block, w8=w.w8)
-    w_dtype = torch.float8_e4m3fn if w.fp8_block else torch.int8 if w.w8 else w.act_dtype
-    layer = ek_hip.HipLayer(w.hidden, w.inter, w.n_experts, w.top_k, act_dtype=w.act_dtype, w_dtype=w_dtype,
-                            max_tokens=max(w.tokens, also.tokens if also else 0))
-    ids, gw = wl.make_routing(w)
-    counts = torch.bincount(ids.reshape(-1).long(), minlength=w.n_experts)
-    order = torch.argsort(counts, descending=True, stable=True).tolist()
-    sample_ids = sorted(order[:: max(1, w.n_experts // max(args.cpu_experts, 1))][: args.cpu_experts]) if args.cpu_experts else []
-    ws_sample = {}
-    for e in range(w.n_experts):
-        ew = wl.make_expert(w, e, device="cuda")
-        layer.set_expert(e, ew)
-        if e in sample_ids:
-            ws_sample[e] = ek_hip.ExpertWeight(*[None if t is None else t.cpu() for t in
-                                                 (ew.up_w, ew.gate_w, ew.down_w, ew.up_scale, ew.gate_scale, ew.down_scale)])
-        del ew
+    sample_ids = sample_experts(w, args.cpu_experts)
+    sample_ids_p = sample_experts(also, args.cpu_experts_prefill) if also is not None else []
+    layer, kept = build_layer(w, max(w.tokens, also.tokens if also else 0), keep=set(sample_ids) | set(sample_ids_p))
     stream = torch.cuda.Stream()          # the calls are enqueue-only on a stream of the caller's
     calibration_copy(args, dev)
-    m = time_layer(layer, w, args, dev, stream)
+    m = time_layer(layer, w, args, dev, stream, graph=args.graph)
     roof, layer_fig, config = roofline_of(m)
     out = {
         "metric": "token-expert pairs/s on 1 MI355X (DSv3 W8A16 layer); % HBM / MFMA roofline",
@@ -358,8 +444,11 @@ def main():
         "roofline": roof,
         "layer": layer_fig,
     }
+    if m["graph_s"] is not None:
+        out["graph_replay_ms_per_step"] = m["graph_s"] * 1e3
     if m["parity"] is not None:
         out["parity"] = m["parity"]
+    torch.set_num_threads(cpu_cores())
     if also is not None:
         mp = time_layer(layer, also, args, dev, stream)
         roof_p, layer_p, config_p = roofline_of(mp)
@@ -371,6 +460,13 @@ def main():
                                                  "peak": MFMA_PEAK_16 / 1e12, "unit": "TFLOP/s", "frac": layer_p["mfma_frac"]}
         if mp["parity"] is not None:
             out["prefill"]["parity"] = mp["parity"]
+        if sample_ids_p:
+            v, pairs, iters = cpu_baseline(also, {e: kept[e] for e in sample_ids_p}, mp["x"], mp["ids"], mp["gw"], max_runs=1)
+            out["prefill"]["cpu_baseline"] = {
+                "value": v, "unit": "pairs/s", "cores": torch.get_num_threads(), "kind": "port", "cpu_model": cpu_model(),
+                "sample": f"pairs routed to {len(sample_ids_p)} of {also.n_experts} experts spread evenly over the experts "
+                          f"ordered by load ({pairs} of {also.pairs} pairs), one run, libtorch CPU ops, weights pre-cast to "
+                          f"{str(also.act_dtype).replace('torch.', '')}"}
     if args.peaks:
         from ek_hip import _capi as C
         import ctypes
@@ -382,16 +478,33 @@ def main():
                         "mfma_bf16_with_int8_dequant_TFLOPs": pk.mfma_bf16_dequant_tflops,
                         "source": "in-library microkernels (csrc/ek_peaks.hip), measured in this run",
                         "published": {"hbm_GBps": HBM_PEAK / 1e9, "mfma_bf16_TFLOPs": MFMA_PEAK_16 / 1e12}}
-    if args.cpu_experts:
-        cores = os.cpu_count() if not os.environ.get("OMP_NUM_THREADS") else int(os.environ["OMP_NUM_THREADS"])
-        torch.set_num_threads(cores)
-        v, pairs, iters = cpu_baseline(w, ws_sample, m["x"], m["ids"], m["gw"])
+    if sample_ids:
+        v, pairs, iters = cpu_baseline(w, {e: kept[e] for e in sample_ids}, m["x"], m["ids"], m["gw"])
         out["cpu_baseline"] = {"value": v, "unit": "pairs/s", "cores": torch.get_num_threads(), "kind": "port",
                                "cpu_model": cpu_model(),
-                               "sample": f"pairs routed to {len(ws_sample)} of {w.n_experts} experts ({pairs} pairs), "
+                               "sample": f"pairs routed to {len(sample_ids)} of {w.n_experts} experts ({pairs} pairs), "
                                          f"median of {iters} runs, libtorch CPU ops, weights pre-cast to "
                                          f"{str(w.act_dtype).replace('torch.', '')}"}
     layer.close()
+    del layer, kept, m
+    if everything:
+        # the other three configurations, each built, gated, timed and freed in turn
+        torch.cuda.empty_cache()
+        for name in ("c1", "c2"):
+            wo = wl.resolve(wl.CONFIGS[name])
+            lo, _ = build_layer(wo, wo.tokens)
+            mo = time_layer(lo, wo, args, dev, stream, graph=True)
+            out[name] = compact(mo, *roofline_of(mo))
+            lo.close()
+            del lo, mo
+            torch.cuda.empty_cache()
+        c5 = bench_chain(args, wl.resolve(wl.CONFIGS["c5"]), dev)
+        out["c5"] = {"config": c5["config"], "ms_per_step": c5["ms_per_step"], "value": c5["value"], "unit": "pairs/s",
+                     "bound": c5["roofline"]["bound"], "frac": c5["roofline"]["frac"], "hbm_frac": c5["layer"]["hbm_frac"],
+                     "mfma_frac": c5["layer"]["mfma_frac"], "eager_ms_per_step": c5["layer"]["eager_ms_per_step"],
+                     "graph_equals_eager_bitwise": True, "routing_bit_exact": True}
+        if "parity" in c5:
+            out["c5"]["parity"] = {k: c5["parity"][k] for k in ("max_err_over_rms", "over_frac", "elements", "tokens", "of")}
     print(json.dumps(out))
 
 
