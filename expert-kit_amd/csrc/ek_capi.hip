@@ -97,7 +97,17 @@ struct Workspace {
     // a list of its own for a shared expert's segment cut into wide streaming items
     ek::WorkItem *wide_items = nullptr;
     int32_t *wide_count = nullptr;           // [kNumLists], only [kListStream] is used
+    // a shared expert whose intermediate size is not the routed experts': lists of its own (its
+    // launches have other shapes) and its own intermediate buffer [T, shared_inter]
+    ek::WorkLists slists{};
+    int64_t slist_cap[ek::kNumLists] = {0, 0, 0, 0};
+    void *hs = nullptr;
 };
+// capacities of a shared segment's own lists for at most T rows (see launch_segment_lists)
+inline int64_t shared_list_cap(int l, int64_t T)
+{
+    return l == ek::kListStream ? T / 16 + 2 : l == ek::kListT128 ? T / 128 + 2 : 1;
+}
 
 struct ek_layer {
     ek_cfg cfg{};             // as the kernels see it: hidden and inter rounded up to what they need
@@ -153,6 +163,9 @@ struct ek_layer {
     // the two FFN kernel families work on disjoint items, so their chains run side by side
     hipStream_t side_stream = nullptr;
     hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+    hipEvent_t ev_sfork = nullptr, ev_sjoin = nullptr;   // around the launches of a shared expert of another width
+    int64_t shared_inter = 0;                // that shared expert's intermediate size (0: none loaded, or the routed experts')
+    size_t hs_bytes = 0;
     // Streams that share a hardware queue run their kernels one after the other (the runtime
     // spreads streams over a few queues in turn), which would undo the fork: the side stream
     // comes from a pool, and for every caller's stream the library finds once, by timing an idle
@@ -239,7 +252,9 @@ void free_layer(ek_layer *L)
     void *bufs[] = {L->d_slabs, L->ws.counts, L->ws.offsets, L->ws.perm, L->ws.inv_perm, L->ws.row_token,
                     L->ws.block_hist, L->ws.err, L->ws.h, L->ws.yp, L->st_x, L->st_w, L->st_y, L->st_xp,
                     L->d_activation, L->st_ids, L->st_raw, L->rt_ids, L->rt_w, L->st_logits, L->st_bias, L->ws.lists.count, L->ws.lists.items[0], L->ws.lists.items[1],
-                    L->ws.lists.items[2], L->ws.lists.items[3], L->ws.wide_items, L->ws.wide_count};
+                    L->ws.lists.items[2], L->ws.lists.items[3], L->ws.wide_items, L->ws.wide_count,
+                    L->ws.slists.count, L->ws.slists.items[0], L->ws.slists.items[1], L->ws.slists.items[2],
+                    L->ws.slists.items[3], L->ws.hs};
     for (void *p : bufs) if (p) (void)hipFree(p);
     for (hipEvent_t ev : L->events) (void)hipEventDestroy(ev);
     if (L->h_err) (void)hipHostFree(L->h_err);
@@ -251,6 +266,8 @@ void free_layer(ek_layer *L)
     if (L->stream) (void)hipStreamDestroy(L->stream);
     if (L->load_stream) (void)hipStreamDestroy(L->load_stream);
     if (L->side_stream) (void)hipStreamDestroy(L->side_stream);
+    if (L->ev_sfork) (void)hipEventDestroy(L->ev_sfork);
+    if (L->ev_sjoin) (void)hipEventDestroy(L->ev_sjoin);
     if (L->ev_fork) (void)hipEventDestroy(L->ev_fork);
     if (L->ev_join) (void)hipEventDestroy(L->ev_join);
     for (hipStream_t ps : L->side_pool) if (ps && ps != L->side_stream) (void)hipStreamDestroy(ps);
@@ -340,6 +357,11 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
     A((void **)&L->ws.lists.count, sizeof(int32_t) * ek::kNumLists, "work list counts");
     A((void **)&L->ws.wide_items, sizeof(ek::WorkItem) * kSharedWideItems, "shared expert's work list");
     A((void **)&L->ws.wide_count, sizeof(int32_t) * ek::kNumLists, "shared expert's work list count");
+    A((void **)&L->ws.slists.count, sizeof(int32_t) * ek::kNumLists, "shared expert's work list counts");
+    for (int l = 0; l < ek::kNumLists; ++l) {
+        L->ws.slist_cap[l] = shared_list_cap(l, cfg->max_tokens);
+        A((void **)&L->ws.slists.items[l], sizeof(ek::WorkItem) * L->ws.slist_cap[l], "shared expert's work list");
+    }
     for (int l = 0; l < ek::kNumLists; ++l) {
         // A layer call's lists hold at most one remainder item per expert (list_capacity); a grouped
         // launch of per-expert calls may name an expert many times, each call a segment of its own,
@@ -370,6 +392,8 @@ ek_status create_layer(const ek_cfg *cfg, int64_t pmax, ek_layer **out)
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->load_stream, hipStreamNonBlocking);
         if (e == hipSuccess) e = hipStreamCreateWithFlags(&L->side_stream, hipStreamNonBlocking);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_sfork, hipEventDisableTiming);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_sjoin, hipEventDisableTiming);
         if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_fork, hipEventDisableTiming);
         if (e == hipSuccess) e = hipEventCreateWithFlags(&L->ev_join, hipEventDisableTiming);
         L->side_pool[0] = L->side_stream;
@@ -467,10 +491,11 @@ ek_status stage_raw(ek_layer *L, const void *src, int mem, size_t bytes, size_t 
     return EK_OK;
 }
 
+// inter_e: the expert's intermediate size (the layer's; a shared expert may have another)
 ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
-                            const ek_weight_desc *gate, const ek_weight_desc *down)
+                            const ek_weight_desc *gate, const ek_weight_desc *down, int64_t inter_e = 0)
 {
-    const int64_t H = L->cfg.hidden, I = L->cfg.inter;
+    const int64_t H = L->cfg.hidden, I = inter_e > 0 ? inter_e : L->cfg.inter;
     EK_TRY(check_desc(up, "up", I, H, L->wmode));
     EK_TRY(check_desc(gate, "gate", I, H, L->wmode));
     EK_TRY(check_desc(down, "down", H, I, L->wmode));
@@ -564,8 +589,40 @@ ek_status set_expert_locked(ek_layer *L, int32_t e, const ek_weight_desc *up,
         }
         L->expert_mem[e] = mem;
         L->h_slabs[e] = slab;
+        if (e == L->cfg.n_experts) L->shared_inter = I != L->cfg.inter ? I : 0;
     }
     if (old) (void)hipFree(old);
+    return EK_OK;
+}
+
+// A shared expert whose intermediate size is not the routed experts' (DeepSeek's shared_experts has
+// moe_intermediate_size * n_shared_experts channels: expertkit_torch/models/deepseek_v3/model.py:57-61):
+// its size must suit the kernels as the layer's own does, and the layer's workspace gets an
+// intermediate buffer of that width.
+ek_status prepare_shared_width(ek_layer *L, const ek_weight_desc *up, int64_t *inter_e)
+{
+    *inter_e = 0;
+    if (!up || up->rows == L->cfg.inter) return EK_OK;
+    const int64_t Is = up->rows;
+    if (L->padded)
+        return fail(EK_INVALID_INPUT, "a shared expert of another intermediate size (%lld) needs a layer whose hidden and "
+                    "inter are multiples of 64 (128 with one-byte weights)", (long long)Is);
+    if (Is < (L->w8 ? 128 : 64) || Is % 64)
+        return fail(EK_INVALID_INPUT, "the shared expert's intermediate size (%lld) must be a multiple of 64, at least %d",
+                    (long long)Is, L->w8 ? 128 : 64);
+    if (ek::block_scaled(L->wmode) && Is > 8192)
+        return fail(EK_INVALID_INPUT, "block-scaled layers hold at most 64 scale blocks per row: the shared expert's "
+                    "intermediate size (%lld) must not exceed 8192", (long long)Is);
+    const size_t need = (size_t)L->cfg.max_tokens * Is * 2;
+    std::lock_guard<std::mutex> lk(L->mu);
+    if (need > L->hs_bytes) {
+        EK_HIP(hipDeviceSynchronize());
+        if (L->ws.hs) (void)hipFree(L->ws.hs);
+        L->ws.hs = nullptr; L->hs_bytes = 0;
+        EK_TRY(dev_alloc(&L->ws.hs, need, "shared expert's intermediate rows"));
+        L->hs_bytes = need;
+    }
+    *inter_e = Is;
     return EK_OK;
 }
 
@@ -720,8 +777,14 @@ size_t carve_workspace(const ek_layer *L, int64_t T, unsigned char *base, size_t
         W->list_cap[l] = ek::list_capacity(l, rows, E + 1) + (l == ek::kListStream ? 264 : 1);
         W->lists.items[l] = (ek::WorkItem *)take(sizeof(ek::WorkItem) * (size_t)W->list_cap[l]);
     }
+    W->slists.count = (int32_t *)take(sizeof(int32_t) * ek::kNumLists);
+    for (int l = 0; l < ek::kNumLists; ++l) {
+        W->slist_cap[l] = shared_list_cap(l, T);
+        W->slists.items[l] = (ek::WorkItem *)take(sizeof(ek::WorkItem) * (size_t)W->slist_cap[l]);
+    }
     W->h = take((size_t)rows * L->cfg.inter * 2);
     W->yp = take((size_t)rows * L->cfg.hidden * 2);
+    W->hs = L->shared_inter ? take((size_t)T * L->shared_inter * 2) : nullptr;
     return off;
 }
 
@@ -1062,6 +1125,7 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
 // How a call's shared-expert segment (if the layer has one) is cut.
 struct SharedCut {
     bool shared, streamed, wide;
+    bool own;        // another intermediate size than the routed experts': lists, launches and buffer of its own
 };
 SharedCut shared_cut(const ek_layer *L, int64_t T)
 {
@@ -1069,6 +1133,7 @@ SharedCut shared_cut(const ek_layer *L, int64_t T)
     c.shared = L->expert_mem[L->cfg.n_experts] != nullptr && T > 0;
     c.streamed = c.shared && T <= kSharedStreamRows;
     c.wide = c.shared && !c.streamed && T <= kSharedWideRows;
+    c.own = c.shared && L->shared_inter != 0;
     return c;
 }
 
@@ -1080,7 +1145,9 @@ ek_status enqueue_route(ek_layer *L, const Workspace &W, const int32_t *ids, int
     const int64_t P = T * L->cfg.top_k;
     ek::launch_pack(pack_args(L, W, ids, P, true), s);
     const SharedCut sc = shared_cut(L, T);
-    if (sc.wide) {
+    if (sc.own) {
+        ek::launch_segment_lists(W.slists, E, (int32_t)P, (int32_t)T, W.row_token, sc.streamed ? 1 : sc.wide ? 2 : 0, s);
+    } else if (sc.wide) {
         ek::WorkLists own = W.lists;
         own.items[ek::kListStream] = W.wide_items;
         own.count = W.wide_count;
@@ -1089,6 +1156,44 @@ ek_status enqueue_route(ek_layer *L, const Workspace &W, const int32_t *ids, int
         ek::launch_append_segment(W.lists, E, (int32_t)P, (int32_t)T, W.row_token, sc.streamed ? 1 : 0, s);
     }
     EK_HIP(hipGetLastError());
+    return EK_OK;
+}
+
+// A shared expert of another intermediate size: both stages over its own lists (W.slists: rows
+// P .. P+T-1 of the packed order, token t at row P + t), with its own shapes, on the side stream
+// beside the routed pairs' launches; the caller's stream waits for L->ev_sjoin before the combine.
+// The intermediate rows live in W.hs [T, shared_inter]: the kernels index rows by packed position,
+// so they get the address row P would have if the buffer started at row 0.
+ek_status enqueue_shared_own(ek_layer *L, const Workspace &W, const void *x, int64_t P, int64_t T, const SharedCut &sc,
+                             hipStream_t s)
+{
+    const int64_t H = L->cfg.hidden, Is = L->shared_inter;
+    if (!W.hs) return fail(EK_INTERNAL, "no intermediate buffer for the shared expert");
+    hipStream_t side = pick_side_stream(L, s);
+    EK_HIP(hipEventRecord(L->ev_sfork, s));
+    EK_HIP(hipStreamWaitEvent(side, L->ev_sfork, 0));
+    ek::FfnArgs a1;
+    a1.x = x; a1.x_stride = H; a1.rows = W.row_token; a1.slabs = L->d_slabs;
+    a1.out = (char *)W.hs - (size_t)P * Is * 2; a1.out_stride = Is;
+    a1.N = (int32_t)Is; a1.Kdim = (int32_t)H; a1.lists = W.slists;
+    ek::FfnArgs a2 = a1;
+    a2.x = a1.out; a2.x_stride = Is; a2.rows = nullptr; a2.out = W.yp; a2.out_stride = H;
+    a2.N = (int32_t)H; a2.Kdim = (int32_t)Is;
+    int64_t cap[ek::kNumLists];
+    for (int l = 0; l < ek::kNumLists; ++l) cap[l] = std::min<int64_t>(shared_list_cap(l, T), W.slist_cap[l]);
+    for (int stage = 1; stage <= 2; ++stage) {
+        const ek::FfnArgs &a = stage == 1 ? a1 : a2;
+        if (sc.streamed) {
+            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, (T + 15) / 16, false, side));
+        } else if (sc.wide) {
+            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, (T + ek::kWideRows - 1) / ek::kWideRows, true, side));
+        } else {
+            cap[ek::kListStream] = 1;        // the usual cut leaves at most one item of <= 16 rows
+            EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, false, side));
+            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, 1, false, side));
+        }
+    }
+    EK_HIP(hipEventRecord(L->ev_sjoin, side));
     return EK_OK;
 }
 
@@ -1119,13 +1224,15 @@ ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const 
     // item re-reads the expert's weights, so beyond that it is cut into items of up to 64 rows,
     // which the streaming kernel's wide form takes in a launch of its own.
     const SharedCut sc = shared_cut(L, T);
-    const bool shared = sc.shared, shared_streamed = sc.streamed, shared_wide = sc.wide;
+    const bool shared = sc.shared, shared_streamed = sc.streamed && !sc.own, shared_wide = sc.wide && !sc.own;
     if (ev) EK_HIP(hipEventRecord(ev[1], s));
+    if (P > 0 && sc.own) EK_TRY(enqueue_shared_own(L, W, x, P, T, sc, s));     // on the side stream, joined before the combine
     if (P > 0) {
-        const bool in_lists = shared && !shared_wide;   // the shared segment's items sit in the routed pairs' lists
+        const bool in_lists = shared && !shared_wide && !sc.own;   // the shared segment's items sit in the routed pairs' lists
         EK_TRY(enqueue_ffn(L, W, x, W.row_token, W.yp, in_lists ? P + T : P, in_lists ? E + 1 : E, s, ev, 0,
                            shared_streamed ? (T + 15) / 16 : 0,
                            shared_wide ? (T + ek::kWideRows - 1) / ek::kWideRows : 0));
+        if (sc.own) EK_HIP(hipStreamWaitEvent(s, L->ev_sjoin, 0));
         if (ev) EK_HIP(hipEventRecord(ev[3], s));
         if (before_combine) EK_TRY((*before_combine)());
         ek::CombineArgs c;
@@ -1221,7 +1328,9 @@ ek_status ek_layer_set_expert(ek_layer *layer, int32_t expert, const ek_weight_d
             if (!up || !gate || !down) return fail(EK_WEIGHT_NOT_FOUND, "a weight matrix is missing");
             return set_expert_padded(layer, expert, up, gate, down);
         }
-        return set_expert_locked(layer, expert, up, gate, down);
+        int64_t inter_e = 0;
+        if (expert == layer->cfg.n_experts) EK_TRY(prepare_shared_width(layer, up, &inter_e));
+        return set_expert_locked(layer, expert, up, gate, down, inter_e);
     )
 }
 
@@ -1240,6 +1349,7 @@ ek_status ek_layer_remove_expert(ek_layer *layer, int32_t expert)
             if (!old) return fail(EK_EXPERT_NOT_FOUND, "expert %d is not loaded", expert);
             EK_HIP(hipDeviceSynchronize());
             layer->expert_mem[expert] = nullptr;
+            if (expert == layer->cfg.n_experts) layer->shared_inter = 0;
             layer->h_slabs[expert] = ek::ExpertSlab{nullptr, nullptr, nullptr, nullptr, nullptr};
             EK_HIP(hipMemcpy(layer->d_slabs + expert, &layer->h_slabs[expert], sizeof(ek::ExpertSlab),
                              hipMemcpyHostToDevice));

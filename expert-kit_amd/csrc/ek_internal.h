@@ -133,6 +133,11 @@ constexpr int kMaxExperts = 1024;
 void launch_pack(const PackArgs &a, hipStream_t s);
 // work lists for one segment [0, n) of expert e (per-expert forward)
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool wide, hipStream_t s);
+// lists that hold the one segment (expert, rows row0 .. row0+n-1) and nothing else; mode 0: the usual
+// cut, 1: 16-row streaming items, 2: streaming items of up to kWideRows rows.  row_token, if given,
+// receives row0 + t -> t.
+void launch_segment_lists(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token, int mode,
+                          hipStream_t s);
 // appends the segment (expert, rows row0 .. row0+n-1) to the lists pack has built and maps
 // its rows to tokens 0 .. n-1.  as_stream: 0 the usual cut; 1 all rows as 16-row streaming items;
 // 2 all rows as streaming items of up to kWideRows rows, which replace the streaming list (the

@@ -172,22 +172,34 @@ __global__ __launch_bounds__(1024) void pack_scan_kernel(PackArgs a)
     }
 }
 
-__global__ void single_lists_kernel(WorkLists l, int32_t e, int32_t n, int32_t wide)
+// Work lists that hold one segment and nothing else: rows row0 .. row0+n-1 of expert e.
+// mode 0: the usual cut; 1: 16-row streaming items; 2: streaming items of up to kWideRows rows.
+// row_token, if given, maps the segment's rows to tokens 0 .. n-1.
+__global__ __launch_bounds__(256) void segment_lists_kernel(WorkLists l, int32_t e, int32_t row0, int32_t n,
+                                                            int32_t *row_token, int32_t mode)
 {
-    if (wide) {
-        int32_t k = 0;
-        for (int32_t r0 = 0; r0 < n; r0 += kWideRows, ++k)
-            l.items[kListStream][k] = WorkItem{e, r0, min(kWideRows, n - r0), 0};
-        l.count[kListT128] = l.count[kListT64] = l.count[kListT32] = 0;
-        l.count[kListStream] = k;
+    if (row_token)
+        for (int32_t t = threadIdx.x; t < n; t += 256) row_token[row0 + t] = t;
+    if (mode) {
+        const int32_t per = mode == 2 ? kWideRows : 16, items = (n + per - 1) / per;
+        for (int32_t t = threadIdx.x; t < items; t += 256)
+            l.items[kListStream][t] = WorkItem{e, row0 + t * per, min(per, n - t * per), 0};
+        if (threadIdx.x == 0) {
+            l.count[kListT128] = l.count[kListT64] = l.count[kListT32] = 0;
+            l.count[kListStream] = items;
+        }
         return;
     }
     const SegmentCut c = cut_segment(n);
-    if (n > 0) emit_items(l, e, 0, n, 0, 0, 0, 0);
-    l.count[kListT128] = c.n128;
-    l.count[kListT64] = c.n64;
-    l.count[kListT32] = c.n32;
-    l.count[kListStream] = c.ns;
+    const int32_t full = n >> 7;
+    for (int32_t t = threadIdx.x; t < full; t += 256) l.items[kListT128][t] = WorkItem{e, row0 + t * 128, 128, 0};
+    if (threadIdx.x == 0) {
+        if (n & 127) emit_items(l, e, row0 + full * 128, n & 127, full, 0, 0, 0);    // the remainder, into its class
+        l.count[kListT128] = c.n128;
+        l.count[kListT64] = c.n64;
+        l.count[kListT32] = c.n32;
+        l.count[kListStream] = c.ns;
+    }
 }
 
 __global__ __launch_bounds__(256) void append_segment_kernel(WorkLists l, int32_t e, int32_t row0, int32_t n,
@@ -235,7 +247,13 @@ void launch_append_segment(const WorkLists &lists, int32_t expert, int32_t row0,
 
 void launch_single_lists(const WorkLists &lists, int32_t expert, int32_t n, bool wide, hipStream_t s)
 {
-    hipLaunchKernelGGL(single_lists_kernel, dim3(1), dim3(1), 0, s, lists, expert, n, wide ? 1 : 0);
+    hipLaunchKernelGGL(segment_lists_kernel, dim3(1), dim3(256), 0, s, lists, expert, 0, n, (int32_t *)nullptr, wide ? 2 : 0);
+}
+
+void launch_segment_lists(const WorkLists &lists, int32_t expert, int32_t row0, int32_t n, int32_t *row_token, int mode,
+                          hipStream_t s)
+{
+    hipLaunchKernelGGL(segment_lists_kernel, dim3(1), dim3(256), 0, s, lists, expert, row0, n, row_token, mode);
 }
 
 __global__ __launch_bounds__(kPackThreads) void pack_rank_kernel(PackArgs a, int nbits)

@@ -174,8 +174,12 @@ ek_status ek_layer_destroy(ek_layer *layer);
  * (expertkit_torch/models/deepseek_v3/model.py:57-61,152); the reference runs
  * it on the attention side.  Once loaded here it is one more segment of the
  * grouped launch (all T tokens, gate weight 1) and ek_layer_forward returns
- * round(routed + shared) in the activation dtype.  Its shape must be the
- * routed experts' (moe_intermediate_size * n_shared_experts == cfg.inter). */
+ * round(routed + shared) in the activation dtype.  Its intermediate size may
+ * differ from the routed experts' (moe_intermediate_size * n_shared_experts:
+ * DeepSeek-V2-Lite has two shared experts): a multiple of 64, at least 128 with
+ * one-byte weights; its segment then gets launches of its own beside the routed
+ * pairs'.  (A layer whose own sizes need padding takes a shared expert of the
+ * routed experts' shape only.) */
 #define EK_SHARED_EXPERT (-1)
 
 /* ExpertDB::insert after ExpertBackend::build (ffn/mod.rs:23-36;
