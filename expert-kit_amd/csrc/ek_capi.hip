@@ -975,6 +975,8 @@ ek::PackArgs pack_args(ek_layer *L, const Workspace &W, const int32_t *ids, int6
 hipStream_t pick_side_stream(ek_layer *L, hipStream_t s)
 {
     for (const auto &p : L->side_for) if (p.first == s) return p.second;
+    // (the choice is remembered per handle; a stream that was destroyed and another created at the same
+    // address inherits it: either choice is correct, a poor one costs the overlap only)
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(s, &cs) != hipSuccess) { (void)hipGetLastError(); return L->side_stream; }
     if (cs != hipStreamCaptureStatusNone) return L->side_stream;

@@ -23,25 +23,53 @@ __global__ __launch_bounds__(256) void combine_kernel(CombineArgs a)
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-    // the rows of up to 8 slots are requested together, then added in slot order
+    // The rows of up to 8 slots are requested together, then added in slot order.  Every load is
+    // unconditional (slots past K and pairs without a row re-read a valid address and are left out
+    // of the sum): conditional loads became a chain of branches in which each load waited for the
+    // one before it.  The rows are read once: non-temporal loads.  (8192 tokens of the
+    // DeepSeek-V3 layer on MI355X: 235 us with the branches, 216 with non-temporal loads alone.)
     for (int k0 = 0; k0 < a.K; k0 += 8) {
         int32_t pos[8];
         float wv[8];
+        bool valid[8];
         V8 v[8];
+        if ((a.K & 7) == 0) {
+            // eight positions and eight gate weights as whole vectors (the addresses are the same for
+            // every lane: two to four scalar loads in flight together)
+            typedef int32_t I4 __attribute__((ext_vector_type(4)));
+            typedef float F4 __attribute__((ext_vector_type(4)));
+            typedef T T8 __attribute__((ext_vector_type(8)));
+            const I4 *ip = (const I4 *)(a.inv_perm + t * a.K + k0);
+            const I4 p0 = ip[0], p1 = ip[1];
+            if constexpr (WF32) {
+                const F4 *wp = (const F4 *)((const float *)a.w + t * a.K + k0);
+                const F4 w0 = wp[0], w1 = wp[1];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int k = k0 + j;
-            pos[j] = k < a.K ? a.inv_perm[t * a.K + k] : -1;
-            wv[j] = 0.f;
-            if (pos[j] >= 0)
+                for (int j = 0; j < 4; ++j) { wv[j] = w0[j]; wv[4 + j] = w1[j]; }
+            } else {
+                const T8 w8 = *(const T8 *)((const T *)a.w + t * a.K + k0);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) wv[j] = (float)w8[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { pos[j] = p0[j]; pos[4 + j] = p1[j]; }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) valid[j] = pos[j] >= 0;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int k = min(k0 + j, a.K - 1);
+                pos[j] = a.inv_perm[t * a.K + k];
                 wv[j] = WF32 ? ((const float *)a.w)[t * a.K + k] : (float)((const T *)a.w)[t * a.K + k];
+                valid[j] = k0 + j < a.K && pos[j] >= 0;
+            }
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j)
-            if (pos[j] >= 0) v[j] = *(const V8 *)((const T *)a.yp + (int64_t)pos[j] * a.H + c);
+            v[j] = __builtin_nontemporal_load((const V8 *)((const T *)a.yp + (int64_t)max(pos[j], 0) * a.H + c));
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            if (pos[j] < 0) continue;
+            if (!valid[j]) continue;       // (the same for every lane)
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 float p = wv[j] * (float)v[j][i];

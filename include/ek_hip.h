@@ -20,7 +20,12 @@
  *    source buffer may be released as soon as the call returns;
  *  - `stream` is a hipStream_t passed as void*.  NULL means "run on the
  *    library's own stream and return after the work has completed".  With a
- *    non-NULL stream and device pointers the call only enqueues work;
+ *    non-NULL stream and device pointers the call only enqueues work.  One
+ *    exception: the first call that forks work to a side stream on a stream
+ *    the layer has not seen before waits for that stream once on the host (a
+ *    few hundred microseconds: it times an idle kernel alone and beside itself
+ *    to find a side stream whose kernels really run beside the caller's);
+ *    the choice is remembered per stream handle;
  *  - all entry points may be called from any thread.  A layer has one
  *    workspace (routing tables, work lists, packed intermediates).  Host code
  *    that uses it runs under the layer's lock; on the device, every call makes

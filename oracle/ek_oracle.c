@@ -205,10 +205,10 @@ float eko_expf_wide(float x)
     const float y = fmaf(r * r, p, r) + 1.0f;
     return ldexpf(y, (int)n);
 }
-/* silu with the kernels' exp and a correctly rounded division (the kernels form the quotient with a
- * reciprocal and one residual correction; that the two agree after the storage rounding for every
- * 16-bit gate is what the GPU test over all gate values holds), and as eko_ffn forms it (libm),
- * for one fp32 gate value */
+/* silu as the kernels form it (their exp, eko_expf_wide's operations one for one, and a correctly
+ * rounded IEEE division) and as eko_ffn forms it (libm), for one fp32 gate value; that the two agree
+ * after the storage rounding for every 16-bit gate is held on the CPU, and that the kernels return
+ * this value for every gate by the GPU test over all gate values */
 float eko_silu_kernel_form(float g) { return g / (1.0f + eko_expf_wide(-g)); }
 float eko_silu_libm_form(float g) { return g / (1.0f + expf(-g)); }
 
