@@ -217,7 +217,8 @@ struct ek_chain {
     void *k_y = nullptr;
     int64_t k_T = -1;
     int32_t k_wdt = -1;
-    std::vector<uint8_t> k_shared;           // which layers had a shared expert when captured
+    std::vector<int64_t> k_shared;           // per layer when captured: -1 no shared expert, 0 one of the routed experts'
+                                             // shape, else its own intermediate size (launches and buffers of its own)
     std::mutex mu;
 };
 
@@ -2066,9 +2067,10 @@ ek_status ek_chain_forward(ek_chain *chain, const void *x, const int32_t *ids, c
             EK_TRY(enqueue_chain(chain, x, ids, w, w_f32, T, y, s));
         } else {
             // a shared expert adds launches to its layer: part of the key
-            std::vector<uint8_t> shared(L);
+            std::vector<int64_t> shared(L);
             for (int l = 0; l < L; ++l)
-                shared[l] = chain->layers[l]->expert_mem[chain->layers[l]->cfg.n_experts] != nullptr;
+                shared[l] = chain->layers[l]->expert_mem[chain->layers[l]->cfg.n_experts] != nullptr
+                                ? chain->layers[l]->shared_inter : -1;
             const bool same = chain->exec && chain->k_x == x && chain->k_ids == ids && chain->k_w == w &&
                               chain->k_y == y && chain->k_T == T && chain->k_wdt == w_dtype &&
                               chain->k_shared == shared;

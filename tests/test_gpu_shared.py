@@ -199,6 +199,15 @@ def test_shared_expert_of_another_width_in_a_chain(ek, cuda):
         got = chain.forward(x, ids, w, use_graph=True)
         assert torch.equal(got.view(torch.int16), step.view(torch.int16)), rep
         torch.cuda.synchronize()
+    # a shared expert of the routed experts' width in layer 0 instead: other launches, the graph is captured again
+    layers[0].set_shared_expert(wl.make_expert(wl.Workload("sc", H, I, 1, 1, 1, dt), E, layer=0, std=0.08))
+    step2 = x
+    for l in range(L):
+        step2 = layers[l].forward(step2, ids[l], w[l])
+    assert not torch.equal(step2, step)
+    for rep in range(2):
+        got = chain.forward(x, ids, w, use_graph=True)
+        assert torch.equal(got.view(torch.int16), step2.view(torch.int16)), rep
     chain.close()
     for layer in layers:
         layer.close()
