@@ -1,7 +1,8 @@
 """Twenty seeded draws of a layer with a shared expert (deepseek_v3/model.py:57-61,152: every token
 once, added to the rounded routed sum): weight kind, activation type, sizes, expert count, top-k and
 1 to 1500 tokens, so that the shared segment is met as 16-row streaming items, as 64-row ones on the
-side stream and as tiles, beside every mix of routed segments.  Held to the oracle's layer plus
+side stream and as tiles, beside every mix of routed segments; in half of the draws the shared
+expert is two or three times as wide as the routed ones (launches of its own).  Held to the oracle's layer plus
 add_shared by test_gpu_shared.py's bound, and to the same call on host tensors.
 EKSEED=n draws another twenty."""
 import os
@@ -25,15 +26,17 @@ def test_fuzz(ek, oracle, cuda, case):
     E, K = r(2, 24), r(1, 4)
     K = min(K, E)
     T = [r(1, 16), r(17, 64), r(65, 256), r(257, 1500)][r(0, 3)]
-    print(f"fuzz-shared seed={SEED} case={case} kind={kind} dt={dt} H={H} I={I} E={E} K={K} T={T}", flush=True)
+    n_shared = [1, 1, 2, 3][r(0, 3)]      # the shared expert has moe_intermediate_size * n_shared_experts channels
+    print(f"fuzz-shared seed={SEED} case={case} kind={kind} dt={dt} H={H} I={I} x{n_shared} E={E} K={K} T={T}", flush=True)
     if kind in KINDS:
         layer = ek.HipLayer(H, I, E, K, act_dtype=dt, max_tokens=T, **KINDS[kind])
-        ws = [make_block_expert(ek, H, I, 100 * case + e, kind) for e in range(5)]
+        ws = [make_block_expert(ek, H, I * (n_shared if e == 4 else 1), 100 * case + e, kind) for e in range(5)]
         ref_w = [ref_weights(oracle, ew, dt) for ew in ws]
     else:
         w = wl.Workload("t", H, I, E, K, T, dt, w8=kind == "i8")
         layer = ek.HipLayer(H, I, E, K, act_dtype=dt, w_dtype=torch.int8 if w.w8 else dt, max_tokens=T)
-        ws = [wl.make_expert(w, 100 * case + e, std=0.05) for e in range(5)]
+        ws = [wl.make_expert(w, 100 * case + e, std=0.05) for e in range(4)]
+        ws.append(wl.make_expert(wl.Workload("t", H, I * n_shared, E, K, T, dt, w8=w.w8), 100 * case + 4, std=0.05))
         cols = oracle_weights(oracle, dict(enumerate(ws)), 5, dt)
         ref_w = [tuple(c[i] for c in cols) for i in range(5)]
     for e in range(E):
