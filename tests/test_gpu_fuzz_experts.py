@@ -20,6 +20,9 @@ SEED = int(os.environ.get("EKSEED", "0"))
 @pytest.mark.parametrize("case", range(30))
 def test_fuzz(ek, oracle, cuda, case):
     g = torch.Generator().manual_seed(SEED * 1000 + case + 77)
+    # the default seed's draws assert the plain bound but for three (cases 1: 2.32e-2 / 2.29e-2 / 2.02e-2 on its
+    # three calls, 11: 2.30e-2, 29: 2.35e-2, each y_ref rounded to the output type); other seeds hold the wide gate
+    plain = SEED == 0 and case not in (1, 11, 29)
     r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
     kind = ["w16", "i8", "fp8", "int8"][r(0, 3)]
     dt = [torch.bfloat16, torch.float16][r(0, 1)]
@@ -49,10 +52,10 @@ def test_fuzz(ek, oracle, cuda, case):
     alone = []
     for e, x in zip(es, xs):
         got = layer.expert_forward(e, x.to(cuda))
-        ffn_gate(got, oracle.ffn(x, *ref_w[e], mode=2), f"fuzz-expert {case} n={x.shape[0]}", plain=False, small=2)
+        ffn_gate(got, oracle.ffn(x, *ref_w[e], mode=2), f"fuzz-expert {case} n={x.shape[0]}", plain=plain, small=2)
         alone.append(got)
     # grouped: one launch for all of them; rows alone and grouped differ at most by accumulation order
     outs = layer.experts_forward(es, [x.to(cuda) for x in xs])
     for e, x, o in zip(es, xs, outs):
-        ffn_gate(o, oracle.ffn(x, *ref_w[e], mode=2), f"fuzz-expert grouped {case} n={x.shape[0]}", plain=False, small=2)
+        ffn_gate(o, oracle.ffn(x, *ref_w[e], mode=2), f"fuzz-expert grouped {case} n={x.shape[0]}", plain=plain, small=2)
     layer.close()

@@ -59,7 +59,9 @@ def test_fuzz(ek, oracle, cuda, case):
     ref, counts, offsets, perm, inv, y3 = oracle.layer_forward(x, ids, gw, list(wu), list(wg), list(wd), mode=2, return_y3=True)
     y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True)
     assert torch.equal(rt.perm.cpu(), perm) and torch.equal(rt.counts.cpu(), counts)
-    layer_gate(y, ref, y3, gw, f"fuzz {case}", plain=False)
+    # the default seed's draws assert the plain bound but for six: cases 5 (3.13e-2 on 5 of 1.3 M outputs), 13
+    # (2.18e-2), 20 (2.22e-2), 22 (2.50e-2), 23 (2.14e-2), 36 (2.45e-2); other seeds hold the wide gate
+    layer_gate(y, ref, y3, gw, f"fuzz {case}", plain=SEED == 0 and case not in (5, 13, 20, 22, 23, 36))
     y2 = layer.forward(x, ids, gw)
     assert torch.equal(y2.view(torch.int16), y.cpu().view(torch.int16))
     layer.close()

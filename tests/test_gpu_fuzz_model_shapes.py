@@ -15,6 +15,9 @@ SHAPES = [(7168, 2048), (2048, 768), (2048, 1408), (5120, 1536), (4096, 1024)]
 @pytest.mark.parametrize("case", range(15))
 def test_fuzz(ek, oracle, cuda, case):
     g = torch.Generator().manual_seed(SEED * 1000 + case + 999)
+    # the default seed's draws assert the plain bound but for case 9 (2.17e-2 on one of 1.9 M outputs, y_ref rounded
+    # to the output type); other seeds hold the wide gate
+    plain = SEED == 0 and case != 9
     r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
     H, I = SHAPES[case % len(SHAPES)]
     kind = ["w16", "i8", "fp8"][(case // len(SHAPES)) % 3]
@@ -39,14 +42,14 @@ def test_fuzz(ek, oracle, cuda, case):
     es = [r(0, E - 1) for _ in sizes]
     refs = [oracle.ffn(x, *ref_w[e], mode=2) for e, x in zip(es, xs)]
     for e, x, ref in zip(es, xs, refs):
-        ffn_gate(layer.expert_forward(e, x.to(cuda)), ref, f"fuzz-model {case} n={x.shape[0]}", plain=False, small=2)
+        ffn_gate(layer.expert_forward(e, x.to(cuda)), ref, f"fuzz-model {case} n={x.shape[0]}", plain=plain, small=2)
     for o, ref in zip(layer.experts_forward(es, [x.to(cuda) for x in xs]), refs):
-        ffn_gate(o, ref, f"fuzz-model grouped {case} n={ref.shape[0]}", plain=False, small=2)
+        ffn_gate(o, ref, f"fuzz-model grouped {case} n={ref.shape[0]}", plain=plain, small=2)
     xa = torch.cat(xs)
     ids = torch.cat([torch.full((x.shape[0], 1), e, dtype=torch.int32) for e, x in zip(es, xs)])
     y = layer.forward(xa.to(cuda), ids.to(cuda), torch.ones(xa.shape[0], 1, dtype=dt, device=cuda))
     o0 = 0
     for x, ref in zip(xs, refs):
-        ffn_gate(y[o0:o0 + x.shape[0]], ref, f"fuzz-model layer {case} n={x.shape[0]}", plain=False, small=2)
+        ffn_gate(y[o0:o0 + x.shape[0]], ref, f"fuzz-model layer {case} n={x.shape[0]}", plain=plain, small=2)
         o0 += x.shape[0]
     layer.close()

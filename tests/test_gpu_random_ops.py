@@ -18,6 +18,11 @@ from test_gpu_parity import ffn_gate, layer_gate, oracle_weights
 pytestmark = pytest.mark.gpu
 
 H, I, E, K, TMAX = 256, 128, 6, 2, 96
+# Steps of the two walks whose gate call exceeds the plain bound 2e-2 * rms (small outputs of 64- to
+# 128-term contractions: 2.03e-2 .. 2.87e-2 on the layer steps 133, 134, 176, 189, 205, 217, 3.2e-2 and
+# 2.86e-2 on the one-expert steps 230 and 239, all but step 133 y_ref rounded to the output type); every
+# other step of either walk asserts the plain bound.
+OVER = (133, 134, 176, 189, 205, 217, 230, 239)
 
 
 @pytest.mark.parametrize("w8", [False, True])
@@ -84,7 +89,7 @@ def test_random_walk(ek, oracle, cuda, w8):
                 done["wire"] += 1
             if n:
                 wu, wg, wd = ref_ws()
-                ffn_gate(got, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: expert {e}, {n} rows", small=tails(n), plain=False)
+                ffn_gate(got, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: expert {e}, {n} rows", small=tails(n), plain=step not in OVER)
             assert tuple(got.shape) == (n, H)
         elif op == 5:                                                 # several per-expert calls, one launch
             among = sorted(loaded) if draw(0, 3) else list(range(E))
@@ -101,7 +106,7 @@ def test_random_walk(ek, oracle, cuda, w8):
             wu, wg, wd = ref_ws()
             for (e, n), x, out in zip(calls, xs, outs):
                 if n:
-                    ffn_gate(out, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: batch, expert {e}, {n} rows", small=tails(n), plain=False)
+                    ffn_gate(out, oracle.ffn(x, wu[e], wg[e], wd[e], mode=2), f"step {step}: batch, expert {e}, {n} rows", small=tails(n), plain=step not in OVER)
             done["experts"] += 1
         elif op in (6, 7, 8):                                         # the whole layer
             T = draw(0, TMAX)
@@ -124,7 +129,7 @@ def test_random_walk(ek, oracle, cuda, w8):
             if T:
                 wu, wg, wd = ref_ws()
                 ref, _, _, _, _, y3 = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=2, return_y3=True)
-                layer_gate(y, ref, y3, gw, f"step {step}: layer, T={T}", small=tails(T), plain=False)
+                layer_gate(y, ref, y3, gw, f"step {step}: layer, T={T}", small=tails(T), plain=step not in OVER)
             done["layer"] += 1
         else:                                                         # calls that must be refused
             kind = draw(0, 3)
