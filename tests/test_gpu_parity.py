@@ -704,3 +704,62 @@ def test_decode_with_skewed_routing_repeats_bitwise(ek, oracle, cuda):
             layer_gate(y, ref, y3, gw, f"decode {name}", small=2)
         assert torch.equal(y.view(torch.int16), first[name].view(torch.int16)), (step, name)
     layer.close()
+
+
+# ------------------------------------------------------------ the packed expert outputs (ek_route_out.expert_out)
+
+def combine_on_host(Y, gw, dt):
+    """The reference's weighted sum (qwen3_moe.py:102-104) of stored expert outputs Y [T, K, H]: each
+    product rounded to the 16-bit type (gate weights of that type) or kept in fp32 (fp32 gate weights),
+    added in k order in fp32, rounded once."""
+    acc = torch.zeros(Y.shape[0], Y.shape[2], dtype=torch.float32)
+    for k in range(Y.shape[1]):
+        p = gw[:, k:k + 1].float() * Y[:, k].float()
+        acc = acc + (p if gw.dtype == torch.float32 else p.to(dt).float())
+    return acc.to(dt)
+
+
+@pytest.mark.parametrize("case", ["c1", "c1_f32_weights", "padded", "w8"])
+def test_expert_outputs_of_a_layer_call(ek, oracle, cuda, case):
+    """expert_out returns every pair's expert output in packed order: found through inv_perm they are
+    the Y [T, K, H] of NaiveExecutor::scatter (controller/executor.rs:203-252).  Held three ways: each
+    row to the oracle's stored Y (one-expert tolerance); the call's y is, bit for bit, the reference's
+    weighted sum of exactly these rows; host-memory calls return the same bits.  A call that runs
+    no experts refuses the field."""
+    from ek_hip import _capi as C
+    import ctypes
+    if case == "padded":
+        w = wl.Workload("padded", 72, 100, 6, 2, 50, torch.bfloat16)          # sizes the kernels take zero-padded
+    elif case == "w8":
+        w = wl.Workload("w8", 256, 128, 8, 2, 300, torch.bfloat16, w8=True, zipf_s=1.0)   # streamed and tiled segments
+    else:
+        w = wl.resolve(wl.C1)
+    dt = w.act_dtype
+    layer, ws = load_layer(ek, w)
+    x = wl.make_x(w)
+    ids, gw = wl.make_routing(w)
+    if case == "c1_f32_weights":
+        gw = gw.float()
+    T, K = ids.shape
+    yp = torch.empty(T * K, w.hidden, dtype=dt, device=cuda)
+    y, rt = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda), return_route=True, expert_out=yp)
+    assert torch.equal(layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda)), y)
+    Y = yp.cpu()[rt.inv_perm.cpu().long()].view(T, K, w.hidden)
+    assert torch.equal(combine_on_host(Y, gw, dt).view(torch.int16), y.cpu().view(torch.int16)), case
+    wu, wg, wd = oracle_weights(oracle, ws, w.n_experts, dt)
+    y3 = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=2, return_y3=True)[5]
+    rms = float(y3.float().pow(2).mean().sqrt())
+    err = (Y.float() - y3.float()).abs()
+    print(f"expert_out {case}: max|Y - Y_ref| / rms = {float(err.max()) / rms:.3e}", flush=True)
+    assert bool((err <= TOL * rms + ulp_of(y3.float(), dt) * 1.0001).all())
+    # host tensors in and out
+    yp_h = torch.empty(T * K, w.hidden, dtype=dt)
+    y_h, rt_h = layer.forward(x, ids, gw, return_route=True, expert_out=yp_h)
+    assert torch.equal(y_h.view(torch.int16), y.cpu().view(torch.int16))
+    assert torch.equal(yp_h.view(torch.int16), yp.cpu().view(torch.int16)) and torch.equal(rt_h.inv_perm, rt.inv_perm.cpu())
+    # ek_layer_pack computes no expert outputs
+    ro = C.ek_route_out(0, 0, 0, 0, yp.data_ptr())
+    idd = ids.to(cuda)
+    st = C.load().ek_layer_pack(layer._h, ctypes.c_void_p(idd.data_ptr()), T, ctypes.byref(ro), None, None, C.EK_DEVICE, None)
+    assert st == C.EK_INVALID_INPUT and b"expert_out" in C.load().ek_last_error()
+    layer.close()
