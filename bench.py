@@ -51,6 +51,71 @@ def measured_traffic(workload: str, stage: int, decode: bool):
     return total if seen else None
 
 
+def kernel_stage(name: str):
+    """(family, stage) of one of the library's FFN kernels from its name as the profiler prints it,
+    demangled (`ek::ffn_tile_kernel<..., E, NMAT, ...>`) or not (`..kernelIDF16bLi<WM>ELi<NMAT>E..`):
+    NMAT = 2 is stage 1 (up + gate), 1 is stage 2 (down)."""
+    import re
+    fam = "stream" if "ffn_stream_kernel" in name else "tile" if "ffn_tile_kernel" in name else None
+    if fam is None:
+        return None, None
+    m = re.search(r"E, (\d),", name.replace(">", ",")) or re.search(r"Li\d+ELi(\d)E", name)
+    return fam, (1 if m and m.group(1) == "2" else 2 if m else None)
+
+
+def live_traffic(n_calls: int):
+    """HBM traffic of the FFN kernels measured in this run: two child runs of this file (the decode
+    configuration and, on the same experts, the prefill configuration, 3 timed calls each) under
+    `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`, each counter scaled by what it reads for a
+    1 GiB device copy launched in the same child.  Returns {"c3": {stage: bytes}, "c4": {...}} (both
+    kernel families of a stage added up, mean per call) or None when the profiler is not there or a
+    child fails; never raises."""
+    import collections, csv, glob, shutil, subprocess, tempfile
+    if shutil.which("rocprofv3") is None:
+        return None
+    per = {}
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            d = tempfile.mkdtemp(prefix="ek_pmc_", dir="/tmp")
+            cmd = ["timeout", "-s", "KILL", "170", "rocprofv3", "--pmc", counter, "-d", d, "-o", "p", "--output-format", "csv",
+                   "--", sys.executable, os.path.abspath(__file__), "--workload", "c3", "--steps", "3", "--warmup", "1",
+                   "--cpu-experts", "0", "--no-parity", "--no-peaks", "--no-live-traffic", "--calib-copy-mib", "1024"]
+            r = subprocess.run(cmd, cwd="/tmp", env={**os.environ, "TMPDIR": "/tmp"}, stdout=subprocess.DEVNULL,
+                               stderr=subprocess.DEVNULL, timeout=200)
+            files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+            if r.returncode != 0 or not files:
+                if os.environ.get("EK_BENCH_DEBUG"): print("live_traffic: child rc", r.returncode, "files", files, file=sys.stderr)
+                shutil.rmtree(d, ignore_errors=True)
+                return None
+            rows = [x for x in csv.DictReader(open(files[0])) if x["Counter_Name"] == counter]
+            shutil.rmtree(d, ignore_errors=True)
+            copies = [float(x["Counter_Value"]) for x in rows if "copyBuffer" in x["Kernel_Name"]]
+            if not copies:
+                if os.environ.get("EK_BENCH_DEBUG"): print("live_traffic: no copy kernel among", sorted(set(x["Kernel_Name"][:40] for x in rows)), file=sys.stderr)
+                return None
+            unit = 1048576.0 * 1024.0 / max(copies)                     # bytes per counter unit: a 1 GiB copy reads and writes 1 GiB
+            # the child launches the calibration copy (three dispatches) before each configuration's calls:
+            # the decode configuration's kernels lie between the two groups of copies, the prefill
+            # configuration's after the second
+            # (the 1 GiB copies stand out by their size among the small copies of weight loading)
+            copy_ids = sorted(int(x["Dispatch_Id"]) for x in rows
+                              if "copyBuffer" in x["Kernel_Name"] and float(x["Counter_Value"]) > 0.5 * max(copies))
+            if len(copy_ids) != 6:
+                if os.environ.get("EK_BENCH_DEBUG"): print("live_traffic: calibration copies", copy_ids, file=sys.stderr)
+                return None
+            for x in rows:
+                fam, stage = kernel_stage(x["Kernel_Name"])
+                did = int(x["Dispatch_Id"])
+                if stage is None or did < copy_ids[2]:
+                    continue
+                cfg = "c3" if did < copy_ids[3] else "c4"
+                c = per.setdefault(cfg, {}).setdefault(stage, {})
+                c[counter] = c.get(counter, 0.0) + float(x["Counter_Value"]) * unit / n_calls
+        return {cfg: {st: sum(c.values()) for st, c in stages.items() if len(c) == 2} for cfg, stages in per.items()}
+    except Exception:
+        return None
+
+
 def cpu_baseline(w, ws_sample, x, ids, gw, target_s=12.0, max_runs=15):
     """Reference-equivalent CPU backend (libtorch ops of ffn/expert_torch.rs:81-84,
     grouped per expert, weighted sum of qwen3_moe.py:102-104) on the pairs routed to
@@ -389,6 +454,9 @@ def main():
     ap.add_argument("--no-parity", dest="parity", action="store_false", help="skip the oracle's output gate before timing")
     ap.add_argument("--no-peaks", dest="peaks", action="store_false", help="skip the copy / read / MFMA microbenchmarks")
     ap.add_argument("--graph", action="store_true", help="also time the call replayed from a graph of the caller's")
+    ap.add_argument("--no-live-traffic", dest="live_traffic", action="store_false",
+                    help="with the default workload: do not measure `roofline.traffic` in this run (two child runs under "
+                         "rocprofv3 --pmc); the figure of the committed profile is reported instead, and labelled so")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
                          "used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -450,6 +518,7 @@ def main():
         out["parity"] = m["parity"]
     torch.set_num_threads(cpu_cores())
     if also is not None:
+        calibration_copy(args, dev)              # (a marker between the two configurations for the profiler's counters)
         mp = time_layer(layer, also, args, dev, stream)
         roof_p, layer_p, config_p = roofline_of(mp)
         out["prefill"] = {"config": config_p, "value": also.pairs / mp["step_s"], "unit": "pairs/s",
@@ -487,6 +556,17 @@ def main():
                                          f"{str(w.act_dtype).replace('torch.', '')}"}
     layer.close()
     del layer, kept, m
+    if everything and args.live_traffic and also is not None:
+        # `traffic` of the two dominant kernels measured now, with the GPU otherwise idle
+        torch.cuda.empty_cache()
+        live = live_traffic(1 + 1 + 3)          # calls per configuration in a child: the gate call, 1 warm-up, 3 timed
+        for cfg, roof_x in (("c3", out["roofline"]), ("c4", out["prefill"]["roofline"])):
+            stage = 1 if "stage 1" in roof_x["kernel"] else 2
+            if live and live.get(cfg, {}).get(stage):
+                roof_x["traffic_committed_profile"] = roof_x["traffic"]
+                roof_x["traffic"] = live[cfg][stage]
+                roof_x["traffic_source"] = ("measured in this run: child runs of this file under rocprofv3 --pmc FETCH_SIZE and "
+                                            "--pmc WRITE_SIZE (3 timed calls), each counter scaled by a 1 GiB device copy")
     if everything:
         # the other three configurations, each built, gated, timed and freed in turn
         torch.cuda.empty_cache()
