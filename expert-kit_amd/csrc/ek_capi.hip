@@ -1038,9 +1038,9 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
         if (cap[l] < 0) cap[l] = 0;
     }
     if (wide_items > 0) {
-        EK_HIP(ek::launch_ffn_stream(a1, 1, L->act, L->wmode, wide_items, true, s));
+        EK_HIP(ek::launch_ffn_stream(a1, 1, L->act, L->wmode, wide_items, true, false, s));
         if (ev) EK_HIP(hipEventRecord(ev[2], s));
-        EK_HIP(ek::launch_ffn_stream(a2, 2, L->act, L->wmode, wide_items, true, s));
+        EK_HIP(ek::launch_ffn_stream(a2, 2, L->act, L->wmode, wide_items, true, false, s));
         return EK_OK;
     }
     // Two independent chains: the weight-streaming kernel (items of <= 16 rows) and the
@@ -1067,6 +1067,7 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
     // pack's tile count, which its kernel left in pinned memory, decides; it may be a call or two
     // old, and either choice computes the same bits.
     const bool have_stream = cap[ek::kListStream] > 0;
+    const bool few_rows = P <= 4 * E;      // streaming items of about four rows or fewer: see launch_ffn_stream
     const bool have_tiles = cap[ek::kListT32] + cap[ek::kListT64] + cap[ek::kListT128] > 0;
     const bool small_expert = 3 * H * I * (L->w8 ? 1 : 2) <= (16ll << 20);
     const bool tiles_lately = exact ? true : ((volatile int32_t *)L->h_err)[1] > 0;   // (exact: have_tiles says it)
@@ -1108,12 +1109,12 @@ ek_status enqueue_ffn(ek_layer *L, const Workspace &W, const void *x, const int3
         // the load would read past the last row of x and past the expert's last weight chunk)
         const bool narrow = known_tile_items > 0 && known_tile_items * wgs_per_item <= 128 && a.Kdim >= 128;
         if (tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, narrow, s_tiles));
-        if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, cap[ek::kListStream], false, s_stream));
+        if (have_stream) EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, cap[ek::kListStream], false, few_rows, s_stream));
         if (shared_wide > 0) {
             ek::FfnArgs aw = a;                  // the same stage over the shared segment's own list
             aw.lists.items[ek::kListStream] = W.wide_items;
             aw.lists.count = W.wide_count;
-            EK_HIP(ek::launch_ffn_stream(aw, stage, L->act, L->wmode, shared_wide, true, side));
+            EK_HIP(ek::launch_ffn_stream(aw, stage, L->act, L->wmode, shared_wide, true, false, side));
         }
         if (!tiles_first && have_tiles) EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, narrow, s_tiles));
         if (stage == 1 && ev) EK_HIP(hipEventRecord(ev[2], s));
@@ -1187,13 +1188,13 @@ ek_status enqueue_shared_own(ek_layer *L, const Workspace &W, const void *x, int
     for (int stage = 1; stage <= 2; ++stage) {
         const ek::FfnArgs &a = stage == 1 ? a1 : a2;
         if (sc.streamed) {
-            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, (T + 15) / 16, false, side));
+            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, (T + 15) / 16, false, T <= 4, side));
         } else if (sc.wide) {
-            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, (T + ek::kWideRows - 1) / ek::kWideRows, true, side));
+            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, (T + ek::kWideRows - 1) / ek::kWideRows, true, false, side));
         } else {
             cap[ek::kListStream] = 1;        // the usual cut leaves at most one item of <= 16 rows
             EK_HIP(ek::launch_ffn_tile(a, stage, L->act, L->wmode, cap, false, side));
-            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, 1, false, side));
+            EK_HIP(ek::launch_ffn_stream(a, stage, L->act, L->wmode, 1, false, false, side));
         }
     }
     EK_HIP(hipEventRecord(L->ev_sjoin, side));

@@ -287,19 +287,35 @@ static hipError_t launch_d(const FfnArgs &a, int32_t nseg, hipStream_t s)
     return hipGetLastError();
 }
 
-// Below this many (item, channel group) waves a launch leaves most of the chip's memory
-// system idle: one wave per slice instead.
-constexpr int64_t kSplitBelow = 1536;
+// The sliced form (eight waves of a workgroup take one slice of the contraction each) against the
+// one-wave form (one wave walks the whole contraction, four or two waves of a workgroup take
+// neighbouring channel groups of one item and share its rows in the CU's cache).  Same bits
+// either way.  Measured on MI355X, enqueue-only layer calls, stage kernel times:
+//  * 16-bit weights: sliced is as fast or faster at every size tried (DeepSeek-V3 shape, 64 experts,
+//    4 / 64 tokens: stage 1 242 -> 222 / 555 -> 546 us, stage 2 118 -> 115 / 287 -> 279 us; Qwen3 shape,
+//    uniform routing, 4 / 64 / 256 tokens: stage 1 38 -> 35 / 127 -> 123 / 101 -> 97 us).
+//  * one-byte weights hold twice the contraction per chunk, and the prefetch slots of the depth that
+//    serves the one-wave form leave room for one sliced workgroup per CU only (164 registers): two
+//    slots deep three fit, and stage 1 of the DeepSeek-V3 int8 layer goes from 47.3 to 39.4 us at
+//    1 token, 242 -> 230 at 8, 681 -> 669 at 32, 1075 -> 1061 at 128.  From 8 rows per expert on the
+//    one-wave form is ahead again (256 tokens: 1157 against 1172 us): every (item, channel group)
+//    reads the item's rows from L2, and neighbouring channel groups in one workgroup share them.
+//    Stage 2 (two channel tiles per wave, two slots deep) gains up to 4 tokens (27.4 -> 23.4 us at
+//    1, 43.7 -> 42.0 at 2) and loses from 8 on (136 -> 141 us at 8, 224 -> 241 at 16, behind a sliced
+//    stage 1).
+constexpr int64_t kSliceStage2Below = 8192;   // (item, channel group) pairs, one-byte weights
 
+// few_rows: the launch's items hold about four rows or fewer on average.
 template <typename T, int WM, int NMAT>
-static hipError_t launch_g(const FfnArgs &a, int32_t nseg, bool wide, hipStream_t s)
+static hipError_t launch_g(const FfnArgs &a, int32_t nseg, bool wide, bool few_rows, hipStream_t s)
 {
+    constexpr bool W8 = WM != kW16;
     constexpr int NG = NMAT == 2 ? kStage1Tiles : kStage2Tiles;
     constexpr int D = NMAT == 2 ? kStage1Depth : kStage2Depth;
     const int NT = a.N / 16;
     if (wide) {
         // four activation fragments per prefetch slot: shallower, the eight slices make up for it
-        constexpr int DW = WM != kW16 ? 2 : 4;
+        constexpr int DW = W8 ? 2 : 4;
         // Channel tiles per workgroup: every workgroup reads its item's rows in full, so more
         // tiles per workgroup mean fewer readers of the rows; a short list wants the workgroups
         // instead.  Measured on MI355X, one DeepSeek-V3 expert: two instead of one (stage 1)
@@ -318,40 +334,48 @@ static hipError_t launch_g(const FfnArgs &a, int32_t nseg, bool wide, hipStream_
                                dim3(64 * kSlices), 0, s, a);
         return hipGetLastError();
     }
-    if (NT % NG == 0 && (int64_t)nseg * (NT / NG) < kSplitBelow) {
-        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, NMAT, NG, D, kSlices, 1>), dim3(NT / NG, nseg),
-                           dim3(64 * kSlices), 0, s, a);
-        return hipGetLastError();
+    if (NT % NG == 0) {
+        // prefetch slots of the sliced form: a slice is an eighth of the contraction
+        constexpr int DS = W8 ? 2 : D;
+        const bool sliced = !W8 ? true
+                            : NMAT == 2 ? few_rows
+                                        : (int64_t)nseg * (NT / NG) < kSliceStage2Below;
+        if (sliced) {
+            hipLaunchKernelGGL((ffn_stream_kernel<T, WM, NMAT, NG, DS, kSlices, 1>), dim3(NT / NG, nseg),
+                               dim3(64 * kSlices), 0, s, a);
+            return hipGetLastError();
+        }
+        return launch_d<T, WM, NMAT, NG, D>(a, nseg, s);
     }
-    if (NT % NG == 0) return launch_d<T, WM, NMAT, NG, D>(a, nseg, s);
     if (NT % 2 == 0) return launch_d<T, WM, NMAT, 2, D>(a, nseg, s);
     return launch_d<T, WM, NMAT, 1, D>(a, nseg, s);
 }
 
 template <typename T>
-static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, int32_t n_segments, bool wide, hipStream_t s)
+static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, int32_t n_segments, bool wide, bool few_rows,
+                           hipStream_t s)
 {
     switch (wmode) {
     case kWI8:
-        return stage == 1 ? launch_g<T, kWI8, 2>(a, n_segments, wide, s) : launch_g<T, kWI8, 1>(a, n_segments, wide, s);
+        return stage == 1 ? launch_g<T, kWI8, 2>(a, n_segments, wide, few_rows, s) : launch_g<T, kWI8, 1>(a, n_segments, wide, few_rows, s);
     case kWF8Block:
-        return stage == 1 ? launch_g<T, kWF8Block, 2>(a, n_segments, wide, s)
-                          : launch_g<T, kWF8Block, 1>(a, n_segments, wide, s);
+        return stage == 1 ? launch_g<T, kWF8Block, 2>(a, n_segments, wide, few_rows, s)
+                          : launch_g<T, kWF8Block, 1>(a, n_segments, wide, few_rows, s);
     case kWI8Block:
-        return stage == 1 ? launch_g<T, kWI8Block, 2>(a, n_segments, wide, s)
-                          : launch_g<T, kWI8Block, 1>(a, n_segments, wide, s);
+        return stage == 1 ? launch_g<T, kWI8Block, 2>(a, n_segments, wide, few_rows, s)
+                          : launch_g<T, kWI8Block, 1>(a, n_segments, wide, few_rows, s);
     default:
-        return stage == 1 ? launch_g<T, kW16, 2>(a, n_segments, wide, s) : launch_g<T, kW16, 1>(a, n_segments, wide, s);
+        return stage == 1 ? launch_g<T, kW16, 2>(a, n_segments, wide, few_rows, s) : launch_g<T, kW16, 1>(a, n_segments, wide, few_rows, s);
     }
 }
 
 hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, int wmode, int64_t max_items, bool wide,
-                             hipStream_t s)
+                             bool few_rows, hipStream_t s)
 {
     const int32_t n_segments = (int32_t)max_items;
     if (n_segments <= 0) return hipSuccess;
-    return act == 0 ? launch_w<__bf16>(a, stage, wmode, n_segments, wide, s)
-                    : launch_w<_Float16>(a, stage, wmode, n_segments, wide, s);
+    return act == 0 ? launch_w<__bf16>(a, stage, wmode, n_segments, wide, few_rows, s)
+                    : launch_w<_Float16>(a, stage, wmode, n_segments, wide, few_rows, s);
 }
 
 }  // namespace ek

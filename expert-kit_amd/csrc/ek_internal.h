@@ -162,9 +162,10 @@ struct FfnArgs {
 // stage = 1: up/gate + SwiGLU epilogue;  stage = 2: down projection
 // act: 0 bf16, 1 f16;  wmode: WeightMode
 // weight-streaming kernel over lists.items[kListStream]; max_items = grid bound;
-// wide: items hold up to kWideRows rows (else up to 16)
+// wide: items hold up to kWideRows rows (else up to 16); few_rows: about four rows or fewer per
+// item on average (a hint for the launch shape; the results do not depend on it)
 hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, int wmode, int64_t max_items, bool wide,
-                             hipStream_t s);
+                             bool few_rows, hipStream_t s);
 // MFMA tile kernel over the three tile lists (128-row items first, then 64,
 // then 32); max_items[l] bounds list l.  A workgroup covers tile_channels(stage, narrow) output
 // channels of one item; the narrow form (half the channels per workgroup, so twice the workgroups
