@@ -1207,9 +1207,18 @@ ek_status enqueue_shared_own(ek_layer *L, const Workspace &W, const void *x, int
 // layers' routing halves and waits for the next layer's there: the wait costs nothing at that
 // point, and the next layer's first kernel then depends on nothing but this layer's combine in
 // its own queue).
+// Most pairs of a call that runs pair-direct (launch_ffn_pairs).  Every pair streams its expert's
+// weights on its own, so tokens that share an expert read it twice, and stage 2's one wave per pair
+// walks the whole contraction where the ordinary launch of so few items slices it.  Measured on
+// MI355X, DeepSeek-V3 int8 layer (256 experts, top-8), enqueue-only calls: 1 token 75.3 -> 62.4 us
+// (352 MB: 5.6 TB/s, 71 % of the 8 TB/s peak, over the whole call), 2 tokens 131.7 -> 121-127 us,
+// 4 tokens 220 -> 231 us, 8 tokens 366 -> 437 us.
+constexpr int64_t kPairDirectPairs = 16;
+
+// want_tables: the caller reads the call's routing tables or packed expert outputs afterwards.
 ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const int32_t *ids, const void *w, int w_f32,
                           int64_t T, void *y, hipStream_t s, bool routed = false,
-                          const std::function<ek_status()> *before_combine = nullptr)
+                          const std::function<ek_status()> *before_combine = nullptr, bool want_tables = true)
 {
     const int64_t H = L->cfg.hidden;
     const int E = L->cfg.n_experts, K = L->cfg.top_k;
@@ -1220,6 +1229,28 @@ ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const 
         L->events_used += 5;
     }
     if (ev) EK_HIP(hipEventRecord(ev[0], s));
+    // A decode call of one or two tokens: its few pairs run as one-row items straight from the ids,
+    // and stage 2 adds a token's pairs itself: two kernels instead of four (no pack, no combine;
+    // DeepSeek-V3 int8 layer on MI355X, 1 / 2 tokens: see kPairDirectPairs).  Same bits.
+    if (!routed && !want_tables && P > 0 && P <= kPairDirectPairs && K <= ek::kPairDirectMaxK && !shared_cut(L, T).shared) {
+        ek::FfnArgs a1;
+        a1.x = x; a1.x_stride = H; a1.rows = nullptr; a1.slabs = L->d_slabs; a1.out = W.h; a1.out_stride = L->cfg.inter;
+        a1.N = (int32_t)L->cfg.inter; a1.Kdim = (int32_t)H; a1.lists = W.lists;
+        a1.pair_ids = ids; a1.pair_K = K; a1.pair_P = (int32_t)P; a1.n_experts = E;
+        a1.pair_err = W.err; a1.pair_activation = L->d_activation; a1.pair_tile_items_host = L->d_tile_items;
+        ek::FfnArgs a2 = a1;
+        a2.x = W.h; a2.x_stride = L->cfg.inter; a2.out = nullptr; a2.out_stride = H;
+        a2.N = (int32_t)H; a2.Kdim = (int32_t)L->cfg.inter;
+        a2.pair_w = w; a2.pair_w_f32 = w_f32; a2.pair_y = y;
+        if (ev) EK_HIP(hipEventRecord(ev[1], s));
+        EK_HIP(ek::launch_ffn_pairs(a1, 1, L->act, L->wmode, s));
+        if (ev) EK_HIP(hipEventRecord(ev[2], s));
+        EK_HIP(ek::launch_ffn_pairs(a2, 2, L->act, L->wmode, s));
+        if (ev) EK_HIP(hipEventRecord(ev[3], s));
+        if (before_combine) EK_TRY((*before_combine)());
+        if (ev) EK_HIP(hipEventRecord(ev[4], s));
+        return EK_OK;
+    }
     if (!routed) EK_TRY(enqueue_route(L, W, ids, T, s));
     // the shared expert is one more segment: every token once, rows P .. P+T-1 of the packed buffers.
     // As tiles a decode-sized shared segment would occupy 8 to 14 CUs for the length of the whole
@@ -1413,12 +1444,12 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
                 d_w = layer->st_w;
             }
             EK_TRY(rows_in(layer, layer->st_x, x, T, mem, s));
-            EK_TRY(enqueue_forward(layer, layer->ws, layer->st_x, d_ids, d_w, w_f32, T, layer->st_y, s));
+            EK_TRY(enqueue_forward(layer, layer->ws, layer->st_x, d_ids, d_w, w_f32, T, layer->st_y, s, false, nullptr, route != nullptr));
             EK_TRY(rows_out(layer, y, layer->st_y, T, mem, s));
             EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
             if (!stream) { st = finish_blocking(layer, layer->ws, s); use.synced(); }
         } else if (mem == EK_DEVICE) {
-            EK_TRY(enqueue_forward(layer, layer->ws, x, ids, w, w_f32, T, y, s));
+            EK_TRY(enqueue_forward(layer, layer->ws, x, ids, w, w_f32, T, y, s, false, nullptr, route != nullptr));
             EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
             if (!stream) { st = finish_blocking(layer, layer->ws, s); use.synced(); }
         } else {
@@ -1430,7 +1461,7 @@ ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, c
                 EK_TRY(h2d(layer, layer->st_w, w, (size_t)P * (w_f32 ? 4 : 2), s));
             }
             EK_TRY(enqueue_forward(layer, layer->ws, layer->st_x, layer->st_ids, layer->st_w, w_f32, T,
-                                   layer->st_y, s));
+                                   layer->st_y, s, false, nullptr, route != nullptr));
             if (T > 0) EK_TRY(d2h(layer, y, layer->st_y, (size_t)T * H * 2, s));
             EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));
             st = finish_blocking(layer, layer->ws, s);
@@ -1485,7 +1516,7 @@ ek_status ek_layer_forward_static(ek_layer *layer, const void *x, const int32_t 
         ek_status st = EK_OK;
         // a blocking call sees everything submitted before it (waiting allocates nothing)
         if (!stream) EK_HIP(hipDeviceSynchronize());
-        EK_TRY(enqueue_forward(layer, W, x, ids, w, w_f32, T, y, s));
+        EK_TRY(enqueue_forward(layer, W, x, ids, w, w_f32, T, y, s, false, nullptr, route != nullptr));
         EK_TRY(copy_route_out(layer, W, route, P, EK_DEVICE, s));
         if (!stream) {
             st = finish_blocking(layer, W, s);
@@ -2302,7 +2333,7 @@ ek_status route_and_forward(ek_layer *layer, const void *x, const void *logits, 
     if (P > 0 && w_out) EK_TRY(give(w_out, layer->rt_w, w_bytes));
     ek_status st = EK_OK;
     if (forward) {
-        EK_TRY(enqueue_forward(layer, layer->ws, d_x, layer->rt_ids, layer->rt_w, w_f32, T, d_y, s));
+        EK_TRY(enqueue_forward(layer, layer->ws, d_x, layer->rt_ids, layer->rt_w, w_f32, T, d_y, s, false, nullptr, route != nullptr));
         if (layer->padded) EK_TRY(rows_out(layer, y, layer->st_y, T, mem, s));
         else if (mem == EK_HOST && T > 0) EK_TRY(d2h(layer, y, layer->st_y, (size_t)T * H * 2, s));
         EK_TRY(copy_route_out(layer, layer->ws, route, P, mem, s));

@@ -47,9 +47,43 @@ constexpr int kSlices = 8;
 
 constexpr int kMaxScaleBlocks = 64;   // 128-wide scale blocks along the contraction: K <= 8192
 
-template <typename T, int WM, int NMAT, int NG, int D, int SK, int RS>
-__global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kernel(FfnArgs a)
+// What the pack kernel would have stored of a pair-direct call's bookkeeping; one wave.
+__device__ __forceinline__ void pair_bookkeeping(const FfnArgs &a, int lane)
 {
+    const int32_t id = lane < a.pair_P ? a.pair_ids[lane] : 0;
+    const bool bad = lane < a.pair_P && (uint32_t)id >= (uint32_t)a.n_experts;
+    const bool ok = lane < a.pair_P && !bad;
+    const bool unloaded = ok && a.slabs[id].upgate == nullptr;
+    const uint64_t any_bad = __ballot(bad), any_unloaded = __ballot(unloaded);
+    if (ok && a.pair_activation) atomicAdd((unsigned long long *)&a.pair_activation[id], 1ull);
+    if (lane == 0) {
+        a.pair_err[0] = (any_bad ? 1 : 0) | (any_unloaded ? 2 : 0);
+        if (a.pair_tile_items_host) *a.pair_tile_items_host = 0;
+    }
+}
+
+// The first wave of a pair-direct stage-2 workgroup adds the token's weighted expert outputs in k
+// order (the arithmetic of combine_kernel) and stores the token's channels of this workgroup.
+template <typename T, int NCH>
+__device__ __forceinline__ void pair_combine(const FfnArgs &a, const float (*prod)[NCH], const int32_t *valid, int64_t t,
+                                             int ch0, int lane)
+{
+    if (lane >= NCH) return;
+    float acc = 0.f;
+    for (int k = 0; k < a.pair_K; ++k)
+        if (valid[k]) acc = acc + prod[k][lane];
+    ((T *)a.pair_y)[t * a.N + ch0 + lane] = (T)acc;
+}
+
+// PD = 0: items from the work list.  PD = 1: pair-direct stage 1 (blockIdx.y is the pair).  PD = 2:
+// pair-direct stage 2 (blockIdx.y is the token, wave k of the workgroup takes its k-th pair and walks
+// the whole contraction, SK = 1; the weighted sum over k replaces the store of the rows).
+template <typename T, int WM, int NMAT, int NG, int D, int SK, int RS, int PD = 0>
+__global__ __launch_bounds__(PD == 2 ? 64 * kPairDirectMaxK : SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kernel(FfnArgs a)
+{
+    static_assert(PD == 0 || RS == 1, "pair-direct items hold one row");
+    static_assert(PD != 1 || (NMAT == 2 && SK == kSlices), "pair-direct stage 1 is a sliced launch");
+    static_assert(PD != 2 || (NMAT == 1 && SK == 1), "pair-direct stage 2: one wave per pair");
     constexpr bool W8 = WM != kW16;    // one-byte weights: 64 contraction elements per chunk
     static_assert(SK == 1 || SK == kSlices, "one wave per launch shape or one wave per slice");
     static_assert(RS == 1 || SK == kSlices, "wide items only in the sliced form");
@@ -59,15 +93,39 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
     constexpr int NW = NMAT * NG;      // weight chunks per k step per wave
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if ((int)blockIdx.y >= a.lists.count[kListStream]) return;
-    const WorkItem item = a.lists.items[kListStream][blockIdx.y];
-    const int e = item.expert, seg0 = item.row0, n = item.nrows;
+    int e, seg0, n;
+    [[maybe_unused]] bool live = true;      // PD = 2: this wave's pair has an expert to run
+    if constexpr (PD == 0) {
+        if ((int)blockIdx.y >= a.lists.count[kListStream]) return;
+        const WorkItem item = a.lists.items[kListStream][blockIdx.y];
+        e = item.expert; seg0 = item.row0; n = item.nrows;
+    } else {
+        if (PD == 1 && blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) pair_bookkeeping(a, lane);
+        seg0 = PD == 1 ? (int)blockIdx.y : (int)blockIdx.y * a.pair_K + wave;
+        n = 1;
+        e = a.pair_ids[seg0];
+        live = (uint32_t)e < (uint32_t)a.n_experts;
+        if (!live) e = 0;
+    }
     const int NT = a.N >> 4;
-    const int nt0 = SK == 1 ? (blockIdx.x * (blockDim.x >> 6) + wave) * NG : blockIdx.x * NG;
-    if (nt0 >= NT) return;             // SK = 8: the same for every wave of the workgroup
+    const int nt0 = SK == 1 && PD != 2 ? (blockIdx.x * (blockDim.x >> 6) + wave) * NG : blockIdx.x * NG;
+    if (nt0 >= NT) return;             // SK = 8, PD = 2: the same for every wave of the workgroup
     const ExpertSlab slab = a.slabs[e];
     const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
-    if (wmat == nullptr) return;   // expert not loaded: pack has flagged the call
+    [[maybe_unused]] __shared__ float pd_prod[PD == 2 ? kPairDirectMaxK : 1][PD == 2 ? NG * 16 : 1];
+    [[maybe_unused]] __shared__ int32_t pd_valid[PD == 2 ? kPairDirectMaxK : 1];
+    if constexpr (PD == 2) {
+        live = live && wmat != nullptr;
+        if (!live) {
+            // nothing to add for this pair; the workgroup's sum still needs this wave at its barrier
+            if (lane == 0) pd_valid[wave] = 0;
+            __syncthreads();
+            if (wave == 0) pair_combine<T, NG * 16>(a, pd_prod, pd_valid, blockIdx.y, nt0 * 16, lane);
+            return;
+        }
+    } else {
+        if (!live || wmat == nullptr) return;   // expert not loaded: the call has been flagged
+    }
     const int KT = a.Kdim / KE;
     const int j = lane & 15, g = lane >> 4;
 
@@ -94,7 +152,7 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
     // Block scales: the wave's 16 channels lie in one 128-row block, so the scale of a chunk is
     // one number per 128 contraction elements: the wave keeps its rows of the scale matrices in
     // LDS (lane b holds block b) and reads one back per chunk.
-    __shared__ float srow[block_scaled(WM) ? (SK == 1 ? 4 : kSlices) : 1][block_scaled(WM) ? NW : 1]
+    __shared__ float srow[block_scaled(WM) ? (PD == 2 ? kPairDirectMaxK : SK == 1 ? 4 : kSlices) : 1][block_scaled(WM) ? NW : 1]
                          [block_scaled(WM) ? kMaxScaleBlocks : 1];
     if constexpr (block_scaled(WM)) {
         const int KB = (a.Kdim + 127) >> 7;
@@ -115,7 +173,8 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs) {
         const int jr = min(rs * 16 + j, n - 1);   // lanes past the segment re-read its last row
-        const int64_t row = a.rows ? (int64_t)a.rows[seg0 + jr] : (int64_t)(seg0 + jr);
+        const int64_t row = PD == 1 ? (int64_t)(seg0 / a.pair_K)
+                            : a.rows ? (int64_t)a.rows[seg0 + jr] : (int64_t)(seg0 + jr);
         xp[rs] = (const T *)a.x + row * a.x_stride + g * (KE / 4);
     }
 
@@ -241,6 +300,25 @@ __global__ __launch_bounds__(SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kerne
                 }
     }
 
+    if constexpr (PD == 2) {
+        // lanes (g, 0) hold the pair's row: its rounded outputs times the gate weight, as the
+        // combine kernel forms them, meet in LDS
+        const float wv = a.pair_w_f32 ? ((const float *)a.pair_w)[seg0] : (float)((const T *)a.pair_w)[seg0];
+        if (j == 0) {
+#pragma unroll
+            for (int gi = 0; gi < NG; ++gi)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float pr = wv * (float)(T)tot[0][0][gi][r];
+                    if (!a.pair_w_f32) pr = (float)(T)pr;
+                    pd_prod[wave][gi * 16 + 4 * g + r] = pr;
+                }
+        }
+        if (lane == 0) pd_valid[wave] = 1;
+        __syncthreads();
+        if (wave == 0) pair_combine<T, NG * 16>(a, pd_prod, pd_valid, blockIdx.y, nt0 * 16, lane);
+        return;
+    }
     // epilogue: lane (g, j) holds channels nt*16 + 4g + r (r = 0..3) of row rs*16 + j
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs) {
@@ -367,6 +445,51 @@ static hipError_t launch_w(const FfnArgs &a, int stage, int wmode, int32_t n_seg
     default:
         return stage == 1 ? launch_g<T, kW16, 2>(a, n_segments, wide, few_rows, s) : launch_g<T, kW16, 1>(a, n_segments, wide, few_rows, s);
     }
+}
+
+template <typename T, int WM>
+static hipError_t launch_pairs_w(const FfnArgs &a, int stage, hipStream_t s)
+{
+    constexpr bool W8 = WM != kW16;
+    const int NT = a.N / 16;
+    const int KT = a.Kdim / (W8 ? 64 : 32);
+    if (stage == 1) {
+        // the sliced form of the ordinary launch, one item per pair
+        constexpr int DS = W8 ? 2 : kStage1Depth;
+        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 2, 1, DS, kSlices, 1, 1>), dim3(NT, a.pair_P), dim3(64 * kSlices), 0, s, a);
+        return hipGetLastError();
+    }
+    const dim3 block(64 * a.pair_K);
+    const int T_ = a.pair_P / a.pair_K;
+    constexpr int NG = kStage2Tiles, D = kStage2Depth;
+    if (NT % NG == 0 && KT % D == 0)
+        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 1, NG, D, 1, 1, 2>), dim3(NT / NG, T_), block, 0, s, a);
+    else if (NT % NG == 0 && KT % (D / 2) == 0)
+        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 1, NG, D / 2, 1, 1, 2>), dim3(NT / NG, T_), block, 0, s, a);
+    else if (NT % NG == 0 && KT % 2 == 0)
+        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 1, NG, 2, 1, 1, 2>), dim3(NT / NG, T_), block, 0, s, a);
+    else
+        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 1, 1, 1, 1, 1, 2>), dim3(NT, T_), block, 0, s, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+static hipError_t launch_pairs_t(const FfnArgs &a, int stage, int wmode, hipStream_t s)
+{
+    switch (wmode) {
+    case kWI8: return launch_pairs_w<T, kWI8>(a, stage, s);
+    case kWF8Block: return launch_pairs_w<T, kWF8Block>(a, stage, s);
+    case kWI8Block: return launch_pairs_w<T, kWI8Block>(a, stage, s);
+    default: return launch_pairs_w<T, kW16>(a, stage, s);
+    }
+}
+
+hipError_t launch_ffn_pairs(const FfnArgs &a, int stage, int act, int wmode, hipStream_t s)
+{
+    if (a.pair_P <= 0) return hipSuccess;
+    if (a.pair_P > kPairDirectMax || a.pair_K <= 0 || a.pair_K > kPairDirectMaxK || a.pair_P % a.pair_K != 0)
+        return hipErrorInvalidValue;
+    return act == 0 ? launch_pairs_t<__bf16>(a, stage, wmode, s) : launch_pairs_t<_Float16>(a, stage, wmode, s);
 }
 
 hipError_t launch_ffn_stream(const FfnArgs &a, int stage, int act, int wmode, int64_t max_items, bool wide,

@@ -158,7 +158,27 @@ struct FfnArgs {
     int32_t N;                // output channels of this stage
     int32_t Kdim;             // contraction length of this stage
     WorkLists lists;          // device work lists and their lengths
+    // pair-direct launches (launch_ffn_pairs): pair p = t * pair_K + k is its own one-row item,
+    // x row t (stage 1) or p (stage 2), out row p; no lists
+    const int32_t *pair_ids = nullptr;   // [pair_P] expert of pair p
+    int32_t pair_K = 0, pair_P = 0, n_experts = 0;
+    const void *pair_w = nullptr;        // [pair_P] gate weights (stage 2)
+    int32_t pair_w_f32 = 0;              // gate weights are fp32 instead of the activation type
+    void *pair_y = nullptr;              // [T, N] stage 2: the weighted sum over a token's pairs
+    int32_t *pair_err = nullptr;         // stage 1 writes the call's error word (PackArgs::err)
+    uint64_t *pair_activation = nullptr; // [n_experts] or nullptr (PackArgs::activation)
+    int32_t *pair_tile_items_host = nullptr;   // receives 0 (PackArgs::tile_items_host), or nullptr
 };
+// Most pairs a pair-direct call may hold (one wave writes the call's bookkeeping) and its
+// largest top-k (one wave per pair of a token in stage 2's workgroups).
+constexpr int kPairDirectMax = 64, kPairDirectMaxK = 8;
+// A decode call of a few pairs without pack and combine kernels: stage 1 runs every pair as a
+// one-row item straight from the ids (and stores what the pack kernel would have stored of the
+// call's bookkeeping: error word, activation counters, zero tile items); stage 2 computes a
+// token's pairs in one workgroup, one wave each, and adds them in k order with the gate weights:
+// the arithmetic of the streaming kernel followed by launch_combine, bit for bit.  Pairs whose
+// id is out of range or whose expert is not loaded add nothing.  T = pair_P / pair_K.
+hipError_t launch_ffn_pairs(const FfnArgs &a, int stage, int act, int wmode, hipStream_t s);
 // stage = 1: up/gate + SwiGLU epilogue;  stage = 2: down projection
 // act: 0 bf16, 1 f16;  wmode: WeightMode
 // weight-streaming kernel over lists.items[kListStream]; max_items = grid bound;
