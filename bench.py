@@ -336,6 +336,40 @@ def time_layer(layer, w, args, dev, stream, graph=False):
             "graph_s": graph_s}
 
 
+def decode_sweep(layer, base, dev, stream, token_counts, calls=30):
+    """The decode layer at other batch sizes (uniform routing, as the configuration's): enqueue-only
+    calls on `stream`, the whole call's algorithmic bytes against the HBM peak.  The routing tables of each
+    size are checked against a stable sort first; the timed calls must reproduce that call's output."""
+    import torch
+    from dataclasses import replace
+    from ek_hip import workloads as wl
+    rows = []
+    for T in token_counts:
+        w = replace(base, tokens=T)
+        ids, gw = wl.make_routing(w)
+        counts = torch.bincount(ids.reshape(-1).long(), minlength=w.n_experts)
+        xd, idd, gwd = wl.make_x(w).to(dev), ids.to(dev), gw.to(dev)
+        y0, rt = layer.forward(xd, idd, gwd, return_route=True)
+        assert torch.equal(rt.perm.cpu(), torch.argsort(ids.reshape(-1).long(), stable=True).to(torch.int32)), T
+        y = torch.empty_like(xd)
+        for _ in range(5):
+            layer.forward(xd, idd, gwd, stream=stream, out=y)
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for _ in range(calls):
+            layer.forward(xd, idd, gwd, stream=stream, out=y)
+        e1.record(stream)
+        stream.synchronize()
+        step_s = max(time.perf_counter() - t0, e0.elapsed_time(e1) * 1e-3) / calls
+        assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), T
+        rows.append({"tokens": T, "ms_per_step": step_s * 1e3, "pairs_per_s": w.pairs / step_s,
+                     "active_experts": int((counts > 0).sum()),
+                     "hbm_frac": wl.algorithmic_bytes(w, counts) / step_s / HBM_PEAK})
+    return rows
+
+
 def roofline_of(m):
     """Roofline of the dominant kernel of one measured workload, and the layer-level figures."""
     w, counts, step_s, k_us = m["w"], m["counts"], m["step_s"], m["k_us"]
@@ -457,6 +491,8 @@ def main():
     ap.add_argument("--no-live-traffic", dest="live_traffic", action="store_false",
                     help="with the default workload: do not measure `roofline.traffic` in this run (two child runs under "
                          "rocprofv3 --pmc); the figure of the committed profile is reported instead, and labelled so")
+    ap.add_argument("--no-sweep", dest="sweep", action="store_false",
+                    help="with --workload all: skip the decode layer's other batch sizes (decode_sweep)")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also launch a plain device copy of this many MiB (a kernel of known traffic, "
                          "used to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -516,6 +552,10 @@ def main():
         out["graph_replay_ms_per_step"] = m["graph_s"] * 1e3
     if m["parity"] is not None:
         out["parity"] = m["parity"]
+    if everything and args.sweep:
+        out["decode_sweep"] = {"what": f"{w.name}'s layer at other batch sizes, {30} enqueue-only calls each, whole call against "
+                                       "8 TB/s; outputs equal the routing-checked call's bit for bit",
+                               "rows": decode_sweep(layer, w, dev, stream, (1, 2, 4, 8, 16, 32, 64, 256, 512))}
     torch.set_num_threads(cpu_cores())
     if also is not None:
         calibration_copy(args, dev)              # (a marker between the two configurations for the profiler's counters)
