@@ -1214,6 +1214,11 @@ ek_status enqueue_shared_own(ek_layer *L, const Workspace &W, const void *x, int
 // (352 MB: 5.6 TB/s, 71 % of the 8 TB/s peak, over the whole call), 2 tokens 131.7 -> 121-127 us,
 // 4 tokens 220 -> 231 us, 8 tokens 366 -> 437 us.
 constexpr int64_t kPairDirectPairs = 16;
+bool pair_direct_fits(const ek_layer *L, int64_t T)
+{
+    const int64_t P = T * L->cfg.top_k;
+    return P > 0 && P <= kPairDirectPairs && L->cfg.top_k <= ek::kPairDirectMaxK && !shared_cut(L, T).shared;
+}
 
 // want_tables: the caller reads the call's routing tables or packed expert outputs afterwards.
 ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const int32_t *ids, const void *w, int w_f32,
@@ -1232,7 +1237,7 @@ ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const 
     // A decode call of one or two tokens: its few pairs run as one-row items straight from the ids,
     // and stage 2 adds a token's pairs itself: two kernels instead of four (no pack, no combine;
     // DeepSeek-V3 int8 layer on MI355X, 1 / 2 tokens: see kPairDirectPairs).  Same bits.
-    if (!routed && !want_tables && P > 0 && P <= kPairDirectPairs && K <= ek::kPairDirectMaxK && !shared_cut(L, T).shared) {
+    if (!routed && !want_tables && pair_direct_fits(L, T)) {
         ek::FfnArgs a1;
         a1.x = x; a1.x_stride = H; a1.rows = nullptr; a1.slabs = L->d_slabs; a1.out = W.h; a1.out_stride = L->cfg.inter;
         a1.N = (int32_t)L->cfg.inter; a1.Kdim = (int32_t)H; a1.lists = W.lists;
@@ -2023,7 +2028,11 @@ static ek_status enqueue_chain(ek_chain *c, const void *x, const int32_t *ids, c
         EK_TRY(rows_in(c->layers[0], c->act_in, x, T, EK_DEVICE, s));
         in = c->act_in;
     }
-    const bool ahead = c->route_stream != nullptr && T > 0;
+    // (a chain of a few pairs per layer has no routing halves to run ahead: its layer calls are
+    // pair-direct, two kernels each)
+    bool pair_direct = true;
+    for (int l = 0; l < L; ++l) pair_direct = pair_direct && pair_direct_fits(c->layers[l], T);
+    const bool ahead = c->route_stream != nullptr && T > 0 && !pair_direct;
     if (ahead) {
         // layer 0's routing half first, alone
         EK_TRY(enqueue_route(c->layers[0], c->layers[0]->ws, ids, T, s));
@@ -2052,7 +2061,7 @@ static ek_status enqueue_chain(ek_chain *c, const void *x, const int32_t *ids, c
         ly->profiling = false;               // no event records inside a chain (capture-safe)
         ek_status st = enqueue_forward(ly, ly->ws, in, ids + (size_t)l * T * K,
                                        (const char *)w + (size_t)l * T * K * w_es, w_f32, T, outp, s, ahead,
-                                       ahead ? &mid : nullptr);
+                                       ahead ? &mid : nullptr, !pair_direct);
         ly->profiling = prof;
         EK_TRY(st);
         // collect the layer's error word with a copy kernel-free D2D memcpy node

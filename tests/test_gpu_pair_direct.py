@@ -172,3 +172,34 @@ def test_wider_top_k_and_more_pairs_take_the_ordinary_path(ek, oracle, cuda):
         y_t, _ = layer.forward(x, ids, gw, return_route=True)
         assert same_bits(y, y_t)
         layer.close()
+
+
+@pytest.mark.parametrize("T", [1, 2, 4])
+def test_chain_of_few_pairs(ek, cuda, T):
+    """A chain's layer calls of one or two tokens are pair-direct as well (4 tokens x top-4 = 16 pairs is
+    the last size that is): eager and replayed graph give the bits of the layers called one by one
+    through pack and combine, also after new inputs arrive in the same buffers."""
+    from test_gpu_chain import build_chain, bits
+    w0 = wl.Workload("decode_x3", 256, 128, 16, 4, T, torch.float16, zipf_s=1.2, n_layers=3)
+    w, layers, weights, ids, gw = build_chain(ek, w0, cuda, std=0.08)
+    xd = wl.make_x(w).to(cuda)
+    chain = ek.HipChain(layers)
+
+    def one_by_one():
+        cur = xd
+        for l, layer in enumerate(layers):
+            cur, _ = layer.forward(cur, ids[l].contiguous(), gw[l].contiguous(), return_route=True)
+        return cur
+
+    for trial in range(2):
+        want = one_by_one()
+        assert torch.equal(bits(chain.forward(xd, ids, gw, use_graph=False)), bits(want)), trial
+        for rep in range(3):
+            assert torch.equal(bits(chain.forward(xd, ids, gw, use_graph=True)), bits(want)), (trial, rep)
+            layers[rep % 3].forward(xd, ids[0].contiguous(), gw[0].contiguous())
+            torch.cuda.synchronize()
+        xd.copy_(torch.randn_like(xd))
+        ids.copy_(torch.stack([wl.make_routing(w, layer=10 + l)[0] for l in range(w.n_layers)]).to(cuda))
+    chain.close()
+    for layer in layers:
+        layer.close()
