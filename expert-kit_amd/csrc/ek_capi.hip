@@ -140,6 +140,7 @@ struct ek_layer {
     // host-built work lists (ek_layer_experts_forward): pinned image of the device lists,
     // reused once ev_items says the previous copy has been consumed
     uint8_t *h_items = nullptr;
+    uint8_t *d_items = nullptr;              // the device's address of h_items (nullptr: asynchronous copies instead)
     hipEvent_t ev_items = nullptr;
     ek::RowCopy *h_segs = nullptr;           // pinned: the row-copy tables of a batched device-memory call, in then out
     ek::RowCopy *d_segs = nullptr;           // the device's address of h_segs
@@ -1736,8 +1737,11 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
                 else if (r > 0) items[ek::kListStream].push_back(rem);
                 row0 += n;
             }
+            // pinned block: the lists' lengths (16 bytes), the table of the copy kernel that takes them to the
+            // device, then the lists
             size_t off[ek::kNumLists + 1];
-            off[0] = 16;
+            off[0] = 256;
+            static_assert(16 + sizeof(ek::RowCopy) * (ek::kNumLists + 1) <= 256, "list-copy table");
             for (int l = 0; l < ek::kNumLists; ++l) {
                 if ((int64_t)items[l].size() > layer->ws.list_cap[l])
                     return fail(EK_INVALID_INPUT, "too many calls for one launch (work list %d holds %lld items)", l,
@@ -1747,19 +1751,35 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             if (!layer->h_items) {
                 EK_HIP(hipHostMalloc((void **)&layer->h_items, off[ek::kNumLists], hipHostMallocDefault));
                 EK_HIP(hipEventCreateWithFlags(&layer->ev_items, hipEventDisableTiming));
+                void *dp = nullptr;
+                if (hipHostGetDevicePointer(&dp, layer->h_items, 0) != hipSuccess) { (void)hipGetLastError(); dp = nullptr; }
+                layer->d_items = (uint8_t *)dp;
             } else {
                 EK_HIP(hipEventSynchronize(layer->ev_items));
             }
+            // One copy kernel reads the lists and their lengths where they lie in pinned memory (up to five
+            // asynchronous copies took the stream ~45 us before the first FFN kernel of a decode-sized batch).
             int32_t *cnt = (int32_t *)layer->h_items;
+            ek::RowCopy *tab = (ek::RowCopy *)(layer->h_items + 16);
+            int n_tab = 0;
+            static_assert(sizeof(ek::WorkItem) == 16 && sizeof(int32_t) * ek::kNumLists == 16, "whole 16-byte units");
             for (int l = 0; l < ek::kNumLists; ++l) {
                 cnt[l] = (int32_t)items[l].size();
-                if (cnt[l]) {
-                    memcpy(layer->h_items + off[l], items[l].data(), sizeof(ek::WorkItem) * items[l].size());
-                    EK_HIP(hipMemcpyAsync(layer->ws.lists.items[l], layer->h_items + off[l],
-                                          sizeof(ek::WorkItem) * items[l].size(), hipMemcpyHostToDevice, s));
-                }
+                if (!cnt[l]) continue;
+                const size_t bytes = sizeof(ek::WorkItem) * items[l].size();
+                memcpy(layer->h_items + off[l], items[l].data(), bytes);
+                if (layer->d_items)
+                    tab[n_tab++] = ek::RowCopy{layer->d_items + off[l], (uint8_t *)layer->ws.lists.items[l], 0, 0, 1, (int32_t)bytes};
+                else
+                    EK_HIP(hipMemcpyAsync(layer->ws.lists.items[l], layer->h_items + off[l], bytes, hipMemcpyHostToDevice, s));
             }
-            EK_HIP(hipMemcpyAsync(layer->ws.lists.count, cnt, sizeof(int32_t) * ek::kNumLists, hipMemcpyHostToDevice, s));
+            if (layer->d_items) {
+                tab[n_tab++] = ek::RowCopy{layer->d_items, (uint8_t *)layer->ws.lists.count, 0, 0, 1, 16};
+                ek::launch_rows_copy((const ek::RowCopy *)(layer->d_items + 16), n_tab, s);
+                EK_HIP(hipGetLastError());
+            } else {
+                EK_HIP(hipMemcpyAsync(layer->ws.lists.count, cnt, sizeof(int32_t) * ek::kNumLists, hipMemcpyHostToDevice, s));
+            }
             EK_HIP(hipEventRecord(layer->ev_items, s));
             EK_TRY(ensure_io_staging(layer));
             // Many small host requests: their rows are gathered in pinned memory and cross the

@@ -382,6 +382,9 @@ static hipError_t launch_d(const FfnArgs &a, int32_t nseg, hipStream_t s)
 //    1, 43.7 -> 42.0 at 2) and loses from 8 on (136 -> 141 us at 8, 224 -> 241 at 16, behind a sliced
 //    stage 1).
 constexpr int64_t kSliceStage2Below = 8192;   // (item, channel group) pairs, one-byte weights
+// Below this many (item, channel group) pairs the one-wave form leaves most of the chip's memory
+// system idle whatever the rows per item (a lone expert, a tiny layer).
+constexpr int64_t kSplitBelow = 1536;
 
 // few_rows: the launch's items hold about four rows or fewer on average.
 template <typename T, int WM, int NMAT>
@@ -415,9 +418,8 @@ static hipError_t launch_g(const FfnArgs &a, int32_t nseg, bool wide, bool few_r
     if (NT % NG == 0) {
         // prefetch slots of the sliced form: a slice is an eighth of the contraction
         constexpr int DS = W8 ? 2 : D;
-        const bool sliced = !W8 ? true
-                            : NMAT == 2 ? few_rows
-                                        : (int64_t)nseg * (NT / NG) < kSliceStage2Below;
+        const int64_t groups = (int64_t)nseg * (NT / NG);
+        const bool sliced = !W8 ? true : NMAT == 2 ? few_rows || groups < kSplitBelow : groups < kSliceStage2Below;
         if (sliced) {
             hipLaunchKernelGGL((ffn_stream_kernel<T, WM, NMAT, NG, DS, kSlices, 1>), dim3(NT / NG, nseg),
                                dim3(64 * kSlices), 0, s, a);
