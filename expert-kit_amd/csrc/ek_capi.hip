@@ -1218,7 +1218,8 @@ constexpr int64_t kPairDirectPairs = 16;
 bool pair_direct_fits(const ek_layer *L, int64_t T)
 {
     const int64_t P = T * L->cfg.top_k;
-    return P > 0 && P <= kPairDirectPairs && L->cfg.top_k <= ek::kPairDirectMaxK && !shared_cut(L, T).shared;
+    const SharedCut sc = shared_cut(L, T);          // a shared expert of the routed experts' shape is one more wave
+    return P > 0 && P <= kPairDirectPairs && L->cfg.top_k <= ek::kPairDirectMaxK && (!sc.shared || !sc.own);
 }
 
 // want_tables: the caller reads the call's routing tables or packed expert outputs afterwards.
@@ -1243,6 +1244,7 @@ ek_status enqueue_forward(ek_layer *L, const Workspace &W, const void *x, const 
         a1.x = x; a1.x_stride = H; a1.rows = nullptr; a1.slabs = L->d_slabs; a1.out = W.h; a1.out_stride = L->cfg.inter;
         a1.N = (int32_t)L->cfg.inter; a1.Kdim = (int32_t)H; a1.lists = W.lists;
         a1.pair_ids = ids; a1.pair_K = K; a1.pair_P = (int32_t)P; a1.n_experts = E;
+        a1.pair_shared = shared_cut(L, T).shared ? 1 : 0;
         a1.pair_err = W.err; a1.pair_activation = L->d_activation; a1.pair_tile_items_host = L->d_tile_items;
         ek::FfnArgs a2 = a1;
         a2.x = W.h; a2.x_stride = L->cfg.inter; a2.out = nullptr; a2.out_stride = H;

@@ -72,14 +72,17 @@ __device__ __forceinline__ void pair_combine(const FfnArgs &a, const float (*pro
     float acc = 0.f;
     for (int k = 0; k < a.pair_K; ++k)
         if (valid[k]) acc = acc + prod[k][lane];
-    ((T *)a.pair_y)[t * a.N + ch0 + lane] = (T)acc;
+    T o = (T)acc;
+    // the shared expert's row (wave pair_K) joins after the sum's rounding
+    if (a.pair_shared && valid[a.pair_K]) o = (T)((float)o + prod[a.pair_K][lane]);
+    ((T *)a.pair_y)[t * a.N + ch0 + lane] = o;
 }
 
 // PD = 0: items from the work list.  PD = 1: pair-direct stage 1 (blockIdx.y is the pair).  PD = 2:
 // pair-direct stage 2 (blockIdx.y is the token, wave k of the workgroup takes its k-th pair and walks
 // the whole contraction, SK = 1; the weighted sum over k replaces the store of the rows).
 template <typename T, int WM, int NMAT, int NG, int D, int SK, int RS, int PD = 0>
-__global__ __launch_bounds__(PD == 2 ? 64 * kPairDirectMaxK : SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kernel(FfnArgs a)
+__global__ __launch_bounds__(PD == 2 ? 64 * (kPairDirectMaxK + 1) : SK == 1 ? 256 : 64 * kSlices) void ffn_stream_kernel(FfnArgs a)
 {
     static_assert(PD == 0 || RS == 1, "pair-direct items hold one row");
     static_assert(PD != 1 || (NMAT == 2 && SK == kSlices), "pair-direct stage 1 is a sliced launch");
@@ -101,10 +104,12 @@ __global__ __launch_bounds__(PD == 2 ? 64 * kPairDirectMaxK : SK == 1 ? 256 : 64
         e = item.expert; seg0 = item.row0; n = item.nrows;
     } else {
         if (PD == 1 && blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) pair_bookkeeping(a, lane);
-        seg0 = PD == 1 ? (int)blockIdx.y : (int)blockIdx.y * a.pair_K + wave;
+        // items past the pairs (stage 1) and wave pair_K (stage 2) are the tokens' rows of the shared expert
+        const bool shared_row = PD == 1 ? (int)blockIdx.y >= a.pair_P : wave == a.pair_K;
+        seg0 = PD == 1 ? (int)blockIdx.y : shared_row ? a.pair_P + (int)blockIdx.y : (int)blockIdx.y * a.pair_K + wave;
         n = 1;
-        e = a.pair_ids[seg0];
-        live = (uint32_t)e < (uint32_t)a.n_experts;
+        e = shared_row ? a.n_experts : a.pair_ids[seg0];
+        live = shared_row || (uint32_t)e < (uint32_t)a.n_experts;
         if (!live) e = 0;
     }
     const int NT = a.N >> 4;
@@ -112,8 +117,8 @@ __global__ __launch_bounds__(PD == 2 ? 64 * kPairDirectMaxK : SK == 1 ? 256 : 64
     if (nt0 >= NT) return;             // SK = 8, PD = 2: the same for every wave of the workgroup
     const ExpertSlab slab = a.slabs[e];
     const uint8_t *wmat = NMAT == 2 ? slab.upgate : slab.down;
-    [[maybe_unused]] __shared__ float pd_prod[PD == 2 ? kPairDirectMaxK : 1][PD == 2 ? NG * 16 : 1];
-    [[maybe_unused]] __shared__ int32_t pd_valid[PD == 2 ? kPairDirectMaxK : 1];
+    [[maybe_unused]] __shared__ float pd_prod[PD == 2 ? kPairDirectMaxK + 1 : 1][PD == 2 ? NG * 16 : 1];
+    [[maybe_unused]] __shared__ int32_t pd_valid[PD == 2 ? kPairDirectMaxK + 1 : 1];
     if constexpr (PD == 2) {
         live = live && wmat != nullptr;
         if (!live) {
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(PD == 2 ? 64 * kPairDirectMaxK : SK == 1 ? 256 : 64
     // Block scales: the wave's 16 channels lie in one 128-row block, so the scale of a chunk is
     // one number per 128 contraction elements: the wave keeps its rows of the scale matrices in
     // LDS (lane b holds block b) and reads one back per chunk.
-    __shared__ float srow[block_scaled(WM) ? (PD == 2 ? kPairDirectMaxK : SK == 1 ? 4 : kSlices) : 1][block_scaled(WM) ? NW : 1]
+    __shared__ float srow[block_scaled(WM) ? (PD == 2 ? kPairDirectMaxK + 1 : SK == 1 ? 4 : kSlices) : 1][block_scaled(WM) ? NW : 1]
                          [block_scaled(WM) ? kMaxScaleBlocks : 1];
     if constexpr (block_scaled(WM)) {
         const int KB = (a.Kdim + 127) >> 7;
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(PD == 2 ? 64 * kPairDirectMaxK : SK == 1 ? 256 : 64
 #pragma unroll
     for (int rs = 0; rs < RS; ++rs) {
         const int jr = min(rs * 16 + j, n - 1);   // lanes past the segment re-read its last row
-        const int64_t row = PD == 1 ? (int64_t)(seg0 / a.pair_K)
+        const int64_t row = PD == 1 ? (int64_t)(seg0 >= a.pair_P ? seg0 - a.pair_P : seg0 / a.pair_K)
                             : a.rows ? (int64_t)a.rows[seg0 + jr] : (int64_t)(seg0 + jr);
         xp[rs] = (const T *)a.x + row * a.x_stride + g * (KE / 4);
     }
@@ -303,14 +308,19 @@ __global__ __launch_bounds__(PD == 2 ? 64 * kPairDirectMaxK : SK == 1 ? 256 : 64
     if constexpr (PD == 2) {
         // lanes (g, 0) hold the pair's row: its rounded outputs times the gate weight, as the
         // combine kernel forms them, meet in LDS
-        const float wv = a.pair_w_f32 ? ((const float *)a.pair_w)[seg0] : (float)((const T *)a.pair_w)[seg0];
+        const bool shared_row = wave == a.pair_K;
+        const int wi = shared_row ? 0 : seg0;
+        const float wv = a.pair_w_f32 ? ((const float *)a.pair_w)[wi] : (float)((const T *)a.pair_w)[wi];
         if (j == 0) {
 #pragma unroll
             for (int gi = 0; gi < NG; ++gi)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    float pr = wv * (float)(T)tot[0][0][gi][r];
-                    if (!a.pair_w_f32) pr = (float)(T)pr;
+                    float pr = (float)(T)tot[0][0][gi][r];
+                    if (!shared_row) {
+                        pr = wv * pr;
+                        if (!a.pair_w_f32) pr = (float)(T)pr;
+                    }
                     pd_prod[wave][gi * 16 + 4 * g + r] = pr;
                 }
         }
@@ -458,10 +468,12 @@ static hipError_t launch_pairs_w(const FfnArgs &a, int stage, hipStream_t s)
     if (stage == 1) {
         // the sliced form of the ordinary launch, one item per pair
         constexpr int DS = W8 ? 2 : kStage1Depth;
-        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 2, 1, DS, kSlices, 1, 1>), dim3(NT, a.pair_P), dim3(64 * kSlices), 0, s, a);
+        const int T1 = a.pair_P / a.pair_K;
+        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 2, 1, DS, kSlices, 1, 1>), dim3(NT, a.pair_P + (a.pair_shared ? T1 : 0)),
+                           dim3(64 * kSlices), 0, s, a);
         return hipGetLastError();
     }
-    const dim3 block(64 * a.pair_K);
+    const dim3 block(64 * (a.pair_K + (a.pair_shared ? 1 : 0)));
     const int T_ = a.pair_P / a.pair_K;
     constexpr int NG = kStage2Tiles, D = kStage2Depth;
     if (NT % NG == 0 && KT % D == 0)

@@ -164,6 +164,9 @@ struct FfnArgs {
     int32_t pair_K = 0, pair_P = 0, n_experts = 0;
     const void *pair_w = nullptr;        // [pair_P] gate weights (stage 2)
     int32_t pair_w_f32 = 0;              // gate weights are fp32 instead of the activation type
+    int32_t pair_shared = 0;             // 1: every token also runs expert n_experts (the shared expert) as item
+                                         // pair_P + t (x row t, out row pair_P + t); its rounded output is added
+                                         // to the rounded weighted sum, as the combine kernel adds it
     void *pair_y = nullptr;              // [T, N] stage 2: the weighted sum over a token's pairs
     int32_t *pair_err = nullptr;         // stage 1 writes the call's error word (PackArgs::err)
     uint64_t *pair_activation = nullptr; // [n_experts] or nullptr (PackArgs::activation)

@@ -216,8 +216,8 @@ ek_status ek_layer_has_expert(ek_layer *layer, int32_t expert, int32_t *loaded);
  * on a side stream of the library's that it forks from and joins to `stream`):
  * it may be captured into the caller's HIP graph, whose grids depend on T only.
  * A call of at most 16 pairs (one or two tokens at top-8) that asks for no
- * routing tables (route == NULL), on a layer with top-k <= 8 and no shared
- * expert, is two kernel launches: no pack and no combine kernel (same results,
+ * routing tables (route == NULL), on a layer with top-k <= 8 (a shared expert
+ * of the routed experts' width included), is two kernel launches: no pack and no combine kernel (same results,
  * same errors, same activation counts). */
 ek_status ek_layer_forward(ek_layer *layer, const void *x, const int32_t *ids, const void *w,
                            int32_t w_dtype, int64_t T, void *y, const ek_route_out *route,

@@ -203,3 +203,45 @@ def test_chain_of_few_pairs(ek, cuda, T):
     chain.close()
     for layer in layers:
         layer.close()
+
+
+@pytest.mark.parametrize("kind", ["w16", "i8", "fp8", "int8"])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,K", [(1, 8), (2, 8), (2, 3), (5, 1)])
+def test_pair_direct_with_a_shared_expert(ek, oracle, cuda, kind, dt, T, K):
+    """A shared expert of the routed experts' shape (deepseek_v3/model.py:57-61,152) is one more wave
+    of stage 2's workgroups: its rounded output joins the rounded weighted sum, as in the call through
+    pack and combine, whose bits the call must give; held to the oracle by test_gpu_shared.py's bound."""
+    from test_gpu_parity import TOL, ulp_of
+    H, I, E = 384 if kind == "w16" else 512, 192 if kind == "w16" else 384, 12
+    layer, (wu, wg, wd) = build(ek, oracle, kind, dt, H, I, E, K)
+    # the shared expert: the weights of slot 3 (build's fourth distinct expert)
+    if kind in KINDS:
+        shared_w = make_block_expert(ek, H, I, 13, kind)
+    else:
+        shared_w = wl.make_expert(wl.Workload("t", H, I, E, K, 8, dt, w8=kind == "i8"), 13, std=0.05)
+    g = torch.Generator().manual_seed(7 * T + K)
+    x = torch.randn(T, H, generator=g).to(dt)
+    ids = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32).reshape(T, K)
+    gw = torch.rand(T, K, generator=g) + 0.1
+    gw = (gw / gw.sum(-1, keepdim=True)).to(dt)
+    y_plain = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda))
+    layer.set_shared_expert(shared_w)
+    for w in (gw, gw.float()):
+        y = layer.forward(x.to(cuda), ids.to(cuda), w.to(cuda))
+        y_t, _ = layer.forward(x.to(cuda), ids.to(cuda), w.to(cuda), return_route=True)
+        assert same_bits(y, y_t), "pair-direct call differs from the call through pack and combine"
+        assert same_bits(layer.forward(x, ids, w), y)
+        assert same_bits(layer.forward_static(x.to(cuda), ids.to(cuda), w.to(cuda)), y)
+    assert not same_bits(y, y_plain)
+    y = layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda))
+    y_r = oracle.layer_forward(x, ids, gw, wu, wg, wd, mode=0)[0]
+    ref32 = oracle.add_shared(y_r, x, wu[3], wg[3], wd[3], rounded=False)
+    y_s = ref32 - y_r.float()
+    rms = float(ref32.pow(2).mean().sqrt())
+    err = (y.float().cpu() - ref32).abs()
+    quanta = 0.5 * ulp_of(ref32, dt) * 1.0001 + ulp_of(y_r.float(), dt) + ulp_of(y_s, dt)
+    assert bool((err <= TOL * rms + quanta).all()), float(err.max()) / rms
+    layer.remove_expert(C.EK_SHARED_EXPERT)
+    assert same_bits(layer.forward(x.to(cuda), ids.to(cuda), gw.to(cuda)), y_plain)
+    layer.close()
