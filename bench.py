@@ -336,10 +336,11 @@ def time_layer(layer, w, args, dev, stream, graph=False):
             "graph_s": graph_s}
 
 
-def decode_sweep(layer, base, dev, stream, token_counts, calls=30):
+def decode_sweep(layer, base, dev, stream, token_counts):
     """The decode layer at other batch sizes (uniform routing, as the configuration's): enqueue-only
-    calls on `stream`, the whole call's algorithmic bytes against the HBM peak.  The routing tables of each
-    size are checked against a stable sort first; the timed calls must reproduce that call's output."""
+    calls on `stream` (200 of them up to 8 tokens, 50 up to 64, 30 beyond: ~15-50 ms of device time per
+    size), the whole call's algorithmic bytes against the HBM peak.  The routing tables of each size are
+    checked against a stable sort first; the timed calls must reproduce that call's output."""
     import torch
     from dataclasses import replace
     from ek_hip import workloads as wl
@@ -352,6 +353,7 @@ def decode_sweep(layer, base, dev, stream, token_counts, calls=30):
         y0, rt = layer.forward(xd, idd, gwd, return_route=True)
         assert torch.equal(rt.perm.cpu(), torch.argsort(ids.reshape(-1).long(), stable=True).to(torch.int32)), T
         y = torch.empty_like(xd)
+        calls = 200 if T <= 8 else 50 if T <= 64 else 30
         for _ in range(5):
             layer.forward(xd, idd, gwd, stream=stream, out=y)
         stream.synchronize()
@@ -364,7 +366,7 @@ def decode_sweep(layer, base, dev, stream, token_counts, calls=30):
         stream.synchronize()
         step_s = max(time.perf_counter() - t0, e0.elapsed_time(e1) * 1e-3) / calls
         assert torch.equal(y.view(torch.int16), y0.view(torch.int16)), T
-        rows.append({"tokens": T, "ms_per_step": step_s * 1e3, "pairs_per_s": w.pairs / step_s,
+        rows.append({"tokens": T, "calls": calls, "ms_per_step": step_s * 1e3, "pairs_per_s": w.pairs / step_s,
                      "active_experts": int((counts > 0).sum()),
                      "hbm_frac": wl.algorithmic_bytes(w, counts) / step_s / HBM_PEAK})
     return rows
@@ -553,7 +555,7 @@ def main():
     if m["parity"] is not None:
         out["parity"] = m["parity"]
     if everything and args.sweep:
-        out["decode_sweep"] = {"what": f"{w.name}'s layer at other batch sizes, {30} enqueue-only calls each, whole call against "
+        out["decode_sweep"] = {"what": f"{w.name}'s layer at other batch sizes, 30 to 200 enqueue-only calls each, whole call against "
                                        "8 TB/s; outputs equal the routing-checked call's bit for bit",
                                "rows": decode_sweep(layer, w, dev, stream, (1, 2, 4, 8, 16, 32, 64, 256, 512))}
     torch.set_num_threads(cpu_cores())
