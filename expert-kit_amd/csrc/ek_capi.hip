@@ -1759,8 +1759,8 @@ ek_status ek_layer_experts_forward(ek_layer *layer, int32_t n_calls, const int32
             } else {
                 EK_HIP(hipEventSynchronize(layer->ev_items));
             }
-            // One copy kernel reads the lists and their lengths where they lie in pinned memory (up to five
-            // asynchronous copies took the stream ~45 us before the first FFN kernel of a decode-sized batch).
+            // One copy kernel reads the lists and their lengths where they lie in pinned memory, instead of up to
+            // five asynchronous copies (8 DeepSeek-V3 int8 requests of one row: 84.5 -> 83.4 us per call).
             int32_t *cnt = (int32_t *)layer->h_items;
             ek::RowCopy *tab = (ek::RowCopy *)(layer->h_items + 16);
             int n_tab = 0;

@@ -478,9 +478,7 @@ static hipError_t launch_pairs_w(const FfnArgs &a, int stage, hipStream_t s)
     constexpr int NG = kStage2Tiles, D = kStage2Depth;
     if (NT % NG == 0 && KT % D == 0)
         hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 1, NG, D, 1, 1, 2>), dim3(NT / NG, T_), block, 0, s, a);
-    else if (NT % NG == 0 && KT % (D / 2) == 0)
-        hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 1, NG, D / 2, 1, 1, 2>), dim3(NT / NG, T_), block, 0, s, a);
-    else if (NT % NG == 0 && KT % 2 == 0)
+    else if (NT % NG == 0 && KT % 2 == 0)      // (the one-wave loop takes contractions of whole prefetch rounds)
         hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 1, NG, 2, 1, 1, 2>), dim3(NT / NG, T_), block, 0, s, a);
     else
         hipLaunchKernelGGL((ffn_stream_kernel<T, WM, 1, 1, 1, 1, 1, 2>), dim3(NT, T_), block, 0, s, a);
